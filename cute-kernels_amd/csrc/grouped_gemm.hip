@@ -1,0 +1,512 @@
+// Scattered grouped GEMMs over tile-aligned expert segments, bf16 / f16 inputs, fp32 accumulation on MFMA.
+//
+// Every expert's rows start at a multiple of the tile height in the padded grouped layout, so a workgroup's M-tile
+// belongs to exactly one expert: no tile straddles two experts and no K loop is repeated per expert. All GEMMs are
+// "NT": both operands are contraction-contiguous (the backward passes get that from transposed copies written by the
+// producing epilogues), so global loads are 128-bit along K and LDS fragments feed v_mfma_f32_32x32x16 directly.
+//
+// Workgroup = 256 threads = 4 waves in a 2x2 grid; wave tile (BM/2)x(BN/2) built from 32x32 MFMA blocks; K step 64
+// staged through double-buffered LDS (rows padded to 72 elements so 16 lanes x 16 bytes cover all banks); the global
+// loads of step k+1 are in flight while step k is multiplied.
+#include <type_traits>
+
+#include "ck_common.h"
+
+namespace ck {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int BK = 64;            // K elements per stage
+constexpr int kLdsStride = 72;    // elements per LDS row (64 + 8 pad)
+constexpr int kChunksPerRow = 8;  // 16-byte chunks per 64-element row
+constexpr int kXcds = 8;
+
+enum Mode { kGrouped = CK_EPI_GROUPED, kScatter = CK_EPI_SCATTER, kSwiglu = CK_EPI_SWIGLU, kSwigluBwd = CK_EPI_SWIGLU_BWD, kDw = 4 };
+
+template <typename T>
+struct Mfma;
+template <>
+struct Mfma<bf16_t> {
+  typedef bf16x8 frag;
+  __device__ static inline f32x16 run(const frag& a, const frag& b, const f32x16& c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct Mfma<f16_t> {
+  typedef f16x8 frag;
+  __device__ static inline f32x16 run(const frag& a, const frag& b, const f32x16& c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
+};
+
+struct GemmParams {
+  const void* a;      // forward modes: [*, K]; dW: a_t [M, ld_t]
+  const void* w;      // forward modes: [E, N, K]; dW: b_t [N, ld_t]
+  int64_t lda;        // row stride of a (elements)
+  int64_t ldw;        // row stride of w (elements)
+  int64_t w_expert_stride;
+  int a_gather_div;   // > 0: A row p comes from a[row_slot[p] / div]
+  int M;              // dW only: rows of a_t
+  int N;              // output columns of the GEMM (2I for kSwiglu)
+  int K;              // contraction length (forward modes)
+  int I;              // kSwiglu / kSwigluBwd: intermediate size
+  int n_tiles;        // tiles along N
+  int m_tiles;        // dW only: tiles along M
+  int align;          // rows per M tile (== BM) in the padded layout
+  int num_experts;
+  const int32_t* seg_starts;
+  const uint32_t* counts;
+  const int32_t* tile_expert;
+  const int32_t* row_slot;
+  void* y;
+  void* y_t;
+  int64_t ld_t;
+  void* aux;
+  const void* aux_in;
+};
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant expression
+template <int N, typename F>
+__device__ inline void static_for(F&& f) {
+  if constexpr (N > 0) {
+    static_for<N - 1>(f);
+    f(std::integral_constant<int, N - 1>{});
+  }
+}
+
+template <typename T>
+__device__ inline uint16_t bits16(T v) {
+  union {
+    T t;
+    uint16_t u;
+  } c;
+  c.t = v;
+  return c.u;
+}
+
+// 4 consecutive 16-bit values as one 8-byte store
+template <typename T>
+__device__ inline void store4(T* p, T v0, T v1, T v2, T v3) {
+  uint2 u;
+  u.x = (uint32_t)bits16(v0) | ((uint32_t)bits16(v1) << 16);
+  u.y = (uint32_t)bits16(v2) | ((uint32_t)bits16(v3) << 16);
+  *reinterpret_cast<uint2*>(p) = u;
+}
+
+template <typename T, int BM, int BN, int MODE>
+__global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams prm) {
+  constexpr int WM = BM / 2, WN = BN / 2;    // wave tile
+  constexpr int MI = WM / 32, NI = WN / 32;  // 32x32 blocks per wave tile
+  constexpr int A_CH = BM / 32, B_CH = BN / 32;  // 16-byte chunks per thread per stage
+  constexpr int kStageElems = (BM + BN) * kLdsStride;
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  T* lds = reinterpret_cast<T*>(lds_raw);
+
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // ---- which tile: blocks are dealt round-robin to the 8 XCDs, so give each XCD a contiguous run of tiles
+  int mt, nt, expert;
+  int64_t k_begin = 0;
+  int k_len;
+  if constexpr (MODE == kDw) {
+    const int per_expert = prm.m_tiles * prm.n_tiles;
+    const int total = per_expert * prm.num_experts;
+    int pid = blockIdx.x;
+    if (total % kXcds == 0) pid = (pid % kXcds) * (total / kXcds) + pid / kXcds;
+    expert = pid / per_expert;
+    const int r = pid - expert * per_expert;
+    // N-tile fastest: consecutive blocks share the a_t panel
+    mt = r / prm.n_tiles;
+    nt = r - mt * prm.n_tiles;
+    k_begin = prm.seg_starts[expert];
+    k_len = (int)((prm.counts[expert] + BK - 1) / BK * BK);
+  } else {
+    const int live_m = prm.seg_starts[prm.num_experts] / prm.align;
+    const int total = live_m * prm.n_tiles;
+    int pid = blockIdx.x;
+    if (pid >= total) return;
+    const int per_xcd = total / kXcds;
+    if (pid < per_xcd * kXcds) pid = (pid % kXcds) * per_xcd + pid / kXcds;  // the ragged end keeps its order
+    // groups of 8 M-tiles, N-tile next, M-tile within the group fastest: a group reuses one W panel 8 times
+    constexpr int GROUP = 8;
+    const int group_sz = GROUP * prm.n_tiles;
+    const int g = pid / group_sz;
+    const int first_m = g * GROUP;
+    const int rows_in_group = min(GROUP, live_m - first_m);
+    const int r = pid - g * group_sz;
+    nt = r / rows_in_group;
+    mt = first_m + (r - nt * rows_in_group);
+    expert = prm.tile_expert[mt];
+    k_len = prm.K;
+  }
+  const int64_t m0 = (int64_t)mt * BM;
+
+  // ---- per-thread global chunk addresses, as 32-bit offsets in 16-byte chunks from the operand base
+  const int cc = tid & (kChunksPerRow - 1);  // chunk within the 64-element K slab
+  const int lr = tid >> 3;                   // row within a group of 32
+  const vec16* a_base = static_cast<const vec16*>(prm.a);
+  const vec16* b_base = static_cast<const vec16*>(prm.w);
+  uint32_t a_chunk[A_CH], b_chunk[B_CH];
+  int64_t valid_end = 0;  // forward modes: first pad row of this expert's segment
+  if constexpr (MODE == kDw) {
+#pragma unroll
+    for (int i = 0; i < A_CH; ++i) {
+      const int64_t row = min(m0 + lr + 32 * i, (int64_t)prm.M - 1);
+      a_chunk[i] = (uint32_t)((row * prm.lda + k_begin) / 8 + cc);
+    }
+#pragma unroll
+    for (int i = 0; i < B_CH; ++i) {
+      const int64_t row = min((int64_t)nt * BN + lr + 32 * i, (int64_t)prm.N - 1);
+      b_chunk[i] = (uint32_t)((row * prm.ldw + k_begin) / 8 + cc);
+    }
+  } else {
+    valid_end = (int64_t)prm.seg_starts[expert] + prm.counts[expert];
+#pragma unroll
+    for (int i = 0; i < A_CH; ++i) {
+      int64_t p = m0 + lr + 32 * i;
+      if (p >= valid_end) p = valid_end - 1;  // pad rows re-read a valid row; their results are never stored
+      const int64_t row = prm.a_gather_div > 0 ? (int64_t)(prm.row_slot[p] / prm.a_gather_div) : p;
+      a_chunk[i] = (uint32_t)(row * prm.lda / 8 + cc);
+    }
+    const int64_t w_off = (int64_t)expert * prm.w_expert_stride;
+#pragma unroll
+    for (int i = 0; i < B_CH; ++i) {
+      const int j = lr + 32 * i;  // row of the LDS B tile
+      int64_t n;
+      if constexpr (MODE == kSwiglu) {
+        // LDS rows [wave column][up half | gate half]: the same lane ends up holding up and gate of one column
+        const int half = (j % WN) / (WN / 2);
+        const int within = (j / WN) * (WN / 2) + (j % (WN / 2));
+        const int64_t col = min((int64_t)nt * (BN / 2) + within, (int64_t)prm.I - 1);
+        n = (int64_t)half * prm.I + col;
+      } else {
+        n = min((int64_t)nt * BN + j, (int64_t)prm.N - 1);
+      }
+      b_chunk[i] = (uint32_t)((w_off + n * prm.ldw) / 8 + cc);
+    }
+  }
+
+  f32x16 acc[MI][NI];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NI; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // ---- main loop
+  vec16 ra[A_CH], rb[B_CH];
+  auto load_global = [&](int kt) {
+    const int k = kt * BK + cc * 8;
+    const bool ok = k < k_len;  // K % 8 == 0, so a chunk is entirely inside or outside
+#pragma unroll
+    for (int i = 0; i < A_CH; ++i) ra[i] = ok ? a_base[a_chunk[i] + (uint32_t)kt * (BK / 8)] : zero16();
+#pragma unroll
+    for (int i = 0; i < B_CH; ++i) rb[i] = ok ? b_base[b_chunk[i] + (uint32_t)kt * (BK / 8)] : zero16();
+  };
+  auto store_lds = [&](int stage) {
+    T* sa = lds + stage * kStageElems;
+    T* sb = sa + BM * kLdsStride;
+#pragma unroll
+    for (int i = 0; i < A_CH; ++i) store16(sa + (lr + 32 * i) * kLdsStride + cc * 8, ra[i]);
+#pragma unroll
+    for (int i = 0; i < B_CH; ++i) store16(sb + (lr + 32 * i) * kLdsStride + cc * 8, rb[i]);
+  };
+  typedef typename Mfma<T>::frag frag_t;
+  auto compute = [&](int stage) {
+    const T* sa = lds + stage * kStageElems + (wm * WM + (lane & 31)) * kLdsStride + (lane >> 5) * 8;
+    const T* sb = lds + stage * kStageElems + BM * kLdsStride + (wn * WN + (lane & 31)) * kLdsStride + (lane >> 5) * 8;
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) {
+      frag_t fa[MI], fb[NI];
+#pragma unroll
+      for (int i = 0; i < MI; ++i) fa[i] = *reinterpret_cast<const frag_t*>(sa + i * 32 * kLdsStride + kk * 16);
+#pragma unroll
+      for (int j = 0; j < NI; ++j) fb[j] = *reinterpret_cast<const frag_t*>(sb + j * 32 * kLdsStride + kk * 16);
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) acc[i][j] = Mfma<T>::run(fa[i], fb[j], acc[i][j]);
+    }
+  };
+
+  const int nk = (k_len + BK - 1) / BK;
+  if (nk > 0) {
+    load_global(0);
+    store_lds(0);
+    __syncthreads();
+    for (int kt = 0; kt < nk; ++kt) {
+      const bool more = kt + 1 < nk;
+      if (more) load_global(kt + 1);
+      compute(kt & 1);
+      if (more) store_lds((kt + 1) & 1);
+      __syncthreads();
+    }
+  }
+
+  // ---- epilogue. Lane holds, per 32x32 block and q in 0..3, rows 8q + 4*(lane/32) + 0..3 of column lane%32.
+  // static_for keeps every accumulator index a compile-time constant (the accumulators live in AGPRs).
+  const int col_in_block = lane & 31;
+  const int row_quad = (lane >> 5) * 4;
+  if constexpr (MODE == kDw) {
+    T* dw = static_cast<T*>(prm.y) + (int64_t)expert * prm.M * prm.N;
+    static_for<MI>([&](auto i) {
+      static_for<NI>([&](auto j) {
+        const int64_t n = (int64_t)nt * BN + wn * WN + j * 32 + col_in_block;
+        static_for<16>([&](auto r) {
+          const int64_t m = m0 + wm * WM + i * 32 + 8 * (r / 4) + row_quad + (r % 4);
+          if (m < prm.M && n < prm.N) dw[m * prm.N + n] = Elem<T>::down(acc[i][j][(int)r]);
+        });
+      });
+    });
+  } else if constexpr (MODE == kGrouped || MODE == kScatter) {
+    T* y = static_cast<T*>(prm.y);
+    T* y_t = static_cast<T*>(prm.y_t);
+    static_for<MI>([&](auto i) {
+      static_for<4>([&](auto q) {
+        const int64_t p_base = m0 + wm * WM + i * 32 + 8 * q + row_quad;
+        int64_t out_row[4];
+        static_for<4>([&](auto s) {
+          const int64_t p = p_base + s;
+          out_row[s] = -1;
+          if (p < valid_end) out_row[s] = (MODE == kScatter) ? (int64_t)prm.row_slot[p] : p;
+        });
+        static_for<NI>([&](auto j) {
+          const int64_t n = (int64_t)nt * BN + wn * WN + j * 32 + col_in_block;
+          if (n < prm.N) {
+            T v[4];
+            static_for<4>([&](auto s) {
+              v[s] = Elem<T>::down(acc[i][j][4 * q + s]);
+              if (out_row[s] >= 0) y[out_row[s] * prm.N + n] = v[s];
+              else v[s] = Elem<T>::down(0.f);
+            });
+            if (MODE == kGrouped && y_t != nullptr) store4(y_t + n * prm.ld_t + p_base, v[0], v[1], v[2], v[3]);
+          }
+        });
+      });
+    });
+  } else if constexpr (MODE == kSwiglu) {
+    // acc[i][j] (j < NI/2) = up, acc[i][j + NI/2] = gate of the same column
+    T* pre = static_cast<T*>(prm.y);
+    T* act = static_cast<T*>(prm.aux);
+    T* act_t = static_cast<T*>(prm.y_t);
+    const int64_t two_i = 2 * (int64_t)prm.I;
+    static_for<MI>([&](auto i) {
+      static_for<4>([&](auto q) {
+        const int64_t p_base = m0 + wm * WM + i * 32 + 8 * q + row_quad;
+        static_for<NI / 2>([&](auto j) {
+          const int64_t col = (int64_t)nt * (BN / 2) + wn * (WN / 2) + j * 32 + col_in_block;
+          if (col < prm.I) {
+            T v[4];
+            static_for<4>([&](auto s) {
+              const int64_t p = p_base + s;
+              const T up = Elem<T>::down(acc[i][j][4 * q + s]);
+              const T gate = Elem<T>::down(acc[i][j + NI / 2][4 * q + s]);
+              const float gf = Elem<T>::up(gate);
+              v[s] = Elem<T>::down(Elem<T>::up(up) * gf * sigmoid_fast(gf));
+              if (p < valid_end) {
+                pre[p * two_i + col] = up;
+                pre[p * two_i + prm.I + col] = gate;
+                act[p * prm.I + col] = v[s];
+              } else {
+                v[s] = Elem<T>::down(0.f);
+              }
+            });
+            if (act_t != nullptr) store4(act_t + col * prm.ld_t + p_base, v[0], v[1], v[2], v[3]);
+          }
+        });
+      });
+    });
+  } else {  // kSwigluBwd: the GEMM result is d_act
+    const T* pre = static_cast<const T*>(prm.aux_in);
+    T* d_pre = static_cast<T*>(prm.y);
+    T* d_pre_t = static_cast<T*>(prm.y_t);
+    const int64_t two_i = 2 * (int64_t)prm.I;
+    static_for<MI>([&](auto i) {
+      static_for<4>([&](auto q) {
+        const int64_t p_base = m0 + wm * WM + i * 32 + 8 * q + row_quad;
+        static_for<NI>([&](auto j) {
+          const int64_t col = (int64_t)nt * BN + wn * WN + j * 32 + col_in_block;
+          if (col < prm.I) {
+            T du[4], dg[4];
+            static_for<4>([&](auto s) {
+              const int64_t p = p_base + s;
+              du[s] = Elem<T>::down(0.f);
+              dg[s] = Elem<T>::down(0.f);
+              if (p < valid_end) {
+                const float dy = Elem<T>::up(Elem<T>::down(acc[i][j][4 * q + s]));  // d_act as the unfused path rounds it
+                const float uf = Elem<T>::up(pre[p * two_i + col]);
+                const float gf = Elem<T>::up(pre[p * two_i + prm.I + col]);
+                const float sg = sigmoid_fast(gf);
+                const float gsg = gf * sg;
+                du[s] = Elem<T>::down(dy * gsg);
+                dg[s] = Elem<T>::down(dy * uf * (sg + gsg * (1.0f - sg)));
+                d_pre[p * two_i + col] = du[s];
+                d_pre[p * two_i + prm.I + col] = dg[s];
+              }
+            });
+            if (d_pre_t != nullptr) {
+              store4(d_pre_t + col * prm.ld_t + p_base, du[0], du[1], du[2], du[3]);
+              store4(d_pre_t + (prm.I + col) * prm.ld_t + p_base, dg[0], dg[1], dg[2], dg[3]);
+            }
+          }
+        });
+      });
+    });
+  }
+}
+
+template <int BM, int BN>
+constexpr size_t lds_bytes() {
+  return (size_t)2 * (BM + BN) * kLdsStride * 2;
+}
+
+template <typename T, int BM, int BN, int MODE>
+int launch(const GemmParams& prm, unsigned blocks, hipStream_t s, const char* name) {
+  auto kernel = grouped_gemm_kernel<T, BM, BN, MODE>;
+  static bool attr_set = false;  // per instantiation; the attribute is idempotent, a race only repeats the call
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)lds_bytes<BM, BN>());
+    if (e != hipSuccess) {
+      set_error("%s: cannot reserve %zu bytes of LDS: %s", name, lds_bytes<BM, BN>(), hipGetErrorString(e));
+      return CK_ERR_LAUNCH;
+    }
+    attr_set = true;
+  }
+  constexpr size_t kLds = lds_bytes<BM, BN>();
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kThreads), kLds, s, prm);
+  CK_CHECK_LAUNCH(name);
+  return CK_OK;
+}
+
+template <typename T, int MODE>
+int launch_by_tile(const GemmParams& prm, int align, unsigned blocks_256, unsigned blocks_128, hipStream_t s,
+                   const char* name) {
+  if (align == 256) return launch<T, 256, 256, MODE>(prm, blocks_256, s, name);
+  return launch<T, 128, 128, MODE>(prm, blocks_128, s, name);
+}
+
+int check_segments(const ck_segments* seg, const char* name) {
+  CK_REQUIRE(seg != nullptr, "%s: seg is NULL", name);
+  CK_REQUIRE(seg->seg_starts && seg->counts && seg->tile_expert && seg->row_slot, "%s: NULL table in seg", name);
+  CK_REQUIRE(seg->align == 128 || seg->align == 256, "%s: align=%d must be 128 or 256", name, seg->align);
+  CK_REQUIRE(seg->num_experts >= 1, "%s: num_experts=%d", name, seg->num_experts);
+  CK_REQUIRE(seg->max_rows >= 0 && seg->max_rows % seg->align == 0, "%s: max_rows=%lld is not a multiple of align", name,
+             (long long)seg->max_rows);
+  return CK_OK;
+}
+
+}  // namespace
+}  // namespace ck
+
+using namespace ck;
+
+extern "C" int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* w, int32_t N, int32_t K,
+                               const ck_segments* seg, int32_t epilogue, void* y, void* y_t, int64_t ld_t, void* aux,
+                               const void* aux_in, int32_t dtype, void* stream) {
+  const char* name = "ck_grouped_gemm";
+  if (int rc = check_segments(seg, name)) return rc;
+  CK_REQUIRE(N >= 8 && K >= 8 && N % 8 == 0 && K % 8 == 0, "%s: N=%d and K=%d must be positive multiples of 8", name, N, K);
+  CK_REQUIRE(a_gather_div >= 0, "%s: a_gather_div=%d is negative", name, a_gather_div);
+  CK_REQUIRE(epilogue >= CK_EPI_GROUPED && epilogue <= CK_EPI_SWIGLU_BWD, "%s: unknown epilogue %d", name, epilogue);
+  if (seg->max_rows == 0) return CK_OK;
+  CK_REQUIRE(a && w && y, "%s: a, w and y are required", name);
+  CK_REQUIRE(aligned16(a) && aligned16(w), "%s: a and w must be 16-byte aligned", name);
+  CK_REQUIRE(y_t == nullptr || (ld_t >= seg->max_rows && ld_t % 8 == 0 && (reinterpret_cast<uintptr_t>(y_t) & 7) == 0),
+             "%s: y_t needs ld_t >= max_rows, ld_t %% 8 == 0 and 8-byte alignment", name);
+  CK_REQUIRE(epilogue != CK_EPI_SCATTER || y_t == nullptr, "%s: the scatter epilogue has no transposed output", name);
+
+  // operands are addressed with 32-bit offsets in 16-byte chunks
+  CK_REQUIRE((int64_t)seg->num_experts * N * K / 8 < (int64_t)0xffffffff, "%s: w is too large", name);
+  GemmParams prm = {};
+  prm.a = a;
+  prm.w = w;
+  prm.lda = K;
+  prm.ldw = K;
+  prm.w_expert_stride = (int64_t)N * K;
+  prm.a_gather_div = a_gather_div;
+  prm.N = N;
+  prm.K = K;
+  prm.align = seg->align;
+  prm.num_experts = seg->num_experts;
+  prm.seg_starts = seg->seg_starts;
+  prm.counts = seg->counts;
+  prm.tile_expert = seg->tile_expert;
+  prm.row_slot = seg->row_slot;
+  prm.y = y;
+  prm.y_t = y_t;
+  prm.ld_t = ld_t;
+  prm.aux = aux;
+  prm.aux_in = aux_in;
+  int out_cols = N;  // columns that tile along the grid
+  if (epilogue == CK_EPI_SWIGLU) {
+    CK_REQUIRE(N % 16 == 0 && aux != nullptr, "%s: the SwiGLU epilogue needs N = 2*I with I %% 8 == 0 and aux", name);
+    prm.I = N / 2;
+    out_cols = N / 2;
+  } else if (epilogue == CK_EPI_SWIGLU_BWD) {
+    CK_REQUIRE(aux_in != nullptr, "%s: the SwiGLU-backward epilogue needs aux_in", name);
+    prm.I = N;
+  }
+  const int64_t m_tiles = seg->max_rows / seg->align;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // kSwiglu tiles cover BN/2 activation columns each
+  auto n_tiles_for = [&](int bn) { return (int)ceil_div(out_cols, epilogue == CK_EPI_SWIGLU ? bn / 2 : bn); };
+  const int bn = seg->align;  // square tiles
+  prm.n_tiles = n_tiles_for(bn);
+  const int64_t blocks = m_tiles * prm.n_tiles;
+  CK_REQUIRE(blocks < (int64_t)0x7fffffff, "%s: grid too large", name);
+#define CK_GEMM_MODE(MODE) \
+  launch_by_tile<scalar_t, MODE>(prm, seg->align, (unsigned)blocks, (unsigned)blocks, s, name)
+  CK_DISPATCH_HALF(dtype, name, {
+    switch (epilogue) {
+      case CK_EPI_GROUPED: return CK_GEMM_MODE(kGrouped);
+      case CK_EPI_SCATTER: return CK_GEMM_MODE(kScatter);
+      case CK_EPI_SWIGLU: return CK_GEMM_MODE(kSwiglu);
+      default: return CK_GEMM_MODE(kSwigluBwd);
+    }
+  });
+#undef CK_GEMM_MODE
+  return CK_OK;
+}
+
+extern "C" int ck_grouped_gemm_dw(const void* a_t, const void* b_t, int64_t ld_t, int32_t M, int32_t N,
+                                  const ck_segments* seg, void* dw, int32_t dtype, void* stream) {
+  const char* name = "ck_grouped_gemm_dw";
+  if (int rc = check_segments(seg, name)) return rc;
+  CK_REQUIRE(M >= 1 && N >= 1, "%s: M=%d N=%d must be positive", name, M, N);
+  CK_REQUIRE(a_t && b_t && dw, "%s: NULL argument", name);
+  CK_REQUIRE(ld_t >= seg->max_rows && ld_t % 8 == 0 && aligned16(a_t) && aligned16(b_t),
+             "%s: operands need ld_t >= max_rows, ld_t %% 8 == 0 and 16-byte alignment", name);
+  CK_REQUIRE((int64_t)M * ld_t / 8 < (int64_t)0xffffffff && (int64_t)N * ld_t / 8 < (int64_t)0xffffffff,
+             "%s: operands are too large", name);
+  GemmParams prm = {};
+  prm.a = a_t;
+  prm.w = b_t;
+  prm.lda = ld_t;
+  prm.ldw = ld_t;
+  prm.M = M;
+  prm.N = N;
+  prm.align = seg->align;
+  prm.num_experts = seg->num_experts;
+  prm.seg_starts = seg->seg_starts;
+  prm.counts = seg->counts;
+  prm.tile_expert = seg->tile_expert;
+  prm.row_slot = seg->row_slot;
+  prm.y = dw;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // tile size follows the problem, not the segment alignment: small weight matrices get 128x128 tiles
+  const bool big = (M >= 1024 && N >= 1024);
+  const int bt = big ? 256 : 128;
+  prm.m_tiles = (int)ceil_div(M, bt);
+  prm.n_tiles = (int)ceil_div(N, bt);
+  const int64_t blocks = (int64_t)prm.m_tiles * prm.n_tiles * seg->num_experts;
+  CK_REQUIRE(blocks < (int64_t)0x7fffffff, "%s: grid too large", name);
+  CK_DISPATCH_HALF(dtype, name, {
+    if (big) return launch<scalar_t, 256, 256, kDw>(prm, (unsigned)blocks, s, name);
+    return launch<scalar_t, 128, 128, kDw>(prm, (unsigned)blocks, s, name);
+  });
+  return CK_OK;
+}

@@ -1,0 +1,169 @@
+// Stand-alone SwiGLU forward / backward: out = up * gate * sigmoid(gate), fp32 math, one rounding on the way out.
+// Row-strided operands so that the [up | gate] halves of a packed tensor are consumed in place.
+#include "ck_common.h"
+
+namespace ck {
+namespace {
+
+constexpr int kBlock = 256;
+
+// N elements moved as one access: N = Elem<T>::per16 (128-bit) on the aligned fast path, N = 1 otherwise.
+template <typename T, int N>
+struct Chunk {
+  T e[N];
+  __device__ static inline Chunk load(const T* p) {
+    Chunk c;
+    if constexpr (N == 1) {
+      c.e[0] = *p;
+    } else {
+      Pack16<T> k;
+      k.v = load16(p);
+#pragma unroll
+      for (int i = 0; i < N; ++i) c.e[i] = k.e[i];
+    }
+    return c;
+  }
+  __device__ inline void store(T* p) const {
+    if constexpr (N == 1) {
+      *p = e[0];
+    } else {
+      Pack16<T> k;
+#pragma unroll
+      for (int i = 0; i < N; ++i) k.e[i] = e[i];
+      store16(p, k.v);
+    }
+  }
+};
+
+template <typename T, int P>
+__global__ __launch_bounds__(kBlock) void swiglu_fwd_kernel(const T* __restrict__ gate, int64_t gate_stride,
+                                                             const T* __restrict__ up, int64_t up_stride,
+                                                             T* __restrict__ out, int64_t out_stride, int64_t rows,
+                                                             int chunks_per_row) {
+  const int64_t total = rows * chunks_per_row;
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  for (int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x; c < total; c += stride) {
+    const int64_t r = c / chunks_per_row;
+    const int64_t col = (c - r * chunks_per_row) * P;
+    const Chunk<T, P> g = Chunk<T, P>::load(gate + r * gate_stride + col);
+    const Chunk<T, P> u = Chunk<T, P>::load(up + r * up_stride + col);
+    Chunk<T, P> o;
+#pragma unroll
+    for (int i = 0; i < P; ++i) {
+      const float gf = Elem<T>::up(g.e[i]);
+      o.e[i] = Elem<T>::down(Elem<T>::up(u.e[i]) * gf * sigmoid_f32(gf));
+    }
+    o.store(out + r * out_stride + col);
+  }
+}
+
+template <typename T, int P>
+__global__ __launch_bounds__(kBlock) void swiglu_bwd_kernel(const T* __restrict__ gate, int64_t gate_stride,
+                                                             const T* __restrict__ up, int64_t up_stride,
+                                                             const T* __restrict__ d_out, int64_t d_out_stride,
+                                                             T* __restrict__ d_gate, int64_t d_gate_stride,
+                                                             T* __restrict__ d_up, int64_t d_up_stride, int64_t rows,
+                                                             int chunks_per_row) {
+  const int64_t total = rows * chunks_per_row;
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  for (int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x; c < total; c += stride) {
+    const int64_t r = c / chunks_per_row;
+    const int64_t col = (c - r * chunks_per_row) * P;
+    const Chunk<T, P> g = Chunk<T, P>::load(gate + r * gate_stride + col);
+    const Chunk<T, P> u = Chunk<T, P>::load(up + r * up_stride + col);
+    const Chunk<T, P> dy = Chunk<T, P>::load(d_out + r * d_out_stride + col);
+    Chunk<T, P> dg, du;
+#pragma unroll
+    for (int i = 0; i < P; ++i) {
+      const float gf = Elem<T>::up(g.e[i]), uf = Elem<T>::up(u.e[i]), dyf = Elem<T>::up(dy.e[i]);
+      const float sg = sigmoid_f32(gf);
+      const float gsg = gf * sg;
+      dg.e[i] = Elem<T>::down(dyf * uf * (sg + gsg * (1.0f - sg)));
+      du.e[i] = Elem<T>::down(dyf * gsg);
+    }
+    dg.store(d_gate + r * d_gate_stride + col);
+    du.store(d_up + r * d_up_stride + col);
+  }
+}
+
+template <typename T>
+bool view_vector_ok(const void* p, int64_t stride, int64_t rows) {
+  return aligned16(p) && (rows == 1 || stride % Elem<T>::per16 == 0);
+}
+
+inline unsigned grid_for(int64_t chunks) {
+  int64_t b = ceil_div(chunks, (int64_t)kBlock * 2);
+  if (b < 1) b = 1;
+  if (b > (1 << 20)) b = (1 << 20);
+  return (unsigned)b;
+}
+
+}  // namespace
+}  // namespace ck
+
+using namespace ck;
+
+extern "C" int ck_swiglu_fwd(const void* gate, int64_t gate_stride, const void* up, int64_t up_stride, void* out,
+                             int64_t out_stride, int64_t rows, int64_t cols, int32_t dtype, void* stream) {
+  CK_REQUIRE(rows >= 0 && cols >= 0, "ck_swiglu_fwd: negative size");
+  if (rows == 0 || cols == 0) return CK_OK;
+  CK_REQUIRE(gate && up && out, "ck_swiglu_fwd: NULL argument");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  CK_DISPATCH_FLOAT(dtype, "ck_swiglu_fwd", {
+    constexpr int P = Elem<scalar_t>::per16;
+    const scalar_t* g = static_cast<const scalar_t*>(gate);
+    const scalar_t* u = static_cast<const scalar_t*>(up);
+    scalar_t* o = static_cast<scalar_t*>(out);
+    const bool vec = view_vector_ok<scalar_t>(gate, gate_stride, rows) && view_vector_ok<scalar_t>(up, up_stride, rows) &&
+                     view_vector_ok<scalar_t>(out, out_stride, rows) && (cols % P == 0 || rows == 1);
+    int64_t done = 0;  // columns covered by the 128-bit kernel
+    if (vec && cols >= P) {
+      done = cols / P * P;
+      hipLaunchKernelGGL((swiglu_fwd_kernel<scalar_t, P>), dim3(grid_for(rows * (done / P))), dim3(kBlock), 0, s, g,
+                         gate_stride, u, up_stride, o, out_stride, rows, (int)(done / P));
+    }
+    if (done < cols) {  // misaligned views, or the ragged end of a flat tensor
+      const int64_t rest = cols - done;
+      hipLaunchKernelGGL((swiglu_fwd_kernel<scalar_t, 1>), dim3(grid_for(rows * rest)), dim3(kBlock), 0, s, g + done,
+                         gate_stride, u + done, up_stride, o + done, out_stride, rows, (int)rest);
+    }
+  });
+  CK_CHECK_LAUNCH("ck_swiglu_fwd");
+  return CK_OK;
+}
+
+extern "C" int ck_swiglu_bwd(const void* gate, int64_t gate_stride, const void* up, int64_t up_stride,
+                             const void* d_out, int64_t d_out_stride, void* d_gate, int64_t d_gate_stride, void* d_up,
+                             int64_t d_up_stride, int64_t rows, int64_t cols, int32_t dtype, void* stream) {
+  CK_REQUIRE(rows >= 0 && cols >= 0, "ck_swiglu_bwd: negative size");
+  if (rows == 0 || cols == 0) return CK_OK;
+  CK_REQUIRE(gate && up && d_out && d_gate && d_up, "ck_swiglu_bwd: NULL argument");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  CK_DISPATCH_FLOAT(dtype, "ck_swiglu_bwd", {
+    constexpr int P = Elem<scalar_t>::per16;
+    const scalar_t* g = static_cast<const scalar_t*>(gate);
+    const scalar_t* u = static_cast<const scalar_t*>(up);
+    const scalar_t* dy = static_cast<const scalar_t*>(d_out);
+    scalar_t* dg = static_cast<scalar_t*>(d_gate);
+    scalar_t* du = static_cast<scalar_t*>(d_up);
+    const bool vec = view_vector_ok<scalar_t>(gate, gate_stride, rows) && view_vector_ok<scalar_t>(up, up_stride, rows) &&
+                     view_vector_ok<scalar_t>(d_out, d_out_stride, rows) &&
+                     view_vector_ok<scalar_t>(d_gate, d_gate_stride, rows) &&
+                     view_vector_ok<scalar_t>(d_up, d_up_stride, rows) && (cols % P == 0 || rows == 1);
+    int64_t done = 0;
+    if (vec && cols >= P) {
+      done = cols / P * P;
+      hipLaunchKernelGGL((swiglu_bwd_kernel<scalar_t, P>), dim3(grid_for(rows * (done / P))), dim3(kBlock), 0, s, g,
+                         gate_stride, u, up_stride, dy, d_out_stride, dg, d_gate_stride, du, d_up_stride, rows,
+                         (int)(done / P));
+    }
+    if (done < cols) {
+      const int64_t rest = cols - done;
+      hipLaunchKernelGGL((swiglu_bwd_kernel<scalar_t, 1>), dim3(grid_for(rows * rest)), dim3(kBlock), 0, s, g + done,
+                         gate_stride, u + done, up_stride, dy + done, d_out_stride, dg + done, d_gate_stride,
+                         du + done, d_up_stride, rows, (int)rest);
+    }
+  });
+  CK_CHECK_LAUNCH("ck_swiglu_bwd");
+  return CK_OK;
+}

@@ -1,0 +1,22 @@
+"""MI355X-native implementation of the MoE hot path of cute-kernels, under the reference's Python API.
+
+Exports mirror the names the reference exposes for this path (cute_kernels/__init__.py:15-58 of the reference):
+the MoE layer, continuous_count_cute, swiglu_cute / swiglu_packed_cute, rmsnorm_cute. Everything runs through the
+ahead-of-time built libck_mi355.so; there is no other backend and no CPU path.
+"""
+
+from .continuous_count import continuous_count_and_offsets_cute, continuous_count_cute
+from .modules import Experts, MoE, MoE_Triton
+from .rmsnorm import rmsnorm_cute
+from .scattermoe import (
+    ExpertSegments,
+    experts_down,
+    experts_up,
+    gather_rows,
+    route_topk_softmax,
+    route_topk_softmax_raw,
+    sort_by_expert,
+    swiglu_experts,
+)
+from .swiglu import swiglu_cute, swiglu_packed_cute
+from .utils import ceil_divide, divide_if_divisible, get_num_elements_and_hidden_size, set_seed

@@ -1,0 +1,432 @@
+"""MoE expert path: routing, token->expert sort, scattered grouped GEMMs, gated combine -- forward and backward.
+
+Semantics follow cute_kernels/kernels/scattermoe/torch_implementation.py:63-201 (reference oracle) and the autograd
+conventions of cute_kernels/kernels/scattermoe/triton_implementation/ops.py:143-292. The data layout does not: rows
+are kept in a padded grouped order where every expert's segment starts at a multiple of the GEMM tile height, and the
+backward GEMMs consume transposed copies that the producing kernels write as they go, so that every matrix product is
+contraction-contiguous on both operands.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from dataclasses import dataclass
+
+import torch
+
+from . import _C
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# routing
+# ---------------------------------------------------------------------------------------------------------------
+class _RouteTopKSoftmax(torch.autograd.Function):
+    """logits [T, E] -> gates [T, k] (softmax over the k largest logits, in logits.dtype), selected [T, k] int64."""
+
+    @staticmethod
+    def forward(ctx, logits: torch.Tensor, k: int):
+        _C.require_gpu(logits)
+        logits = logits.contiguous()
+        T, E = logits.shape
+        selected = torch.empty(T, k, dtype=torch.int32, device=logits.device)
+        gates = torch.empty(T, k, dtype=torch.float32, device=logits.device)
+        lib = _C.lib()
+        with torch.cuda.device(logits.device):
+            _C.check(
+                lib.ck_route_topk_softmax(
+                    _C.ptr(logits), _C.dtype_code(logits.dtype), T, E, k, _C.ptr(selected), _C.ptr(gates), None, _C.stream()
+                )
+            )
+        ctx.save_for_backward(gates, selected)
+        ctx.E = E
+        ctx.dtype = logits.dtype
+        selected_long = selected.long()
+        ctx.mark_non_differentiable(selected_long)
+        return gates.to(logits.dtype), selected_long
+
+    @staticmethod
+    def backward(ctx, d_gates: torch.Tensor, _d_selected):
+        gates, selected = ctx.saved_tensors
+        T, k = gates.shape
+        d_gates = d_gates.float().contiguous()
+        d_logits = torch.empty(T, ctx.E, dtype=ctx.dtype, device=gates.device)
+        lib = _C.lib()
+        with torch.cuda.device(gates.device):
+            _C.check(
+                lib.ck_route_topk_softmax_bwd(
+                    _C.ptr(gates), _C.ptr(d_gates), _C.ptr(selected), T, ctx.E, k, _C.ptr(d_logits),
+                    _C.dtype_code(ctx.dtype), _C.stream(),
+                )
+            )
+        return d_logits, None
+
+
+def route_topk_softmax(logits: torch.Tensor, k: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """Top-k over the logits and softmax over the k selected logits in fp32, cast back to logits.dtype
+    (torch_implementation.py:122-135). Equal logits: the lowest expert index wins."""
+    return _RouteTopKSoftmax.apply(logits, k)
+
+
+@torch.no_grad()
+def route_topk_softmax_raw(logits: torch.Tensor, k: int) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """(selected int32 [T, k], gates fp32 [T, k], top-k values [T, k] in logits.dtype), no autograd."""
+    _C.require_gpu(logits)
+    logits = logits.contiguous()
+    T, E = logits.shape
+    selected = torch.empty(T, k, dtype=torch.int32, device=logits.device)
+    gates = torch.empty(T, k, dtype=torch.float32, device=logits.device)
+    values = torch.empty(T, k, dtype=logits.dtype, device=logits.device)
+    lib = _C.lib()
+    with torch.cuda.device(logits.device):
+        _C.check(
+            lib.ck_route_topk_softmax(
+                _C.ptr(logits), _C.dtype_code(logits.dtype), T, E, k, _C.ptr(selected), _C.ptr(gates), _C.ptr(values),
+                _C.stream(),
+            )
+        )
+    return selected, gates, values
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# sort + segments
+# ---------------------------------------------------------------------------------------------------------------
+@dataclass
+class ExpertSegments:
+    """Result of the stable sort by expert, in the reference's vocabulary plus the padded grouped layout."""
+
+    sorted_expert_idxs: torch.Tensor  # int32 [R]
+    sorted_scattered_idxs: torch.Tensor  # int32 [R]
+    counts: torch.Tensor  # uint32 [E]
+    ends: torch.Tensor  # uint32 [E]  inclusive prefix sums (the reference's expert_offsets)
+    starts: torch.Tensor  # uint32 [E]  exclusive prefix sums
+    seg_starts: torch.Tensor  # int32 [E + 1]
+    row_slot: torch.Tensor  # int32 [max_rows]
+    tile_expert: torch.Tensor  # int32 [max_rows / align]
+    max_rows: int
+    num_experts: int
+    align: int
+
+    def c_struct(self) -> _C.ck_segments:
+        return _C.ck_segments(
+            self.seg_starts.data_ptr(),
+            self.counts.data_ptr(),
+            self.tile_expert.data_ptr(),
+            self.row_slot.data_ptr(),
+            self.max_rows,
+            self.num_experts,
+            self.align,
+        )
+
+    @property
+    def ld_t(self) -> int:
+        """Leading dimension of transposed padded-grouped operands."""
+        return self.max_rows
+
+
+def choose_align(num_rows: int, num_experts: int) -> int:
+    """Tile height of the padded layout: 256-row tiles once experts average at least 2048 rows, else 128."""
+    return 256 if num_rows >= 2048 * num_experts else 128
+
+
+@torch.no_grad()
+def sort_by_expert(expert_ids: torch.Tensor, num_experts: int, align: int | None = None) -> ExpertSegments:
+    """Stable sort of the flat (token, slot) expert ids, with counts / offsets and the tile-aligned segment tables."""
+    _C.require_gpu(expert_ids)
+    assert expert_ids.dtype in (torch.int32, torch.long)
+    ids = expert_ids.contiguous().view(-1)
+    R = ids.numel()
+    if align is None:
+        align = choose_align(R, num_experts)
+    lib = _C.lib()
+    dev = ids.device
+    max_rows = lib.ck_sort_max_rows(R, num_experts, align)
+    i32 = dict(dtype=torch.int32, device=dev)
+    u32 = dict(dtype=torch.uint32, device=dev)
+    seg = ExpertSegments(
+        sorted_expert_idxs=torch.empty(R, **i32),
+        sorted_scattered_idxs=torch.empty(R, **i32),
+        counts=torch.empty(num_experts, **u32),
+        ends=torch.empty(num_experts, **u32),
+        starts=torch.empty(num_experts, **u32),
+        seg_starts=torch.empty(num_experts + 1, **i32),
+        row_slot=torch.empty(max(max_rows, 1), **i32),
+        tile_expert=torch.empty(max(max_rows // align, 1), **i32),
+        max_rows=max_rows,
+        num_experts=num_experts,
+        align=align,
+    )
+    ws = _C.zero_workspace(dev, lib.ck_sort_workspace_words(R, num_experts), "sort")
+    with torch.cuda.device(dev):
+        _C.check(
+            lib.ck_sort_by_expert(
+                _C.ptr(ids), int(ids.dtype == torch.long), R, num_experts, align, _C.ptr(seg.sorted_expert_idxs),
+                _C.ptr(seg.sorted_scattered_idxs), _C.ptr(seg.counts), _C.ptr(seg.ends), _C.ptr(seg.starts),
+                _C.ptr(seg.seg_starts), _C.ptr(seg.row_slot), _C.ptr(seg.tile_expert), _C.ptr(ws), _C.stream(),
+            )
+        )
+    return seg
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# thin launch helpers (allocate outputs, pass pointers)
+# ---------------------------------------------------------------------------------------------------------------
+def _gemm(a, gather_div, w, seg: ExpertSegments, epilogue, y, y_t=None, aux=None, aux_in=None):
+    E, N, K = w.shape
+    cs = seg.c_struct()
+    with torch.cuda.device(w.device):
+        _C.check(
+            _C.lib().ck_grouped_gemm(
+                _C.ptr(a), gather_div, _C.ptr(w), N, K, ctypes.byref(cs), epilogue, _C.ptr(y), _C.ptr(y_t), seg.ld_t,
+                _C.ptr(aux), _C.ptr(aux_in), _C.dtype_code(w.dtype), _C.stream(),
+            )
+        )
+
+
+def _gemm_dw(a_t, b_t, seg: ExpertSegments, dw):
+    E, M, N = dw.shape
+    cs = seg.c_struct()
+    with torch.cuda.device(dw.device):
+        _C.check(
+            _C.lib().ck_grouped_gemm_dw(
+                _C.ptr(a_t), _C.ptr(b_t), seg.ld_t, M, N, ctypes.byref(cs), _C.ptr(dw), _C.dtype_code(dw.dtype), _C.stream()
+            )
+        )
+
+
+def _group_rows(src, coeff, fan_out, seg: ExpertSegments, want_grouped: bool, want_transposed: bool):
+    """Padded grouped copy of `src` rows (fan_out == 0: src is already padded-grouped) and / or its transpose."""
+    H = src.size(-1)
+    grouped = torch.empty(seg.max_rows, H, dtype=src.dtype, device=src.device) if want_grouped else None
+    grouped_t = torch.empty(H, seg.ld_t, dtype=src.dtype, device=src.device) if want_transposed else None
+    with torch.cuda.device(src.device):
+        _C.check(
+            _C.lib().ck_group_rows_padded(
+                _C.ptr(src), _C.ptr(coeff), fan_out, H, _C.ptr(seg.row_slot), _C.ptr(seg.seg_starts), _C.ptr(seg.counts),
+                _C.ptr(seg.tile_expert), seg.align, seg.max_rows, _C.ptr(grouped), _C.ptr(grouped_t), seg.ld_t,
+                _C.dtype_code(src.dtype), _C.stream(),
+            )
+        )
+    return grouped, grouped_t
+
+
+def _transpose_weights(w: torch.Tensor) -> torch.Tensor:
+    E, N, K = w.shape
+    w_t = torch.empty(E, K, N, dtype=w.dtype, device=w.device)
+    with torch.cuda.device(w.device):
+        _C.check(_C.lib().ck_transpose_batched(_C.ptr(w), E, N, K, _C.ptr(w_t), _C.dtype_code(w.dtype), _C.stream()))
+    return w_t
+
+
+def _combine(expanded, gates, T, k, H, grad_out=None, want_out=True, want_d_gates=False):
+    out = torch.empty(T, H, dtype=expanded.dtype, device=expanded.device) if want_out else None
+    d_gates = torch.empty(T, k, dtype=expanded.dtype, device=expanded.device) if want_d_gates else None
+    with torch.cuda.device(expanded.device):
+        _C.check(
+            _C.lib().ck_combine_rows(
+                _C.ptr(expanded), _C.ptr(gates), T, k, H, _C.ptr(out), _C.ptr(grad_out), _C.ptr(d_gates),
+                _C.dtype_code(expanded.dtype), _C.stream(),
+            )
+        )
+    return out, d_gates
+
+
+def gather_rows(src: torch.Tensor, idx: torch.Tensor, coeff: torch.Tensor | None = None, fan_out: int = 1) -> torch.Tensor:
+    """out[n] = src[idx[n] // fan_out] * coeff[idx[n]] -- the reference's `group` (ops.py:108-140)."""
+    _C.require_gpu(src, idx)
+    src = src.contiguous()
+    out = torch.empty(idx.numel(), src.size(-1), dtype=src.dtype, device=src.device)
+    with torch.cuda.device(src.device):
+        _C.check(
+            _C.lib().ck_gather_rows(
+                _C.ptr(src), _C.ptr(idx), _C.ptr(coeff), fan_out, idx.numel(), src.size(-1), _C.ptr(out),
+                _C.dtype_code(src.dtype), _C.stream(),
+            )
+        )
+    return out
+
+
+def _check_expert_dtypes(x: torch.Tensor, *weights: torch.Tensor) -> None:
+    if x.dtype not in (torch.bfloat16, torch.float16):
+        raise NotImplementedError(
+            f"the MI355X expert GEMMs take bf16 / fp16 inputs with fp32 accumulation; got {x.dtype}"
+        )
+    for w in weights:
+        assert w.dtype == x.dtype, "expert weights and activations should have the same dtype"
+    assert x.size(-1) % 8 == 0, "hidden size should be a multiple of 8"
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# generic expert linears (any activation between them)
+# ---------------------------------------------------------------------------------------------------------------
+class _ExpertsUp(torch.autograd.Function):
+    """x [T, H] (token order) -> y [max_rows, N] (padded grouped): the reference's c_fc with grouped_out=True."""
+
+    @staticmethod
+    def forward(ctx, x, w, seg: ExpertSegments, k: int):
+        x = x.contiguous()
+        w = w.contiguous()
+        E, N, K = w.shape
+        # pad rows are never written by the kernel; zeros keep any activation applied on top finite
+        y = torch.zeros(seg.max_rows, N, dtype=x.dtype, device=x.device)
+        _gemm(x, k, w, seg, _C.CK_EPI_GROUPED, y)
+        ctx.save_for_backward(x, w)
+        ctx.seg, ctx.k = seg, k
+        return y
+
+    @staticmethod
+    def backward(ctx, d_y):
+        x, w = ctx.saved_tensors
+        seg, k = ctx.seg, ctx.k
+        T, K = x.shape
+        d_y = d_y.contiguous()
+        d_x = d_w = None
+        if ctx.needs_input_grad[1]:
+            _, d_y_t = _group_rows(d_y, None, 0, seg, False, True)
+            _, x_t = _group_rows(x, None, k, seg, False, True)
+            d_w = torch.empty_like(w)
+            _gemm_dw(d_y_t, x_t, seg, d_w)
+        if ctx.needs_input_grad[0]:
+            w_t = _transpose_weights(w)  # [E, K, N]
+            d_expanded = torch.empty(T * k, K, dtype=x.dtype, device=x.device)
+            _gemm(d_y, 0, w_t, seg, _C.CK_EPI_SCATTER, d_expanded)
+            d_x = d_expanded if k == 1 else _combine(d_expanded, None, T, k, K)[0]
+        return d_x, d_w, None, None
+
+
+class _ExpertsDown(torch.autograd.Function):
+    """h [max_rows, I] (padded grouped), gates [T, k] -> out [T, H]: the reference's c_proj with grouped_in=True."""
+
+    @staticmethod
+    def forward(ctx, h, w, gates, seg: ExpertSegments):
+        h = h.contiguous()
+        w = w.contiguous()
+        gates = gates.contiguous()
+        T, k = gates.shape
+        E, N, K = w.shape
+        expanded = torch.empty(T * k, N, dtype=h.dtype, device=h.device)
+        _gemm(h, 0, w, seg, _C.CK_EPI_SCATTER, expanded)
+        out, _ = _combine(expanded, gates, T, k, N)
+        ctx.save_for_backward(h, w, gates, expanded)
+        ctx.seg = seg
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        h, w, gates, expanded = ctx.saved_tensors
+        seg = ctx.seg
+        T, k = gates.shape
+        E, N, K = w.shape
+        grad_out = grad_out.contiguous()
+        d_h = d_w = d_gates = None
+        if ctx.needs_input_grad[2]:
+            _, d_gates = _combine(expanded, None, T, k, N, grad_out=grad_out, want_out=False, want_d_gates=True)
+        need_w = ctx.needs_input_grad[1]
+        d_y, d_y_t = _group_rows(grad_out, gates, k, seg, True, need_w)
+        if need_w:
+            _, h_t = _group_rows(h, None, 0, seg, False, True)
+            d_w = torch.empty_like(w)
+            _gemm_dw(d_y_t, h_t, seg, d_w)
+        if ctx.needs_input_grad[0]:
+            w_t = _transpose_weights(w)  # [E, K, N]
+            d_h = torch.zeros(seg.max_rows, K, dtype=h.dtype, device=h.device)
+            _gemm(d_y, 0, w_t, seg, _C.CK_EPI_GROUPED, d_h)
+        return d_h, d_w, d_gates, None
+
+
+def experts_up(x: torch.Tensor, weight: torch.Tensor, seg: ExpertSegments, k: int) -> torch.Tensor:
+    _C.require_gpu(x, weight)
+    _check_expert_dtypes(x, weight)
+    return _ExpertsUp.apply(x, weight, seg, k)
+
+
+def experts_down(h: torch.Tensor, weight: torch.Tensor, gates: torch.Tensor, seg: ExpertSegments) -> torch.Tensor:
+    _C.require_gpu(h, weight, gates)
+    _check_expert_dtypes(h, weight)
+    return _ExpertsDown.apply(h, weight, gates.to(h.dtype), seg)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# fused SwiGLU expert block
+# ---------------------------------------------------------------------------------------------------------------
+class _SwigluExperts(torch.autograd.Function):
+    """out = combine_k( gates * c_proj( swiglu_packed( c_fc(x) ) ) ) with the SwiGLU forward fused into the c_fc
+    epilogue and the SwiGLU backward fused into the epilogue of the c_proj input-gradient GEMM."""
+
+    @staticmethod
+    def forward(ctx, x, w_fc, w_proj, gates, seg: ExpertSegments):
+        x = x.contiguous()
+        w_fc = w_fc.contiguous()
+        w_proj = w_proj.contiguous()
+        gates = gates.contiguous()
+        T, H = x.shape
+        k = gates.size(1)
+        E, two_i, _ = w_fc.shape
+        I = two_i // 2
+        dev, dt = x.device, x.dtype
+        need_grad = any(ctx.needs_input_grad[:4])
+
+        pre = torch.empty(seg.max_rows, two_i, dtype=dt, device=dev)
+        act = torch.empty(seg.max_rows, I, dtype=dt, device=dev)
+        act_t = torch.empty(I, seg.ld_t, dtype=dt, device=dev) if ctx.needs_input_grad[2] else None
+        _gemm(x, k, w_fc, seg, _C.CK_EPI_SWIGLU, pre, y_t=act_t, aux=act)
+
+        expanded = torch.empty(T * k, H, dtype=dt, device=dev)
+        _gemm(act, 0, w_proj, seg, _C.CK_EPI_SCATTER, expanded)
+        out, _ = _combine(expanded, gates, T, k, H)
+
+        if need_grad:
+            ctx.save_for_backward(x, w_fc, w_proj, gates, pre, act_t, expanded)
+        ctx.seg = seg
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, w_fc, w_proj, gates, pre, act_t, expanded = ctx.saved_tensors
+        seg = ctx.seg
+        T, H = x.shape
+        k = gates.size(1)
+        E, two_i, _ = w_fc.shape
+        I = two_i // 2
+        dev, dt = x.device, x.dtype
+        grad_out = grad_out.contiguous()
+        need_x, need_fc, need_proj, need_gates = ctx.needs_input_grad[:4]
+        d_x = d_w_fc = d_w_proj = d_gates = None
+
+        if need_gates:
+            _, d_gates = _combine(expanded, None, T, k, H, grad_out=grad_out, want_out=False, want_d_gates=True)
+
+        # gate-scaled grad_out rows in padded grouped order (+ transpose for d_w_proj)
+        d_y, d_y_t = _group_rows(grad_out, gates, k, seg, True, need_proj)
+        if need_proj:
+            d_w_proj = torch.empty_like(w_proj)
+            _gemm_dw(d_y_t, act_t, seg, d_w_proj)
+            del d_y_t
+
+        if need_x or need_fc:
+            # d_act = d_y @ w_proj, SwiGLU backward in the epilogue -> d_pre (+ transpose for d_w_fc)
+            w_proj_t = _transpose_weights(w_proj)  # [E, I, H]
+            d_pre = torch.empty(seg.max_rows, two_i, dtype=dt, device=dev)
+            d_pre_t = torch.empty(two_i, seg.ld_t, dtype=dt, device=dev) if need_fc else None
+            _gemm(d_y, 0, w_proj_t, seg, _C.CK_EPI_SWIGLU_BWD, d_pre, y_t=d_pre_t, aux_in=pre)
+            del w_proj_t, d_y
+            if need_fc:
+                _, x_t = _group_rows(x, None, k, seg, False, True)
+                d_w_fc = torch.empty_like(w_fc)
+                _gemm_dw(d_pre_t, x_t, seg, d_w_fc)
+                del d_pre_t, x_t
+            if need_x:
+                w_fc_t = _transpose_weights(w_fc)  # [E, H, 2I]
+                d_expanded = torch.empty(T * k, H, dtype=dt, device=dev)
+                _gemm(d_pre, 0, w_fc_t, seg, _C.CK_EPI_SCATTER, d_expanded)
+                d_x = d_expanded if k == 1 else _combine(d_expanded, None, T, k, H)[0]
+        return d_x, d_w_fc, d_w_proj, d_gates, None
+
+
+def swiglu_experts(
+    x: torch.Tensor, w_fc: torch.Tensor, w_proj: torch.Tensor, gates: torch.Tensor, seg: ExpertSegments
+) -> torch.Tensor:
+    """Fused expert block for `activation_function = swiglu_packed_cute`, `is_glu=True` (c_fc columns [up | gate])."""
+    _C.require_gpu(x, w_fc, w_proj, gates)
+    _check_expert_dtypes(x, w_fc, w_proj)
+    assert w_fc.size(1) % 16 == 0, "intermediate size should be a multiple of 8"
+    return _SwigluExperts.apply(x, w_fc, w_proj, gates.to(x.dtype), seg)

@@ -1,0 +1,201 @@
+/*
+ * ck_mi355.h -- C ABI of libck_mi355.so: the MoE hot path of cute-kernels on one MI355X (gfx950).
+ *
+ * Conventions (all entry points):
+ *   - plain pointers and sizes only; every pointer is DEVICE memory unless said otherwise;
+ *   - the caller allocates every output and every workspace; the library never allocates device memory;
+ *   - `stream` is a hipStream_t passed as void*; launches are asynchronous on it, nothing synchronises the host;
+ *   - return value 0 = launched; non-zero = rejected (bad argument or launch failure), and
+ *     ck_last_error_string() then holds a thread-local message;
+ *   - `dtype` codes: CK_F32 = 0, CK_F16 = 1, CK_BF16 = 2;
+ *   - activations are row-major and contiguous; expert weights are [E, out_features, in_features] with
+ *     in_features contiguous, exactly as the reference stores them
+ *     (cute_kernels/kernels/scattermoe/torch_implementation.py:18).
+ *
+ * Each declaration cites the reference interface it replaces (paths relative to the reference root).
+ */
+#ifndef CK_MI355_H
+#define CK_MI355_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define CK_F32 0
+#define CK_F16 1
+#define CK_BF16 2
+
+#define CK_OK 0
+#define CK_ERR_ARG 1
+#define CK_ERR_LAUNCH 2
+
+/* Message for the last non-zero return on this thread ("" if none). Host pointer, valid until the next failing call. */
+const char* ck_last_error_string(void);
+/* ABI revision of the library; bumps when a signature changes. */
+int32_t ck_abi_version(void);
+
+/* ---------------------------------------------------------------------------------------------------------------
+ * (a) expert histogram + offsets
+ * Replaces: continuous_count_cuda(x, output, C, ...) -- cute_kernels/kernels/continuous_count/cuda_implementation/
+ *           ops.cpp:7-15, forward.cu:72-178 -- and the bincount(...).cumsum(-1) of
+ *           cute_kernels/kernels/scattermoe/triton_implementation/ops.py:19-28.
+ * ids: n values, int32 (ids_are_i64 = 0) or int64 (1). Values outside [0, num_bins) are not counted.
+ * counts[num_bins] (uint32) is required; ends (inclusive prefix sum) and starts (exclusive) may be NULL.
+ * workspace: ck_count_workspace_words(num_bins) uint32 words that are ALL ZERO on entry; the kernel leaves them
+ * all zero again on exit, so one zero-initialised buffer per stream can be reused forever.
+ * num_bins <= 16384 (same cap as forward.cu:12).
+ * ------------------------------------------------------------------------------------------------------------- */
+int64_t ck_count_workspace_words(int32_t num_bins);
+int ck_count_offsets(const void* ids, int32_t ids_are_i64, int64_t n, int32_t num_bins, uint32_t* counts,
+                     uint32_t* ends, uint32_t* starts, uint32_t* workspace, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------------
+ * (b1) router: top-k over logits, softmax over the k selected logits
+ * Replaces: MoE_Torch._get_topk + F.softmax(values.float()) --
+ *           cute_kernels/kernels/scattermoe/torch_implementation.py:122-135,195-201.
+ * logits [T, E] of `dtype`. selected [T, k] int32 (descending by logit; equal logits: lowest expert index first).
+ * gates [T, k] fp32 = softmax over the k selected logits. topk_values [T, k] of `dtype` may be NULL.
+ * E <= 1024, 1 <= k <= min(E, 32).
+ * ------------------------------------------------------------------------------------------------------------- */
+int ck_route_topk_softmax(const void* logits, int32_t dtype, int64_t T, int32_t E, int32_t k, int32_t* selected,
+                          float* gates, void* topk_values, void* stream);
+/* Backward of the above with respect to the logits (autograd of topk + softmax at
+ * torch_implementation.py:127-133): d_logits [T, E] of `dtype`, every element written (zeros off the selection).
+ * d_gates [T, k] fp32. */
+int ck_route_topk_softmax_bwd(const float* gates, const float* d_gates, const int32_t* selected, int64_t T,
+                              int32_t E, int32_t k, void* d_logits, int32_t dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------------
+ * (b2) stable sort of (token, slot) pairs by expert + tile-aligned expert segments
+ * Replaces: selected_experts.flatten().sort() and bincount(...).cumsum(-1) --
+ *           cute_kernels/kernels/scattermoe/triton_implementation/__init__.py:82-83; the argsort / bincount of
+ *           torch_implementation.py:171-193.
+ * expert_ids: R = T*k flat ids (int32 or int64), all in [0, E). E <= 4096.
+ * Outputs (all int32 unless noted):
+ *   sorted_expert_idxs[R], sorted_scattered_idxs[R]  -- the stable sort and its permutation
+ *   counts[E], ends[E], starts[E] (uint32)            -- histogram, inclusive and exclusive prefix sums
+ *   seg_starts[E + 1]  -- start row of each expert in the PADDED grouped layout: every expert's segment begins at
+ *                         a multiple of `align` rows; seg_starts[E] = number of padded rows in use
+ *   row_slot[max_rows] -- padded row p of expert e (seg_starts[e] <= p < seg_starts[e] + counts[e]) holds the flat
+ *                         (token, slot) index sorted_scattered_idxs[starts[e] + p - seg_starts[e]]; other rows
+ *                         are left unwritten
+ *   tile_expert[max_tiles] -- expert that owns rows [t*align, (t+1)*align) of the padded layout, -1 past the end
+ * max_rows = ck_sort_max_rows(R, E, align), max_tiles = max_rows / align.
+ * workspace: ck_sort_workspace_words(R, E) uint32 words; word 0 must be zero on entry and is zero again on exit.
+ * ------------------------------------------------------------------------------------------------------------- */
+int64_t ck_sort_max_rows(int64_t R, int32_t E, int32_t align);
+int64_t ck_sort_workspace_words(int64_t R, int32_t E);
+int ck_sort_by_expert(const void* expert_ids, int32_t ids_are_i64, int64_t R, int32_t E, int32_t align,
+                      int32_t* sorted_expert_idxs, int32_t* sorted_scattered_idxs, uint32_t* counts, uint32_t* ends,
+                      uint32_t* starts, int32_t* seg_starts, int32_t* row_slot, int32_t* tile_expert,
+                      uint32_t* workspace, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------------
+ * (b3) token-row gather / gated combine
+ * Replaces: group(...) / group_triton_kernel -- triton_implementation/ops.py:108-140, kernels.py:225-280 -- and the
+ *           bmm-based combine and d_gates of ops.py:173-174,214, and the .sum(-2) of ops.py:273-276.
+ * ------------------------------------------------------------------------------------------------------------- */
+/* out[n, :] = src[idx[n] / fan_out, :] * (coeff ? coeff[idx[n]] : 1), n < num_rows; src [*, H], out [num_rows, H].
+ * coeff has the dtype of src. H * sizeof(dtype) must be a multiple of 16. */
+int ck_gather_rows(const void* src, const int32_t* idx, const void* coeff, int32_t fan_out, int64_t num_rows,
+                   int32_t H, void* out, int32_t dtype, void* stream);
+/* out[t, :] = sum_j (gates ? gates[t, j] : 1) * expanded[t, j, :], fp32 accumulation; expanded [T, k, H].
+ * If d_gates_out != NULL (needs grad_out [T, H]): d_gates_out[t, j] = <expanded[t, j, :], grad_out[t, :]> and `out`
+ * may be NULL. gates / d_gates_out have the dtype of expanded. */
+int ck_combine_rows(const void* expanded, const void* gates, int64_t T, int32_t k, int32_t H, void* out,
+                    const void* grad_out, void* d_gates_out, int32_t dtype, void* stream);
+/* Padded grouped copy of token rows and (optionally) its transpose, for the grouped GEMMs below:
+ *   row p valid : grouped[p, :] = src[row_slot[p] / fan_out, :] * (coeff ? coeff[row_slot[p]] : 1)
+ *   row p pad   : zeros
+ * fan_out == 0 (coeff must be NULL): src is itself padded-grouped [max_rows, H] and valid row p reads src[p, :].
+ * grouped [max_rows, H] may be NULL; grouped_t [H, ld_t] (ld_t >= max_rows) may be NULL. bf16 / f16 only. */
+int ck_group_rows_padded(const void* src, const void* coeff, int32_t fan_out, int32_t H, const int32_t* row_slot,
+                         const int32_t* seg_starts, const uint32_t* counts, const int32_t* tile_expert,
+                         int32_t align, int64_t max_rows, void* grouped, void* grouped_t, int64_t ld_t,
+                         int32_t dtype, void* stream);
+/* Batched 2-D transpose: dst[b, c, r] = src[b, r, c]; src [batch, rows, cols]. 16-bit dtypes only. */
+int ck_transpose_batched(const void* src, int64_t batch, int32_t rows, int32_t cols, void* dst, int32_t dtype,
+                         void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------------
+ * (c) scattered grouped GEMMs over tile-aligned expert segments (bf16 / f16 inputs, fp32 accumulation on MFMA)
+ * Replaces: scatter2scatter + scatter2scatter_triton_kernel -- triton_implementation/ops.py:31-78, kernels.py:12-133 --
+ *           group_bwd_W + groupXtY_triton_kernel -- ops.py:81-105, kernels.py:136-222 -- and the per-expert
+ *           F.linear loop of torch_implementation.py:32-49.
+ * Shared layout arguments come from ck_sort_by_expert (same `align`; align must be 128 or 256).
+ * K and N must be multiples of 8.
+ * ------------------------------------------------------------------------------------------------------------- */
+typedef struct ck_segments {
+  const int32_t* seg_starts;  /* [E + 1] */
+  const uint32_t* counts;     /* [E] */
+  const int32_t* tile_expert; /* [max_rows / align] */
+  const int32_t* row_slot;    /* [max_rows] */
+  int64_t max_rows;
+  int32_t num_experts;
+  int32_t align;
+} ck_segments;
+
+/* Y = A_e * W[e]^T for every expert segment e. W [E, N, K].
+ * A rows: a_gather_div > 0 : row p reads a[row_slot[p] / a_gather_div, :]   (a is [*, K], token order)
+ *         a_gather_div == 0: row p reads a[p, :]                            (a is padded-grouped [max_rows, K])
+ * Epilogue, selected by `epilogue`:
+ *   CK_EPI_GROUPED        : y [max_rows, N] padded-grouped (valid rows only); y_t [N, ld_t] transposed copy with
+ *                           zeros in pad rows, optional (NULL to skip)
+ *   CK_EPI_SCATTER        : y [R, N]: valid row p is written to row row_slot[p] (back to (token, slot) order)
+ *   CK_EPI_SWIGLU         : N = 2*I packed [up | gate] (cute_kernels/kernels/swiglu/__init__.py:121): writes the
+ *                           pre-activation to y [max_rows, 2I], act = up*silu(gate) (computed from the rounded
+ *                           pre-activation, as the unfused path would) to aux [max_rows, I], and act^T to
+ *                           y_t [I, ld_t] (optional)
+ *   CK_EPI_SWIGLU_BWD     : the GEMM result is d_act [rows, N = I]; aux_in = saved pre-activation [max_rows, 2I];
+ *                           writes d_preact to y [max_rows, 2I] and its transpose to y_t [2I, ld_t] (optional)
+ *                           (backward formula: cute_kernels/kernels/swiglu/cuda_implementation/backward.cu:27-41)
+ */
+#define CK_EPI_GROUPED 0
+#define CK_EPI_SCATTER 1
+#define CK_EPI_SWIGLU 2
+#define CK_EPI_SWIGLU_BWD 3
+int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* w, int32_t N, int32_t K,
+                    const ck_segments* seg, int32_t epilogue, void* y, void* y_t, int64_t ld_t, void* aux,
+                    const void* aux_in, int32_t dtype, void* stream);
+/* dW[e] = A_t[:, seg_e] * B_t[:, seg_e]^T : A_t [M, ld_t], B_t [N, ld_t] are transposed padded-grouped operands with
+ * zeros in pad rows; dw [E, M, N]. Experts with no rows get exact zeros (ops.py:252, kernels.py:181). */
+int ck_grouped_gemm_dw(const void* a_t, const void* b_t, int64_t ld_t, int32_t M, int32_t N, const ck_segments* seg,
+                       void* dw, int32_t dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------------
+ * SwiGLU, stand-alone
+ * Replaces: swiglu_forward_cuda / swiglu_backward_cuda -- cute_kernels/kernels/swiglu/cuda_implementation/ops.cpp:7-22,
+ *           forward.cu:18-94, backward.cu:18-129 (and the strided Triton variants used for the packed form).
+ * gate/up/out are [rows, cols] views with row strides in ELEMENTS (so the two halves of a packed tensor can be
+ * passed without a copy). Any size is accepted; accesses are 128-bit when every pointer is 16-byte aligned and every
+ * row stride and cols are multiples of 16 bytes (a flat tensor, rows == 1, only needs the pointers aligned), element-wise
+ * otherwise.
+ * ------------------------------------------------------------------------------------------------------------- */
+int ck_swiglu_fwd(const void* gate, int64_t gate_stride, const void* up, int64_t up_stride, void* out,
+                  int64_t out_stride, int64_t rows, int64_t cols, int32_t dtype, void* stream);
+int ck_swiglu_bwd(const void* gate, int64_t gate_stride, const void* up, int64_t up_stride, const void* d_out,
+                  int64_t d_out_stride, void* d_gate, int64_t d_gate_stride, void* d_up, int64_t d_up_stride,
+                  int64_t rows, int64_t cols, int32_t dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------------
+ * (d) RMSNorm
+ * Replaces: rmsnorm_forward_triton / rmsnorm_backward_triton -- cute_kernels/kernels/rmsnorm/triton_implementation/
+ *           forward.py:14-85, backward.py:14-129; numerics follow F.rms_norm (rmsnorm/torch_implementation.py:9-10):
+ *           the weight multiply happens in fp32 before the single rounding.
+ * x, out, d_out, d_x [B, H] contiguous; weight [H] or NULL; rstd [B] fp32 or NULL (forward: written if non-NULL;
+ * backward: read if non-NULL, recomputed from x and eps otherwise).
+ * backward: d_weight_partial [ck_rmsnorm_bwd_partial_rows(B), H] fp32 workspace and d_weight [H] fp32 output, both
+ * NULL when weight is NULL.
+ * ------------------------------------------------------------------------------------------------------------- */
+int ck_rmsnorm_fwd(const void* x, const void* weight, float eps, int64_t B, int32_t H, void* out, float* rstd,
+                   int32_t dtype, void* stream);
+int64_t ck_rmsnorm_bwd_partial_rows(int64_t B);
+int ck_rmsnorm_bwd(const void* x, const void* weight, const void* d_out, const float* rstd, float eps, int64_t B,
+                   int32_t H, void* d_x, float* d_weight_partial, float* d_weight, int32_t dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* CK_MI355_H */

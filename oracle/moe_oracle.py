@@ -1,0 +1,126 @@
+"""torch (CPU) restatement of the floating-point stages of the cute-kernels MoE path.
+
+TEST INFRASTRUCTURE ONLY -- the checker and the cpu_baseline of bench.py, never the product.
+
+The reference's oracle for these stages is itself a handful of torch library calls; this file restates them (it does
+not import the reference) and cites the lines it follows. Pinned in tests/test_oracle.py against an independent dense
+per-token formulation in fp64, closed forms and torch.autograd.gradcheck.
+"""
+
+from __future__ import annotations
+
+from typing import Callable
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+
+def continuous_count_torch(x: torch.Tensor, size: int) -> torch.Tensor:
+    """cute_kernels/kernels/continuous_count/torch_implementation.py:8-10"""
+    return x.bincount(minlength=size).to(torch.uint32)
+
+
+def swiglu_torch(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
+    """cute_kernels/kernels/swiglu/torch_implementation.py:9-18: fp32 math, one rounding."""
+    dtype = gate.dtype
+    return (up.float() * F.silu(gate.float())).to(dtype)
+
+
+def swiglu_packed_torch(x: torch.Tensor) -> torch.Tensor:
+    """cute_kernels/kernels/swiglu/torch_implementation.py:21-23: first half = up, second half = gate."""
+    up, gate = x.chunk(2, dim=-1)
+    return swiglu_torch(gate, up)
+
+
+def rmsnorm_torch(x: torch.Tensor, weight: torch.Tensor | None, eps: float | None) -> torch.Tensor:
+    """cute_kernels/kernels/rmsnorm/torch_implementation.py:9-10; eps=None -> finfo(dtype).eps as
+    cute_kernels/kernels/rmsnorm/__init__.py:23-24."""
+    if eps is None:
+        eps = torch.finfo(x.dtype).eps
+    return F.rms_norm(x, (x.size(-1),), weight=weight, eps=eps)
+
+
+def topk_lowest_index_first(logits: torch.Tensor, k: int) -> tuple[torch.Tensor, torch.Tensor]:
+    """Top-k with a fixed tie rule (equal logits: lowest expert index first). torch.topk's own tie order is
+    unspecified (torch_implementation.py:195-201 just calls it); values are identical either way."""
+    order = torch.sort(logits.float(), dim=-1, descending=True, stable=True).indices[..., :k]
+    return logits.gather(-1, order), order
+
+
+class ExpertsOracle(nn.Module):
+    """cute_kernels/kernels/scattermoe/torch_implementation.py:12-60"""
+
+    def __init__(self, num_experts: int, in_features: int, out_features: int, add_bias: bool, std: float) -> None:
+        super().__init__()
+        self.weight = nn.Parameter(torch.empty(num_experts, out_features, in_features))
+        self.bias = nn.Parameter(torch.empty(num_experts, out_features)) if add_bias else None
+        self.num_experts = num_experts
+        with torch.no_grad():
+            nn.init.normal_(self.weight, mean=0, std=std)
+            if self.bias is not None:
+                self.bias.zero_()
+
+    def forward(self, inputs, expert_frequency: torch.Tensor, return_list: bool):
+        if isinstance(inputs, torch.Tensor):
+            inputs = inputs.split(expert_frequency.tolist(), dim=0)
+        outs = [
+            F.linear(inputs[i], self.weight[i], None if self.bias is None else self.bias[i])
+            for i in range(self.num_experts)
+        ]
+        return outs if return_list else torch.cat(outs)
+
+
+class MoEOracle(nn.Module):
+    """cute_kernels/kernels/scattermoe/torch_implementation.py:63-201, with the tie rule of topk made explicit."""
+
+    def __init__(
+        self,
+        num_experts: int,
+        num_experts_per_tok: int,
+        hidden_size: int,
+        intermediate_size: int,
+        activation_function: Callable,
+        is_glu: bool,
+        add_bias: bool,
+        std: float,
+    ) -> None:
+        super().__init__()
+        self.num_experts = num_experts
+        self.top_k = num_experts_per_tok
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.gate = nn.Linear(hidden_size, num_experts, bias=False)
+        self.c_fc = ExpertsOracle(num_experts, hidden_size, 2 * intermediate_size if is_glu else intermediate_size, add_bias, std)
+        self.act = activation_function
+        self.c_proj = ExpertsOracle(num_experts, intermediate_size, hidden_size, add_bias, std)
+
+    def forward(self, hidden_states: torch.Tensor):
+        original_shape = hidden_states.shape
+        hidden_states = hidden_states.view(-1, self.hidden_size)
+        router_logits, router_weights, selected_experts = self._compute_routing_weights(hidden_states)
+        hidden_states = self._compute_experts(hidden_states, router_weights, selected_experts)
+        return hidden_states.view(original_shape), router_logits
+
+    def _compute_routing_weights(self, hidden_states: torch.Tensor):
+        router_logits = self.gate(hidden_states)                                  # :124
+        router_weights, selected_experts = topk_lowest_index_first(router_logits, self.top_k)  # :127, :195-201
+        router_weights = F.softmax(router_weights.float(), dim=-1)                # :132
+        router_weights = router_weights.type_as(hidden_states)                    # :133
+        return router_logits, router_weights, selected_experts
+
+    def _compute_experts(self, hidden_states, router_weights, selected_experts):
+        total_q = hidden_states.shape[0]
+        selected_experts = selected_experts.flatten()                             # :175
+        expert_frequency = selected_experts.bincount(minlength=self.num_experts)  # :179
+        index_sorted_experts = selected_experts.argsort(stable=True)              # :182
+        fan_in_index = index_sorted_experts // self.top_k                         # :184
+        batch_gates = router_weights.flatten()[index_sorted_experts]              # :188-190
+
+        hidden_states = hidden_states[fan_in_index]                               # :152
+        hidden_states = self.c_fc(hidden_states, expert_frequency, return_list=True)   # :156
+        hidden_states = [self.act(i) for i in hidden_states]                      # :158
+        hidden_states = self.c_proj(hidden_states, expert_frequency, return_list=False)  # :160
+        hidden_states = hidden_states * batch_gates.unsqueeze(-1)                 # :163
+        zeros = torch.zeros((total_q, self.hidden_size), dtype=hidden_states.dtype, device=hidden_states.device)
+        return zeros.index_add(0, fan_in_index, hidden_states)                    # :164-165

@@ -1,0 +1,224 @@
+"""Pins the CPU oracle (oracle/) before anything is compared against it.
+
+Each oracle function is checked against something that is NOT its own formula: a numpy/torch library routine, brute
+force on tiny inputs, an independent dense formulation in fp64, invariants, and the committed fixtures in tests/golden.
+"""
+
+import os
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import integer_oracle as io
+from oracle import moe_oracle as mo
+
+GOLDEN = np.load(os.path.join(os.path.dirname(__file__), "golden", "routing_fixtures.npz"))
+
+
+# ---- integer stages ------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("n,bins", [(0, 5), (1, 1), (7, 3), (1000, 72), (65536, 64), (4099, 16384)])
+def test_count_matches_bincount_and_brute_force(n, bins):
+    rng = np.random.default_rng(n + bins)
+    ids = rng.integers(0, bins, size=n, dtype=np.int64)
+    got = io.count(ids, bins)
+    assert got.dtype == np.uint32
+    np.testing.assert_array_equal(got, np.bincount(ids, minlength=bins))
+    if n <= 1000:
+        brute = [sum(1 for v in ids if v == e) for e in range(bins)]
+        np.testing.assert_array_equal(got, brute)
+    assert int(got.sum()) == n
+
+
+def test_count_ignores_out_of_range():
+    ids = np.array([-1, 0, 3, 3, 4, 100, 2**40], dtype=np.int64)
+    np.testing.assert_array_equal(io.count(ids, 4), [1, 0, 0, 2])
+
+
+def test_count_golden_c1():
+    ids = np.random.default_rng(int(GOLDEN["c1_seed"][0])).integers(0, 64, size=65536, dtype=np.int64)
+    counts = io.count(ids, 64)
+    np.testing.assert_array_equal(counts, GOLDEN["c1_counts"])
+    ends, starts = io.offsets(counts)
+    np.testing.assert_array_equal(ends, GOLDEN["c1_ends"])
+    np.testing.assert_array_equal(starts, GOLDEN["c1_starts"])
+
+
+def test_offsets_match_cumsum():
+    counts = np.random.default_rng(0).integers(0, 1000, size=129).astype(np.uint32)
+    ends, starts = io.offsets(counts)
+    np.testing.assert_array_equal(ends, np.cumsum(counts))
+    np.testing.assert_array_equal(starts, np.cumsum(counts) - counts)
+    assert ends[-1] == counts.sum() and starts[0] == 0
+    assert np.all(np.diff(ends.astype(np.int64)) >= 0)
+
+
+@pytest.mark.parametrize("n,E", [(0, 4), (1, 1), (50, 3), (32768, 8), (65536, 64), (5000, 128)])
+def test_sort_matches_stable_argsort(n, E):
+    rng = np.random.default_rng(n * 31 + E)
+    ids = rng.integers(0, E, size=n, dtype=np.int64)
+    se, ss = io.sort_by_expert(ids, E)
+    order = np.argsort(ids, kind="stable")
+    np.testing.assert_array_equal(ss, order)
+    np.testing.assert_array_equal(se, ids[order])
+    t_sorted, t_order = torch.sort(torch.from_numpy(ids), stable=True)
+    np.testing.assert_array_equal(ss, t_order.numpy())
+    np.testing.assert_array_equal(se, t_sorted.numpy())
+    # invariants: a permutation, keys non-decreasing, positions increasing inside each expert
+    assert sorted(ss.tolist()) == list(range(n))
+    assert np.all(np.diff(se) >= 0)
+    same = np.diff(se) == 0
+    assert np.all(np.diff(ss)[same] > 0)
+
+
+def test_sort_golden_small():
+    ids = GOLDEN["small_ids"]
+    E = int(GOLDEN["small_num_experts"][0])
+    se, ss = io.sort_by_expert(ids, E)
+    np.testing.assert_array_equal(se, GOLDEN["small_sorted_expert_idxs"])
+    np.testing.assert_array_equal(ss, GOLDEN["small_sorted_scattered_idxs"])
+    np.testing.assert_array_equal(io.count(ids, E), GOLDEN["small_counts"])
+
+
+@pytest.mark.parametrize("align", [1, 4, 128])
+def test_segments_brute_force(align):
+    rng = np.random.default_rng(align)
+    E = 6
+    ids = rng.choice(np.array([0, 1, 3, 5]), size=37).astype(np.int64)  # experts 2 and 4 are empty
+    counts = io.count(ids, E)
+    _, ss = io.sort_by_expert(ids, E)
+    max_rows = -(-(ids.size + E * (align - 1)) // align) * align
+    seg_starts, row_slot, tile_expert = io.segments(counts, ss, align, max_rows)
+    # brute force, expert by expert
+    run = 0
+    for e in range(E):
+        assert seg_starts[e] == run and run % align == 0
+        members = [i for i in range(ids.size) if ids[i] == e]  # already in increasing order = stable order
+        assert row_slot[run : run + len(members)].tolist() == members
+        padded = -(-len(members) // align) * align
+        assert np.all(row_slot[run + len(members) : run + padded] == -1)
+        assert np.all(tile_expert[run // align : (run + padded) // align] == e)
+        run += padded
+    assert seg_starts[E] == run
+    assert np.all(tile_expert[run // align :] == -1)
+    assert np.all(row_slot[run:] == -1)
+
+
+# ---- routing -------------------------------------------------------------------------------------------------
+def test_topk_values_and_non_tie_indices_match_torch_topk():
+    torch.manual_seed(0)
+    logits = torch.randn(2048, 64).to(torch.bfloat16).float()
+    k = 2
+    sel, gates, vals = io.topk_softmax(logits.numpy(), k)
+    t_vals, t_idx = logits.topk(k, dim=-1)
+    np.testing.assert_array_equal(vals, t_vals.numpy())  # values are unique whatever the tie order
+    srt = torch.sort(logits, dim=-1, descending=True).values
+    tie_rows = (srt[:, k - 1] == srt[:, k]) | (srt[:, 0] == srt[:, 1])
+    assert tie_rows.any() and not tie_rows.all()  # bf16-rounded logits do tie
+    np.testing.assert_array_equal(sel[~tie_rows.numpy()], t_idx.numpy()[~tie_rows.numpy()])
+    # tie rows: still a valid selection of the right values, without repeats
+    picked = np.take_along_axis(logits.numpy(), sel.astype(np.int64), axis=1)
+    np.testing.assert_array_equal(picked, vals)
+    assert all(len(set(r)) == k for r in sel.tolist())
+    # agrees with the stable descending sort (the tie rule, via a library routine)
+    o_vals, o_idx = mo.topk_lowest_index_first(logits, k)
+    np.testing.assert_array_equal(sel, o_idx.numpy())
+    np.testing.assert_array_equal(vals, o_vals.numpy())
+
+
+def test_topk_tie_rule_and_special_values():
+    row = np.array([[1.0, 3.0, 3.0, -0.0, 0.0, 3.0, np.nan, 2.0]], dtype=np.float32)
+    sel, gates, vals = io.topk_softmax(row, 5)
+    assert sel.tolist() == [[6, 1, 2, 5, 7]]  # NaN first (torch order), then equal 3.0s by index
+    sel, _, _ = io.topk_softmax(np.array([[0.0, -0.0, -0.0, 0.0]], dtype=np.float32), 4)
+    assert sel.tolist() == [[0, 1, 2, 3]]  # signed zeros tie
+
+
+def test_topk_gates_are_softmax_of_selected():
+    rng = np.random.default_rng(3)
+    logits = rng.standard_normal((257, 40)).astype(np.float32)
+    sel, gates, vals = io.topk_softmax(logits, 8)
+    expect = torch.softmax(torch.from_numpy(vals), dim=-1).numpy()
+    np.testing.assert_allclose(gates, expect, rtol=1e-6, atol=1e-7)
+    np.testing.assert_allclose(gates.sum(-1), 1.0, rtol=1e-6)
+    # equivalent to softmax over all experts, top-k, renormalise
+    full = torch.softmax(torch.from_numpy(logits).double(), dim=-1)
+    top = full.gather(-1, torch.from_numpy(sel.astype(np.int64)))
+    np.testing.assert_allclose(gates, (top / top.sum(-1, keepdim=True)).numpy(), rtol=1e-5)
+
+
+# ---- floating-point stages -------------------------------------------------------------------------------------
+def test_swiglu_closed_form_and_packed_order():
+    torch.manual_seed(1)
+    gate, up = torch.randn(33, 17, dtype=torch.float64), torch.randn(33, 17, dtype=torch.float64)
+    expect = up * gate / (1 + torch.exp(-gate))
+    # the reference computes in fp32 whatever the input dtype (.float(), swiglu/torch_implementation.py:11-12)
+    torch.testing.assert_close(mo.swiglu_torch(gate, up), expect, rtol=2e-6, atol=2e-6)
+    # packed: FIRST half is up, SECOND half is gate (reference swiglu/__init__.py:121)
+    torch.testing.assert_close(mo.swiglu_packed_torch(torch.cat([up, gate], -1)), expect, rtol=2e-6, atol=2e-6)
+    assert not torch.allclose(mo.swiglu_packed_torch(torch.cat([gate, up], -1)), expect)
+
+
+def test_rmsnorm_closed_form_and_gradcheck():
+    torch.manual_seed(2)
+    x = torch.randn(5, 24, dtype=torch.float64, requires_grad=True)
+    w = torch.randn(24, dtype=torch.float64, requires_grad=True)
+    eps = 1e-5
+    expect = x / torch.sqrt((x * x).mean(-1, keepdim=True) + eps) * w
+    torch.testing.assert_close(mo.rmsnorm_torch(x, w, eps), expect, rtol=1e-12, atol=1e-12)
+    assert torch.autograd.gradcheck(lambda a, b: mo.rmsnorm_torch(a, b, eps), (x, w))
+    # backward closed form of the reference README (rmsnorm/README.md:27-29)
+    dy = torch.randn(5, 24, dtype=torch.float64)
+    (gx,) = torch.autograd.grad(mo.rmsnorm_torch(x, w, eps), x, dy)
+    rstd = 1 / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+    expect_gx = rstd * dy * w - x * rstd**3 / 24 * (dy * w * x).sum(-1, keepdim=True)
+    torch.testing.assert_close(gx, expect_gx, rtol=1e-10, atol=1e-12)
+    assert mo.rmsnorm_torch(x.detach().float(), None, None).dtype == torch.float32
+
+
+def _dense_moe_fp64(moe: mo.MoEOracle, x: torch.Tensor) -> torch.Tensor:
+    """Independent formulation: per token, loop over its k experts; no sort, no bincount, no index_add."""
+    xd = x.double()
+    logits = xd @ moe.gate.weight.double().t()
+    out = torch.zeros_like(xd)
+    for t in range(xd.size(0)):
+        order = sorted(range(moe.num_experts), key=lambda e: (-float(logits[t, e]), e))[: moe.top_k]
+        v = torch.stack([logits[t, e] for e in order])
+        g = torch.exp(v - v.max())
+        g = g / g.sum()
+        for j, e in enumerate(order):
+            h = moe.c_fc.weight[e].double() @ xd[t]
+            h = moe.act(h)
+            out[t] += g[j] * (moe.c_proj.weight[e].double() @ h)
+    return out
+
+
+@pytest.mark.parametrize("is_glu", [True, False])
+@pytest.mark.parametrize("E,k", [(4, 2), (6, 4), (8, 1)])
+def test_moe_oracle_matches_dense_per_token_formulation(E, k, is_glu):
+    torch.manual_seed(E * 10 + k)
+    def glu64(v):  # [up | gate] packed SwiGLU kept in fp64 (swiglu_packed_torch itself computes in fp32)
+        up, gate = v.chunk(2, dim=-1)
+        return up * F.silu(gate)
+
+    act = glu64 if is_glu else torch.nn.GELU(approximate="tanh")
+    moe = mo.MoEOracle(E, k, 16, 24, act, is_glu, False, 0.5).double()
+    x = torch.randn(19, 16, dtype=torch.float64)
+    y, logits = moe(x)
+    torch.testing.assert_close(y, _dense_moe_fp64(moe, x), rtol=1e-9, atol=1e-11)
+    torch.testing.assert_close(logits, x @ moe.gate.weight.t())
+    assert y.shape == x.shape and logits.shape == (19, E)
+    # leading dims are flattened and restored (torch_implementation.py:103-120)
+    y3, _ = moe(x.view(1, 19, 16))
+    torch.testing.assert_close(y3.view(19, 16), y)
+
+
+def test_moe_oracle_state_dict_keys_and_shapes():
+    moe = mo.MoEOracle(4, 2, 16, 24, mo.swiglu_packed_torch, True, False, 0.02)
+    sd = moe.state_dict()
+    assert list(sd) == ["gate.weight", "c_fc.weight", "c_proj.weight"]
+    assert sd["gate.weight"].shape == (4, 16)
+    assert sd["c_fc.weight"].shape == (4, 48, 16)  # 2*I rows when is_glu
+    assert sd["c_proj.weight"].shape == (4, 16, 24)
+    assert abs(float(sd["c_fc.weight"].std()) - 0.02) < 0.005
