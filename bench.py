@@ -1,0 +1,271 @@
+"""Benchmark of the MoE hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu-baseline] [--skip-secondary]
+
+A step is one forward+backward of the Mixtral-shape MoE layer of the baseline (T=16,384 tokens, H=4096, E=8, top-2,
+I=14,336, SwiGLU, bf16 with fp32 accumulation, Zipf(1.0) expert load, synthetic data, inputs resident in HBM).
+Prints ONE JSON line: whole-layer TFLOP/s (expert-GEMM FLOPs 18*R*H*I over wall time, router and bookkeeping time
+included), the roofline record of the dominant kernel measured with events on the launch stream inside the timed
+region, and the torch CPU path (oracle/) timed on this box's host cores on a bounded sample.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "cute-kernels_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0  # MI355X HBM3E
+
+# workload: configs[2] of the baseline, the configuration its headline metric (MoE fwd+bwd TFLOP/s) is quoted on
+T, H, E, TOP_K, I = 16384, 4096, 8, 2, 14336
+SEED = 42
+
+
+def zipf_bias(logits, k: int, s: float = 1.0):
+    """Per-expert additive logit bias c*log(1/rank) with c chosen so the routed load is closest to Zipf(s)."""
+    import torch
+
+    E_ = logits.size(1)
+    ranks = torch.arange(1, E_ + 1, device=logits.device, dtype=torch.float32)
+    target = (1.0 / ranks**s) / (1.0 / ranks**s).sum()
+    best = None
+    for c in [x * 0.05 for x in range(0, 81)]:
+        bias = -c * torch.log(ranks)
+        sel = (logits.float() + bias).topk(k, dim=-1).indices.flatten()
+        freq = torch.bincount(sel, minlength=E_).float()
+        freq = freq / freq.sum()
+        err = float((freq - target).abs().sum())
+        if best is None or err < best[0]:
+            best = (err, c, bias, freq)
+    return best[2], best[3], best[1]
+
+
+def build_layer(dev):
+    import torch
+
+    import cute_kernels
+
+    torch.manual_seed(SEED)
+    moe = cute_kernels.MoE(E, TOP_K, H, I, cute_kernels.swiglu_packed_cute, True, False, 0.02)
+    moe = moe.to(torch.bfloat16).to(dev)
+    x = torch.randn(T, H, generator=torch.Generator().manual_seed(SEED)).to(torch.bfloat16).to(dev)
+    with torch.no_grad():
+        bias, freq, c = zipf_bias(moe.gate(x), TOP_K, 1.0)
+    bias = bias.to(torch.bfloat16)
+    # the router has no bias parameter (torch_implementation.py:83 of the reference): skew goes in through a hook
+    moe.gate.register_forward_hook(lambda mod, inp, out: out + bias)
+    grad_out = torch.randn(T, H, generator=torch.Generator().manual_seed(SEED + 1)).to(torch.bfloat16).to(dev)
+    return moe, x, grad_out, freq.tolist(), c
+
+
+def step(moe, x, grad_out):
+    for p in moe.parameters():
+        p.grad = None
+    x.grad = None
+    y, _ = moe(x)
+    y.backward(grad_out)
+
+
+def cpu_baseline(moe_gpu, bias_fn_freq, sample_tokens: int = 512):
+    """The torch CPU path (restated in oracle/moe_oracle.py) on `sample_tokens` tokens of the same layer."""
+    import torch
+    import torch.nn.functional as F
+
+    from oracle import moe_oracle as mo
+
+    oracle = mo.MoEOracle(E, TOP_K, H, I, mo.swiglu_packed_torch, True, False, 0.02).to(torch.bfloat16)
+    oracle.load_state_dict({k: v.cpu() for k, v in moe_gpu.state_dict().items()})
+    xs = torch.randn(sample_tokens, H, generator=torch.Generator().manual_seed(SEED)).to(torch.bfloat16).requires_grad_()
+    g = torch.randn(sample_tokens, H, generator=torch.Generator().manual_seed(SEED + 1)).to(torch.bfloat16)
+    warm = xs[:32].detach().clone().requires_grad_()
+    oracle(warm)[0].backward(g[:32])
+    for p in oracle.parameters():
+        p.grad = None
+    t0 = time.perf_counter()
+    y, _ = oracle(xs)
+    y.backward(g)
+    dt = time.perf_counter() - t0
+    flops = 18.0 * sample_tokens * TOP_K * H * I
+    return {
+        "value": flops / dt / 1e12,
+        "unit": "TFLOP/s",
+        "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"1 fwd+bwd of the same layer on T={sample_tokens} tokens (of {T}), bf16, unskewed router, {dt:.2f} s; "
+        f"os.cpu_count()={os.cpu_count()}",
+    }
+
+
+def secondary_hbm_kernels(dev):
+    """count+scatter GB/s: the HBM-bound kernels on their own, algorithmic bytes / event time."""
+    import torch
+
+    import cute_kernels
+    from cute_kernels import scattermoe
+
+    def timed(fn, iters=20):
+        for _ in range(3):
+            fn()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        s.record()
+        for _ in range(iters):
+            fn()
+        e.record()
+        torch.cuda.synchronize()
+        return s.elapsed_time(e) / iters * 1e-3
+
+    out = {}
+    g = torch.Generator().manual_seed(SEED)
+    for n in (1 << 16, 1 << 28):
+        ids = torch.randint(0, 64, (n,), generator=g, dtype=torch.int32).to(dev) if n <= (1 << 20) else torch.randint(0, 64, (n,), dtype=torch.int32, device=dev)
+        dt = timed(lambda: cute_kernels.continuous_count_and_offsets_cute(ids, 64))
+        b = 4 * n + 8 * 64 + 4 * 64
+        out[f"count_offsets_N{n}_E64"] = {"us": dt * 1e6, "GB/s": b / dt / 1e9, "frac_hbm": b / dt / 1e9 / PEAK_HBM_GBS}
+        del ids
+    # C2 routing bookkeeping: logits [16384, 64] bf16, top-2 -> ids, gates, sort, offsets
+    logits = torch.randn(16384, 64, generator=g).to(torch.bfloat16).to(dev)
+
+    def routing():
+        sel, gates, _ = cute_kernels.route_topk_softmax_raw(logits, 2)
+        cute_kernels.sort_by_expert(sel, 64)
+
+    dt = timed(routing)
+    b = 2 * 16384 * 64 + 4 * 4 * 32768 + 8 * 64
+    out["route_sort_C2"] = {"us": dt * 1e6, "GB/s": b / dt / 1e9, "frac_hbm": b / dt / 1e9 / PEAK_HBM_GBS}
+    # row gather / gated combine at the C3 shape
+    R = T * TOP_K
+    src = torch.randn(T, H, device=dev, dtype=torch.bfloat16)
+    idx = torch.randperm(R, device=dev).to(torch.int32)
+    dt = timed(lambda: cute_kernels.gather_rows(src, idx, None, TOP_K))
+    b = 2 * R * H * 2
+    out["gather_rows_C3"] = {"us": dt * 1e6, "GB/s": b / dt / 1e9, "frac_hbm": b / dt / 1e9 / PEAK_HBM_GBS}
+    expanded = torch.randn(R, H, device=dev, dtype=torch.bfloat16)
+    gates = torch.rand(T, TOP_K, device=dev, dtype=torch.bfloat16)
+    dt = timed(lambda: scattermoe._combine(expanded, gates, T, TOP_K, H))
+    b = R * H * 2 + T * H * 2 + 2 * R
+    out["combine_rows_C3"] = {"us": dt * 1e6, "GB/s": b / dt / 1e9, "frac_hbm": b / dt / 1e9 / PEAK_HBM_GBS}
+    return out
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--skip-cpu-baseline", action="store_true")
+    ap.add_argument("--skip-secondary", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build uses no second GPU (no collectives, no sharding); run with --gpus 1",
+              file=sys.stderr)
+        return 2
+
+    import torch
+
+    from cute_kernels import scattermoe
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    moe, x, grad_out, freq, zipf_c = build_layer(dev)
+    x.requires_grad_()
+
+    for _ in range(args.warmup):
+        step(moe, x, grad_out)
+    torch.cuda.synchronize()
+
+    timer = scattermoe.LaunchTimer()
+    scattermoe.launch_timer = timer
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step(moe, x, grad_out)
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / args.steps
+    scattermoe.launch_timer = None
+
+    R = T * TOP_K
+    flops_step = 18.0 * R * H * I
+    value = flops_step / dt / 1e12
+
+    # per-kernel launch durations from the events recorded inside the timed region
+    per_kernel: dict = {}
+    for name, dims, s, e in timer.records:
+        rec = per_kernel.setdefault(name, {"ms": 0.0, "launches": 0, "flops": 0.0})
+        rec["ms"] += s.elapsed_time(e)
+        rec["launches"] += 1
+        rec["flops"] += 2.0 * R * dims[0] * dims[1]  # 2*R*N*K (forward shapes) or 2*R*M*N (weight gradients)
+    dominant = max(per_kernel, key=lambda n: per_kernel[n]["ms"])
+    d = per_kernel[dominant]
+    achieved = d["flops"] / (d["ms"] * 1e-3) / 1e12
+    roofline = {
+        "bound": "mfma",
+        "kernel": dominant,
+        "achieved": achieved,
+        "peak": PEAK_BF16_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": achieved / PEAK_BF16_TFLOPS,
+        "traffic": None,
+        "avg_launch_ms": d["ms"] / d["launches"],
+        "flops_per_launch": d["flops"] / d["launches"],
+    }
+    kernels = {
+        n: {
+            "avg_launch_ms": r["ms"] / r["launches"],
+            "launches_per_step": r["launches"] / args.steps,
+            "TFLOP/s": r["flops"] / (r["ms"] * 1e-3) / 1e12,
+            "frac_mfma": r["flops"] / (r["ms"] * 1e-3) / 1e12 / PEAK_BF16_TFLOPS,
+        }
+        for n, r in per_kernel.items()
+    }
+    gemm_ms_per_step = sum(r["ms"] for r in per_kernel.values()) / args.steps
+
+    line = {
+        "metric": "MoE fwd+bwd TFLOP/s",
+        "value": value,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": dt * 1e3,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": "C3 Mixtral-shape MoE layer fwd+bwd: T=16384 H=4096 E=8 top-2 I=14336 SwiGLU, Zipf(1.0) load",
+            "routed_rows": R,
+            "flops_per_step": flops_step,
+            "expert_load": [round(f, 4) for f in freq],
+            "zipf_bias_scale": zipf_c,
+        },
+        "frac_mfma_peak": value / PEAK_BF16_TFLOPS,
+        "gemm_ms_per_step": gemm_ms_per_step,
+        "roofline": roofline,
+        "kernels": kernels,
+    }
+    if not args.skip_secondary:
+        del moe, x, grad_out
+        torch.cuda.empty_cache()
+        line["count_scatter"] = secondary_hbm_kernels(dev)
+        moe = None
+    if not args.skip_cpu_baseline:
+        if moe is None:
+            moe = build_layer(dev)[0]
+        line["cpu_baseline"] = cpu_baseline(moe, None)
+    else:
+        line["cpu_baseline"] = None
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -94,6 +94,19 @@ __device__ inline void store4(T* p, T v0, T v1, T v2, T v3) {
   *reinterpret_cast<uint2*>(p) = u;
 }
 
+// Tile order inside a run of tiles: groups of 8 along `a` (the side with a_count tiles), then `b`, with `a` fastest
+// inside a group -- 32 consecutive tiles form an 8 x 4 block that shares 8 + 4 operand panels.
+__device__ inline void grouped_order(int r, int a_count, int b_count, int& a, int& b) {
+  constexpr int GROUP = 8;
+  const int group_sz = GROUP * b_count;
+  const int g = r / group_sz;
+  const int first = g * GROUP;
+  const int in_group = min(GROUP, a_count - first);
+  const int q = r - g * group_sz;
+  b = q / in_group;
+  a = first + (q - b * in_group);
+}
+
 template <typename T, int BM, int BN, int MODE>
 __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams prm) {
   constexpr int WM = BM / 2, WN = BN / 2;    // wave tile
@@ -111,15 +124,24 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
   int64_t k_begin = 0;
   int k_len;
   if constexpr (MODE == kDw) {
+    // Experts differ in contraction length (their row counts), so every XCD gets a slice of EVERY expert's tile grid:
+    // the grid is cut in 8 along its longer side, and a slice is walked in groups of 8 tiles along that side.
     const int per_expert = prm.m_tiles * prm.n_tiles;
-    const int total = per_expert * prm.num_experts;
-    int pid = blockIdx.x;
-    if (total % kXcds == 0) pid = (pid % kXcds) * (total / kXcds) + pid / kXcds;
-    expert = pid / per_expert;
-    const int r = pid - expert * per_expert;
-    // N-tile fastest: consecutive blocks share the a_t panel
-    mt = r / prm.n_tiles;
-    nt = r - mt * prm.n_tiles;
+    const bool m_major = prm.m_tiles >= prm.n_tiles;
+    const int major = m_major ? prm.m_tiles : prm.n_tiles, minor = m_major ? prm.n_tiles : prm.m_tiles;
+    int pid = blockIdx.x, a, b;  // a: index along the major side, b: along the minor side
+    if (major % kXcds == 0) {
+      const int xcd = pid % kXcds, j = pid / kXcds;
+      const int slice = major / kXcds, per_slice = slice * minor;
+      expert = j / per_slice;
+      grouped_order(j - expert * per_slice, slice, minor, a, b);
+      a += xcd * slice;
+    } else {
+      expert = pid / per_expert;
+      grouped_order(pid - expert * per_expert, major, minor, a, b);
+    }
+    mt = m_major ? a : b;
+    nt = m_major ? b : a;
     k_begin = prm.seg_starts[expert];
     k_len = (int)((prm.counts[expert] + BK - 1) / BK * BK);
   } else {
@@ -129,15 +151,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     if (pid >= total) return;
     const int per_xcd = total / kXcds;
     if (pid < per_xcd * kXcds) pid = (pid % kXcds) * per_xcd + pid / kXcds;  // the ragged end keeps its order
-    // groups of 8 M-tiles, N-tile next, M-tile within the group fastest: a group reuses one W panel 8 times
-    constexpr int GROUP = 8;
-    const int group_sz = GROUP * prm.n_tiles;
-    const int g = pid / group_sz;
-    const int first_m = g * GROUP;
-    const int rows_in_group = min(GROUP, live_m - first_m);
-    const int r = pid - g * group_sz;
-    nt = r / rows_in_group;
-    mt = first_m + (r - nt * rows_in_group);
+    grouped_order(pid, live_m, prm.n_tiles, mt, nt);
     expert = prm.tile_expert[mt];
     k_len = prm.K;
   }
@@ -146,20 +160,22 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
   // ---- per-thread global chunk addresses, as 32-bit offsets in 16-byte chunks from the operand base
   const int cc = tid & (kChunksPerRow - 1);  // chunk within the 64-element K slab
   const int lr = tid >> 3;                   // row within a group of 32
-  const vec16* a_base = static_cast<const vec16*>(prm.a);
-  const vec16* b_base = static_cast<const vec16*>(prm.w);
+  // 32-bit byte offsets from a wave-uniform base: the loads use scalar-base + vector-offset addressing, and stepping
+  // along K only moves the scalar base
+  const char* a_base = static_cast<const char*>(prm.a);
+  const char* b_base = static_cast<const char*>(prm.w);
   uint32_t a_chunk[A_CH], b_chunk[B_CH];
   int64_t valid_end = 0;  // forward modes: first pad row of this expert's segment
   if constexpr (MODE == kDw) {
 #pragma unroll
     for (int i = 0; i < A_CH; ++i) {
       const int64_t row = min(m0 + lr + 32 * i, (int64_t)prm.M - 1);
-      a_chunk[i] = (uint32_t)((row * prm.lda + k_begin) / 8 + cc);
+      a_chunk[i] = (uint32_t)((row * prm.lda + k_begin) * 2 + cc * 16);
     }
 #pragma unroll
     for (int i = 0; i < B_CH; ++i) {
       const int64_t row = min((int64_t)nt * BN + lr + 32 * i, (int64_t)prm.N - 1);
-      b_chunk[i] = (uint32_t)((row * prm.ldw + k_begin) / 8 + cc);
+      b_chunk[i] = (uint32_t)((row * prm.ldw + k_begin) * 2 + cc * 16);
     }
   } else {
     valid_end = (int64_t)prm.seg_starts[expert] + prm.counts[expert];
@@ -168,9 +184,9 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
       int64_t p = m0 + lr + 32 * i;
       if (p >= valid_end) p = valid_end - 1;  // pad rows re-read a valid row; their results are never stored
       const int64_t row = prm.a_gather_div > 0 ? (int64_t)(prm.row_slot[p] / prm.a_gather_div) : p;
-      a_chunk[i] = (uint32_t)(row * prm.lda / 8 + cc);
+      a_chunk[i] = (uint32_t)(row * prm.lda * 2 + cc * 16);
     }
-    const int64_t w_off = (int64_t)expert * prm.w_expert_stride;
+    b_base += (int64_t)expert * prm.w_expert_stride * 2;
 #pragma unroll
     for (int i = 0; i < B_CH; ++i) {
       const int j = lr + 32 * i;  // row of the LDS B tile
@@ -184,7 +200,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
       } else {
         n = min((int64_t)nt * BN + j, (int64_t)prm.N - 1);
       }
-      b_chunk[i] = (uint32_t)((w_off + n * prm.ldw) / 8 + cc);
+      b_chunk[i] = (uint32_t)(n * prm.ldw * 2 + cc * 16);
     }
   }
 
@@ -197,14 +213,25 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   // ---- main loop
+  // Per K step of 64: the global loads of step k+1 are issued first and stay in flight; the 64 MFMAs of step k run
+  // with the LDS fragment reads of the next 16-wide slice interleaved between them (double-buffered fragments); the
+  // LDS stores of step k+1 are interleaved with the MFMAs of the last slice; one barrier closes the step.
   vec16 ra[A_CH], rb[B_CH];
-  auto load_global = [&](int kt) {
-    const int k = kt * BK + cc * 8;
-    const bool ok = k < k_len;  // K % 8 == 0, so a chunk is entirely inside or outside
+  auto load_global = [&](int kt, auto full) {
+    const char* ak = a_base + (int64_t)kt * (BK * 2);
+    const char* bk = b_base + (int64_t)kt * (BK * 2);
+    if constexpr (decltype(full)::value) {
 #pragma unroll
-    for (int i = 0; i < A_CH; ++i) ra[i] = ok ? a_base[a_chunk[i] + (uint32_t)kt * (BK / 8)] : zero16();
+      for (int i = 0; i < A_CH; ++i) ra[i] = load16(ak + a_chunk[i]);
 #pragma unroll
-    for (int i = 0; i < B_CH; ++i) rb[i] = ok ? b_base[b_chunk[i] + (uint32_t)kt * (BK / 8)] : zero16();
+      for (int i = 0; i < B_CH; ++i) rb[i] = load16(bk + b_chunk[i]);
+    } else {
+      const bool ok = kt * BK + cc * 8 < k_len;  // K % 8 == 0, so a chunk is entirely inside or outside
+#pragma unroll
+      for (int i = 0; i < A_CH; ++i) ra[i] = ok ? load16(ak + a_chunk[i]) : zero16();
+#pragma unroll
+      for (int i = 0; i < B_CH; ++i) rb[i] = ok ? load16(bk + b_chunk[i]) : zero16();
+    }
   };
   auto store_lds = [&](int stage) {
     T* sa = lds + stage * kStageElems;
@@ -215,35 +242,80 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     for (int i = 0; i < B_CH; ++i) store16(sb + (lr + 32 * i) * kLdsStride + cc * 8, rb[i]);
   };
   typedef typename Mfma<T>::frag frag_t;
-  auto compute = [&](int stage) {
-    const T* sa = lds + stage * kStageElems + (wm * WM + (lane & 31)) * kLdsStride + (lane >> 5) * 8;
-    const T* sb = lds + stage * kStageElems + BM * kLdsStride + (wn * WN + (lane & 31)) * kLdsStride + (lane >> 5) * 8;
+  const int frag_a_off = (wm * WM + (lane & 31)) * kLdsStride + (lane >> 5) * 8;
+  const int frag_b_off = BM * kLdsStride + (wn * WN + (lane & 31)) * kLdsStride + (lane >> 5) * 8;
+  constexpr int KK = BK / 16;  // 16-wide slices per K step; even, so slice 0 always lands in fragment buffer 0
+  frag_t fa[2][MI], fb[2][NI];
+  auto read_frags = [&](int stage, int kk, int buf) {
+    const T* sa = lds + stage * kStageElems + frag_a_off + kk * 16;
+    const T* sb = lds + stage * kStageElems + frag_b_off + kk * 16;
 #pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      frag_t fa[MI], fb[NI];
+    for (int i = 0; i < MI; ++i) fa[buf][i] = *reinterpret_cast<const frag_t*>(sa + i * 32 * kLdsStride);
 #pragma unroll
-      for (int i = 0; i < MI; ++i) fa[i] = *reinterpret_cast<const frag_t*>(sa + i * 32 * kLdsStride + kk * 16);
+    for (int j = 0; j < NI; ++j) fb[buf][j] = *reinterpret_cast<const frag_t*>(sb + j * 32 * kLdsStride);
+  };
+  // MFMAs [first, last) of one slice, row-major over the wave's MI x NI blocks
+  auto mfma_range = [&](int buf, int first, int last) {
 #pragma unroll
-      for (int j = 0; j < NI; ++j) fb[j] = *reinterpret_cast<const frag_t*>(sb + j * 32 * kLdsStride + kk * 16);
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
-      for (int i = 0; i < MI; ++i)
+      for (int j = 0; j < NI; ++j)
+        if (i * NI + j >= first && i * NI + j < last) acc[i][j] = Mfma<T>::run(fa[buf][i], fb[buf][j], acc[i][j]);
+  };
+  constexpr int kMfmaPerSlice = MI * NI, kReadsPerSlice = MI + NI, kWritesPerStep = A_CH + B_CH;
+  // One K step out of LDS stage `stage`, whose slice-0 fragments are already in buffer 0.
+  // HAS_NEXT: also prefetch step kt + 1 from global memory (FULL: all of its 64 columns exist), store it into the other
+  // LDS stage and fetch its slice-0 fragments.
+  auto k_step = [&](int stage, int kt, auto has_next, auto full) {
+    constexpr bool HAS_NEXT = decltype(has_next)::value;
+    if constexpr (HAS_NEXT) load_global(kt + 1, full);
 #pragma unroll
-        for (int j = 0; j < NI; ++j) acc[i][j] = Mfma<T>::run(fa[i], fb[j], acc[i][j]);
+    for (int kk = 0; kk + 1 < KK; ++kk) {
+      read_frags(stage, kk + 1, (kk + 1) & 1);
+      mfma_range(kk & 1, 0, kMfmaPerSlice);
+#pragma unroll
+      for (int g = 0; g < kReadsPerSlice; ++g) {  // pin the interleave: 1 global load, 1 LDS read, a share of the MFMAs
+        if constexpr (HAS_NEXT) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerSlice / kReadsPerSlice, 0);
+      }
+    }
+    constexpr int last = (KK - 1) & 1;
+    if constexpr (HAS_NEXT) {
+      // last slice: its first half hides the LDS stores of the next step, the barrier, then its second half hides the
+      // first fragment reads of the next step
+      store_lds(stage ^ 1);
+      mfma_range(last, 0, kMfmaPerSlice / 2);
+#pragma unroll
+      for (int g = 0; g < kMfmaPerSlice / 2; ++g) {
+        __builtin_amdgcn_sched_group_barrier(0x200, (kWritesPerStep + kMfmaPerSlice / 2 - 1) / (kMfmaPerSlice / 2), 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      }
+      __syncthreads();
+      read_frags(stage ^ 1, 0, 0);
+      mfma_range(last, kMfmaPerSlice / 2, kMfmaPerSlice);
+#pragma unroll
+      for (int g = 0; g < kMfmaPerSlice / 2; ++g) {
+        __builtin_amdgcn_sched_group_barrier(0x100, (kReadsPerSlice + kMfmaPerSlice / 2 - 1) / (kMfmaPerSlice / 2), 0);
+        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+      }
+    } else {
+      mfma_range(last, 0, kMfmaPerSlice);
     }
   };
 
   const int nk = (k_len + BK - 1) / BK;
+  const int nk_full = k_len / BK;  // steps whose 64 columns all exist
   if (nk > 0) {
-    load_global(0);
+    if (nk_full > 0) load_global(0, std::true_type{});
+    else load_global(0, std::false_type{});
     store_lds(0);
     __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
-      const bool more = kt + 1 < nk;
-      if (more) load_global(kt + 1);
-      compute(kt & 1);
-      if (more) store_lds((kt + 1) & 1);
-      __syncthreads();
-    }
+    read_frags(0, 0, 0);
+    int kt = 0;
+    for (; kt + 1 < nk_full; ++kt) k_step(kt & 1, kt, std::true_type{}, std::true_type{});
+    for (; kt + 1 < nk; ++kt) k_step(kt & 1, kt, std::true_type{}, std::false_type{});  // ragged last columns
+    k_step((nk - 1) & 1, nk - 1, std::false_type{}, std::false_type{});
   }
 
   // ---- epilogue. Lane holds, per 32x32 block and q in 0..3, rows 8q + 4*(lane/32) + 0..3 of column lane%32.
@@ -419,8 +491,10 @@ extern "C" int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* 
              "%s: y_t needs ld_t >= max_rows, ld_t %% 8 == 0 and 8-byte alignment", name);
   CK_REQUIRE(epilogue != CK_EPI_SCATTER || y_t == nullptr, "%s: the scatter epilogue has no transposed output", name);
 
-  // operands are addressed with 32-bit offsets in 16-byte chunks
-  CK_REQUIRE((int64_t)seg->num_experts * N * K / 8 < (int64_t)0xffffffff, "%s: w is too large", name);
+  // rows are addressed with 32-bit byte offsets: from the operand base for a, from the expert's slice for w
+  CK_REQUIRE((int64_t)N * K * 2 < ((int64_t)1 << 32), "%s: one expert's weight matrix must stay below 4 GiB", name);
+  CK_REQUIRE(a_gather_div > 0 || seg->max_rows * (int64_t)K * 2 < ((int64_t)1 << 32),
+             "%s: the grouped input must stay below 4 GiB", name);
   GemmParams prm = {};
   prm.a = a;
   prm.w = w;
@@ -480,8 +554,8 @@ extern "C" int ck_grouped_gemm_dw(const void* a_t, const void* b_t, int64_t ld_t
   CK_REQUIRE(a_t && b_t && dw, "%s: NULL argument", name);
   CK_REQUIRE(ld_t >= seg->max_rows && ld_t % 8 == 0 && aligned16(a_t) && aligned16(b_t),
              "%s: operands need ld_t >= max_rows, ld_t %% 8 == 0 and 16-byte alignment", name);
-  CK_REQUIRE((int64_t)M * ld_t / 8 < (int64_t)0xffffffff && (int64_t)N * ld_t / 8 < (int64_t)0xffffffff,
-             "%s: operands are too large", name);
+  CK_REQUIRE((int64_t)M * ld_t * 2 < ((int64_t)1 << 32) && (int64_t)N * ld_t * 2 < ((int64_t)1 << 32),
+             "%s: each transposed operand must stay below 4 GiB", name);
   GemmParams prm = {};
   prm.a = a_t;
   prm.w = b_t;

@@ -170,27 +170,67 @@ def sort_by_expert(expert_ids: torch.Tensor, num_experts: int, align: int | None
 # ---------------------------------------------------------------------------------------------------------------
 # thin launch helpers (allocate outputs, pass pointers)
 # ---------------------------------------------------------------------------------------------------------------
+class LaunchTimer:
+    """Optional per-launch timing of the grouped GEMMs with events on the launch stream (used by bench.py).
+    records: list of (kernel name, [N, K] or [M, N] of the launch, start event, end event)."""
+
+    def __init__(self) -> None:
+        self.records: list = []
+
+    def time(self, name: str, dims: tuple, fn) -> None:
+        start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        start.record()
+        fn()
+        end.record()
+        self.records.append((name, dims, start, end))
+
+
+launch_timer: LaunchTimer | None = None
+
+_EPILOGUE_NAMES = {
+    _C.CK_EPI_GROUPED: "grouped_gemm<grouped>",
+    _C.CK_EPI_SCATTER: "grouped_gemm<scatter>",
+    _C.CK_EPI_SWIGLU: "grouped_gemm<swiglu>",
+    _C.CK_EPI_SWIGLU_BWD: "grouped_gemm<swiglu_bwd>",
+}
+
+
 def _gemm(a, gather_div, w, seg: ExpertSegments, epilogue, y, y_t=None, aux=None, aux_in=None):
     E, N, K = w.shape
     cs = seg.c_struct()
-    with torch.cuda.device(w.device):
-        _C.check(
-            _C.lib().ck_grouped_gemm(
-                _C.ptr(a), gather_div, _C.ptr(w), N, K, ctypes.byref(cs), epilogue, _C.ptr(y), _C.ptr(y_t), seg.ld_t,
-                _C.ptr(aux), _C.ptr(aux_in), _C.dtype_code(w.dtype), _C.stream(),
+
+    def launch():
+        with torch.cuda.device(w.device):
+            _C.check(
+                _C.lib().ck_grouped_gemm(
+                    _C.ptr(a), gather_div, _C.ptr(w), N, K, ctypes.byref(cs), epilogue, _C.ptr(y), _C.ptr(y_t), seg.ld_t,
+                    _C.ptr(aux), _C.ptr(aux_in), _C.dtype_code(w.dtype), _C.stream(),
+                )
             )
-        )
+
+    if launch_timer is None:
+        launch()
+    else:
+        launch_timer.time(_EPILOGUE_NAMES[epilogue], (N, K), launch)
 
 
 def _gemm_dw(a_t, b_t, seg: ExpertSegments, dw):
     E, M, N = dw.shape
     cs = seg.c_struct()
-    with torch.cuda.device(dw.device):
-        _C.check(
-            _C.lib().ck_grouped_gemm_dw(
-                _C.ptr(a_t), _C.ptr(b_t), seg.ld_t, M, N, ctypes.byref(cs), _C.ptr(dw), _C.dtype_code(dw.dtype), _C.stream()
+
+    def launch():
+        with torch.cuda.device(dw.device):
+            _C.check(
+                _C.lib().ck_grouped_gemm_dw(
+                    _C.ptr(a_t), _C.ptr(b_t), seg.ld_t, M, N, ctypes.byref(cs), _C.ptr(dw), _C.dtype_code(dw.dtype),
+                    _C.stream(),
+                )
             )
-        )
+
+    if launch_timer is None:
+        launch()
+    else:
+        launch_timer.time("grouped_gemm<dw>", (M, N), launch)
 
 
 def _group_rows(src, coeff, fan_out, seg: ExpertSegments, want_grouped: bool, want_transposed: bool):
