@@ -40,6 +40,12 @@ struct Mfma<f16_t> {
   }
 };
 
+#ifndef CK_ABLATE
+#define CK_ABLATE 0  // measurement builds only: 1 no barrier, 2 no loads in the loop, 4 no fragment reads, 8 no load wait
+#endif
+
+bool g_force_pipe0 = false;  // set from the environment (CK_GEMM_PIPE=0) for A/B measurements
+
 struct GemmParams {
   const void* a;      // forward modes: [*, K]; dW: a_t [M, ld_t]
   const void* w;      // forward modes: [E, N, K]; dW: b_t [N, ld_t]
@@ -107,7 +113,10 @@ __device__ inline void grouped_order(int r, int a_count, int b_count, int& a, in
   a = first + (q - b * in_group);
 }
 
-template <typename T, int BM, int BN, int MODE>
+// PIPE 0: K step 64, global -> registers -> padded LDS, two stages (any K % 8 == 0).
+// PIPE 1: K step 32, global -> LDS directly (no register staging), four XOR-swizzled stages, loads three steps ahead
+//         (needs K % 32 == 0).
+template <typename T, int BM, int BN, int MODE, int PIPE>
 __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams prm) {
   constexpr int WM = BM / 2, WN = BN / 2;    // wave tile
   constexpr int MI = WM / 32, NI = WN / 32;  // 32x32 blocks per wave tile
@@ -157,52 +166,8 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
   }
   const int64_t m0 = (int64_t)mt * BM;
 
-  // ---- per-thread global chunk addresses, as 32-bit offsets in 16-byte chunks from the operand base
-  const int cc = tid & (kChunksPerRow - 1);  // chunk within the 64-element K slab
-  const int lr = tid >> 3;                   // row within a group of 32
-  // 32-bit byte offsets from a wave-uniform base: the loads use scalar-base + vector-offset addressing, and stepping
-  // along K only moves the scalar base
-  const char* a_base = static_cast<const char*>(prm.a);
-  const char* b_base = static_cast<const char*>(prm.w);
-  uint32_t a_chunk[A_CH], b_chunk[B_CH];
   int64_t valid_end = 0;  // forward modes: first pad row of this expert's segment
-  if constexpr (MODE == kDw) {
-#pragma unroll
-    for (int i = 0; i < A_CH; ++i) {
-      const int64_t row = min(m0 + lr + 32 * i, (int64_t)prm.M - 1);
-      a_chunk[i] = (uint32_t)((row * prm.lda + k_begin) * 2 + cc * 16);
-    }
-#pragma unroll
-    for (int i = 0; i < B_CH; ++i) {
-      const int64_t row = min((int64_t)nt * BN + lr + 32 * i, (int64_t)prm.N - 1);
-      b_chunk[i] = (uint32_t)((row * prm.ldw + k_begin) * 2 + cc * 16);
-    }
-  } else {
-    valid_end = (int64_t)prm.seg_starts[expert] + prm.counts[expert];
-#pragma unroll
-    for (int i = 0; i < A_CH; ++i) {
-      int64_t p = m0 + lr + 32 * i;
-      if (p >= valid_end) p = valid_end - 1;  // pad rows re-read a valid row; their results are never stored
-      const int64_t row = prm.a_gather_div > 0 ? (int64_t)(prm.row_slot[p] / prm.a_gather_div) : p;
-      a_chunk[i] = (uint32_t)(row * prm.lda * 2 + cc * 16);
-    }
-    b_base += (int64_t)expert * prm.w_expert_stride * 2;
-#pragma unroll
-    for (int i = 0; i < B_CH; ++i) {
-      const int j = lr + 32 * i;  // row of the LDS B tile
-      int64_t n;
-      if constexpr (MODE == kSwiglu) {
-        // LDS rows [wave column][up half | gate half]: the same lane ends up holding up and gate of one column
-        const int half = (j % WN) / (WN / 2);
-        const int within = (j / WN) * (WN / 2) + (j % (WN / 2));
-        const int64_t col = min((int64_t)nt * (BN / 2) + within, (int64_t)prm.I - 1);
-        n = (int64_t)half * prm.I + col;
-      } else {
-        n = min((int64_t)nt * BN + j, (int64_t)prm.N - 1);
-      }
-      b_chunk[i] = (uint32_t)(n * prm.ldw * 2 + cc * 16);
-    }
-  }
+  if constexpr (MODE != kDw) valid_end = (int64_t)prm.seg_starts[expert] + prm.counts[expert];
 
   f32x16 acc[MI][NI];
 #pragma unroll
@@ -212,110 +177,290 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // ---- main loop
-  // Per K step of 64: the global loads of step k+1 are issued first and stay in flight; the 64 MFMAs of step k run
-  // with the LDS fragment reads of the next 16-wide slice interleaved between them (double-buffered fragments); the
-  // LDS stores of step k+1 are interleaved with the MFMAs of the last slice; one barrier closes the step.
-  vec16 ra[A_CH], rb[B_CH];
-  auto load_global = [&](int kt, auto full) {
-    const char* ak = a_base + (int64_t)kt * (BK * 2);
-    const char* bk = b_base + (int64_t)kt * (BK * 2);
-    if constexpr (decltype(full)::value) {
-#pragma unroll
-      for (int i = 0; i < A_CH; ++i) ra[i] = load16(ak + a_chunk[i]);
-#pragma unroll
-      for (int i = 0; i < B_CH; ++i) rb[i] = load16(bk + b_chunk[i]);
-    } else {
-      const bool ok = kt * BK + cc * 8 < k_len;  // K % 8 == 0, so a chunk is entirely inside or outside
-#pragma unroll
-      for (int i = 0; i < A_CH; ++i) ra[i] = ok ? load16(ak + a_chunk[i]) : zero16();
-#pragma unroll
-      for (int i = 0; i < B_CH; ++i) rb[i] = ok ? load16(bk + b_chunk[i]) : zero16();
-    }
-  };
-  auto store_lds = [&](int stage) {
-    T* sa = lds + stage * kStageElems;
-    T* sb = sa + BM * kLdsStride;
-#pragma unroll
-    for (int i = 0; i < A_CH; ++i) store16(sa + (lr + 32 * i) * kLdsStride + cc * 8, ra[i]);
-#pragma unroll
-    for (int i = 0; i < B_CH; ++i) store16(sb + (lr + 32 * i) * kLdsStride + cc * 8, rb[i]);
-  };
-  typedef typename Mfma<T>::frag frag_t;
-  const int frag_a_off = (wm * WM + (lane & 31)) * kLdsStride + (lane >> 5) * 8;
-  const int frag_b_off = BM * kLdsStride + (wn * WN + (lane & 31)) * kLdsStride + (lane >> 5) * 8;
-  constexpr int KK = BK / 16;  // 16-wide slices per K step; even, so slice 0 always lands in fragment buffer 0
-  frag_t fa[2][MI], fb[2][NI];
-  auto read_frags = [&](int stage, int kk, int buf) {
-    const T* sa = lds + stage * kStageElems + frag_a_off + kk * 16;
-    const T* sb = lds + stage * kStageElems + frag_b_off + kk * 16;
-#pragma unroll
-    for (int i = 0; i < MI; ++i) fa[buf][i] = *reinterpret_cast<const frag_t*>(sa + i * 32 * kLdsStride);
-#pragma unroll
-    for (int j = 0; j < NI; ++j) fb[buf][j] = *reinterpret_cast<const frag_t*>(sb + j * 32 * kLdsStride);
-  };
-  // MFMAs [first, last) of one slice, row-major over the wave's MI x NI blocks
-  auto mfma_range = [&](int buf, int first, int last) {
-#pragma unroll
-    for (int i = 0; i < MI; ++i)
-#pragma unroll
-      for (int j = 0; j < NI; ++j)
-        if (i * NI + j >= first && i * NI + j < last) acc[i][j] = Mfma<T>::run(fa[buf][i], fb[buf][j], acc[i][j]);
-  };
-  constexpr int kMfmaPerSlice = MI * NI, kReadsPerSlice = MI + NI, kWritesPerStep = A_CH + B_CH;
-  // One K step out of LDS stage `stage`, whose slice-0 fragments are already in buffer 0.
-  // HAS_NEXT: also prefetch step kt + 1 from global memory (FULL: all of its 64 columns exist), store it into the other
-  // LDS stage and fetch its slice-0 fragments.
-  auto k_step = [&](int stage, int kt, auto has_next, auto full) {
-    constexpr bool HAS_NEXT = decltype(has_next)::value;
-    if constexpr (HAS_NEXT) load_global(kt + 1, full);
-#pragma unroll
-    for (int kk = 0; kk + 1 < KK; ++kk) {
-      read_frags(stage, kk + 1, (kk + 1) & 1);
-      mfma_range(kk & 1, 0, kMfmaPerSlice);
-#pragma unroll
-      for (int g = 0; g < kReadsPerSlice; ++g) {  // pin the interleave: 1 global load, 1 LDS read, a share of the MFMAs
-        if constexpr (HAS_NEXT) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerSlice / kReadsPerSlice, 0);
+  if constexpr (PIPE == 0) {
+    // ---- per-thread global chunk addresses, as 32-bit offsets in 16-byte chunks from the operand base
+    const int cc = tid & (kChunksPerRow - 1);  // chunk within the 64-element K slab
+    const int lr = tid >> 3;                   // row within a group of 32
+    // 32-bit byte offsets from a wave-uniform base: the loads use scalar-base + vector-offset addressing, and stepping
+    // along K only moves the scalar base
+    const char* a_base = static_cast<const char*>(prm.a);
+    const char* b_base = static_cast<const char*>(prm.w);
+    uint32_t a_chunk[A_CH], b_chunk[B_CH];
+    if constexpr (MODE == kDw) {
+  #pragma unroll
+      for (int i = 0; i < A_CH; ++i) {
+        const int64_t row = min(m0 + lr + 32 * i, (int64_t)prm.M - 1);
+        a_chunk[i] = (uint32_t)((row * prm.lda + k_begin) * 2 + cc * 16);
       }
-    }
-    constexpr int last = (KK - 1) & 1;
-    if constexpr (HAS_NEXT) {
-      // last slice: its first half hides the LDS stores of the next step, the barrier, then its second half hides the
-      // first fragment reads of the next step
-      store_lds(stage ^ 1);
-      mfma_range(last, 0, kMfmaPerSlice / 2);
-#pragma unroll
-      for (int g = 0; g < kMfmaPerSlice / 2; ++g) {
-        __builtin_amdgcn_sched_group_barrier(0x200, (kWritesPerStep + kMfmaPerSlice / 2 - 1) / (kMfmaPerSlice / 2), 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-      }
-      __syncthreads();
-      read_frags(stage ^ 1, 0, 0);
-      mfma_range(last, kMfmaPerSlice / 2, kMfmaPerSlice);
-#pragma unroll
-      for (int g = 0; g < kMfmaPerSlice / 2; ++g) {
-        __builtin_amdgcn_sched_group_barrier(0x100, (kReadsPerSlice + kMfmaPerSlice / 2 - 1) / (kMfmaPerSlice / 2), 0);
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+  #pragma unroll
+      for (int i = 0; i < B_CH; ++i) {
+        const int64_t row = min((int64_t)nt * BN + lr + 32 * i, (int64_t)prm.N - 1);
+        b_chunk[i] = (uint32_t)((row * prm.ldw + k_begin) * 2 + cc * 16);
       }
     } else {
-      mfma_range(last, 0, kMfmaPerSlice);
+  #pragma unroll
+      for (int i = 0; i < A_CH; ++i) {
+        int64_t p = m0 + lr + 32 * i;
+        if (p >= valid_end) p = valid_end - 1;  // pad rows re-read a valid row; their results are never stored
+        const int64_t row = prm.a_gather_div > 0 ? (int64_t)(prm.row_slot[p] / prm.a_gather_div) : p;
+        a_chunk[i] = (uint32_t)(row * prm.lda * 2 + cc * 16);
+      }
+      b_base += (int64_t)expert * prm.w_expert_stride * 2;
+  #pragma unroll
+      for (int i = 0; i < B_CH; ++i) {
+        const int j = lr + 32 * i;  // row of the LDS B tile
+        int64_t n;
+        if constexpr (MODE == kSwiglu) {
+          // LDS rows [wave column][up half | gate half]: the same lane ends up holding up and gate of one column
+          const int half = (j % WN) / (WN / 2);
+          const int within = (j / WN) * (WN / 2) + (j % (WN / 2));
+          const int64_t col = min((int64_t)nt * (BN / 2) + within, (int64_t)prm.I - 1);
+          n = (int64_t)half * prm.I + col;
+        } else {
+          n = min((int64_t)nt * BN + j, (int64_t)prm.N - 1);
+        }
+        b_chunk[i] = (uint32_t)(n * prm.ldw * 2 + cc * 16);
+      }
     }
-  };
 
-  const int nk = (k_len + BK - 1) / BK;
-  const int nk_full = k_len / BK;  // steps whose 64 columns all exist
-  if (nk > 0) {
-    if (nk_full > 0) load_global(0, std::true_type{});
-    else load_global(0, std::false_type{});
-    store_lds(0);
-    __syncthreads();
-    read_frags(0, 0, 0);
-    int kt = 0;
-    for (; kt + 1 < nk_full; ++kt) k_step(kt & 1, kt, std::true_type{}, std::true_type{});
-    for (; kt + 1 < nk; ++kt) k_step(kt & 1, kt, std::true_type{}, std::false_type{});  // ragged last columns
-    k_step((nk - 1) & 1, nk - 1, std::false_type{}, std::false_type{});
+    // ---- main loop
+    // Per K step of 64: the global loads of step k+1 are issued first and stay in flight; the 64 MFMAs of step k run
+    // with the LDS fragment reads of the next 16-wide slice interleaved between them (double-buffered fragments); the
+    // LDS stores of step k+1 are interleaved with the MFMAs of the last slice; one barrier closes the step.
+    vec16 ra[A_CH], rb[B_CH];
+    auto load_global = [&](int kt, auto full) {
+      const char* ak = a_base + (int64_t)kt * (BK * 2);
+      const char* bk = b_base + (int64_t)kt * (BK * 2);
+      if constexpr (decltype(full)::value) {
+  #pragma unroll
+        for (int i = 0; i < A_CH; ++i) ra[i] = load16(ak + a_chunk[i]);
+  #pragma unroll
+        for (int i = 0; i < B_CH; ++i) rb[i] = load16(bk + b_chunk[i]);
+      } else {
+        const bool ok = kt * BK + cc * 8 < k_len;  // K % 8 == 0, so a chunk is entirely inside or outside
+  #pragma unroll
+        for (int i = 0; i < A_CH; ++i) ra[i] = ok ? load16(ak + a_chunk[i]) : zero16();
+  #pragma unroll
+        for (int i = 0; i < B_CH; ++i) rb[i] = ok ? load16(bk + b_chunk[i]) : zero16();
+      }
+    };
+    auto store_lds = [&](int stage) {
+      T* sa = lds + stage * kStageElems;
+      T* sb = sa + BM * kLdsStride;
+  #pragma unroll
+      for (int i = 0; i < A_CH; ++i) store16(sa + (lr + 32 * i) * kLdsStride + cc * 8, ra[i]);
+  #pragma unroll
+      for (int i = 0; i < B_CH; ++i) store16(sb + (lr + 32 * i) * kLdsStride + cc * 8, rb[i]);
+    };
+    typedef typename Mfma<T>::frag frag_t;
+    const int frag_a_off = (wm * WM + (lane & 31)) * kLdsStride + (lane >> 5) * 8;
+    const int frag_b_off = BM * kLdsStride + (wn * WN + (lane & 31)) * kLdsStride + (lane >> 5) * 8;
+    constexpr int KK = BK / 16;  // 16-wide slices per K step; even, so slice 0 always lands in fragment buffer 0
+    frag_t fa[2][MI], fb[2][NI];
+    auto read_frags = [&](int stage, int kk, int buf) {
+      const T* sa = lds + stage * kStageElems + frag_a_off + kk * 16;
+      const T* sb = lds + stage * kStageElems + frag_b_off + kk * 16;
+  #pragma unroll
+      for (int i = 0; i < MI; ++i) fa[buf][i] = *reinterpret_cast<const frag_t*>(sa + i * 32 * kLdsStride);
+  #pragma unroll
+      for (int j = 0; j < NI; ++j) fb[buf][j] = *reinterpret_cast<const frag_t*>(sb + j * 32 * kLdsStride);
+    };
+    // MFMAs [first, last) of one slice, row-major over the wave's MI x NI blocks
+    auto mfma_range = [&](int buf, int first, int last) {
+  #pragma unroll
+      for (int i = 0; i < MI; ++i)
+  #pragma unroll
+        for (int j = 0; j < NI; ++j)
+          if (i * NI + j >= first && i * NI + j < last) acc[i][j] = Mfma<T>::run(fa[buf][i], fb[buf][j], acc[i][j]);
+    };
+    constexpr int kMfmaPerSlice = MI * NI, kReadsPerSlice = MI + NI, kWritesPerStep = A_CH + B_CH;
+    // One K step out of LDS stage `stage`, whose slice-0 fragments are already in buffer 0.
+    // HAS_NEXT: also prefetch step kt + 1 from global memory (FULL: all of its 64 columns exist), store it into the other
+    // LDS stage and fetch its slice-0 fragments.
+    auto k_step = [&](int stage, int kt, auto has_next, auto full) {
+      constexpr bool HAS_NEXT = decltype(has_next)::value;
+      if constexpr (HAS_NEXT) load_global(kt + 1, full);
+  #pragma unroll
+      for (int kk = 0; kk + 1 < KK; ++kk) {
+        read_frags(stage, kk + 1, (kk + 1) & 1);
+        mfma_range(kk & 1, 0, kMfmaPerSlice);
+  #pragma unroll
+        for (int g = 0; g < kReadsPerSlice; ++g) {  // pin the interleave: 1 global load, 1 LDS read, a share of the MFMAs
+          if constexpr (HAS_NEXT) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, kMfmaPerSlice / kReadsPerSlice, 0);
+        }
+      }
+      constexpr int last = (KK - 1) & 1;
+      if constexpr (HAS_NEXT) {
+        // last slice: its first half hides the LDS stores of the next step, the barrier, then its second half hides the
+        // first fragment reads of the next step
+        store_lds(stage ^ 1);
+        mfma_range(last, 0, kMfmaPerSlice / 2);
+  #pragma unroll
+        for (int g = 0; g < kMfmaPerSlice / 2; ++g) {
+          __builtin_amdgcn_sched_group_barrier(0x200, (kWritesPerStep + kMfmaPerSlice / 2 - 1) / (kMfmaPerSlice / 2), 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+        __syncthreads();
+        read_frags(stage ^ 1, 0, 0);
+        mfma_range(last, kMfmaPerSlice / 2, kMfmaPerSlice);
+  #pragma unroll
+        for (int g = 0; g < kMfmaPerSlice / 2; ++g) {
+          __builtin_amdgcn_sched_group_barrier(0x100, (kReadsPerSlice + kMfmaPerSlice / 2 - 1) / (kMfmaPerSlice / 2), 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+      } else {
+        mfma_range(last, 0, kMfmaPerSlice);
+      }
+    };
+
+    const int nk = (k_len + BK - 1) / BK;
+    const int nk_full = k_len / BK;  // steps whose 64 columns all exist
+    if (nk > 0) {
+      if (nk_full > 0) load_global(0, std::true_type{});
+      else load_global(0, std::false_type{});
+      store_lds(0);
+      __syncthreads();
+      read_frags(0, 0, 0);
+      int kt = 0;
+      for (; kt + 1 < nk_full; ++kt) k_step(kt & 1, kt, std::true_type{}, std::true_type{});
+      for (; kt + 1 < nk; ++kt) k_step(kt & 1, kt, std::true_type{}, std::false_type{});  // ragged last columns
+      k_step((nk - 1) & 1, nk - 1, std::false_type{}, std::false_type{});
+    }
+
+  } else {
+    // ---- PIPE 1: direct-to-LDS pipeline
+    constexpr int BK1 = 32, NSTAGE = 4, KS = BK1 / 16;
+    constexpr int A_LD = BM / 64, B_LD = BN / 64;  // 1 KiB wave-loads per wave per step and operand
+    constexpr int kStageBytes = (BM + BN) * BK1 * 2;
+    constexpr int kRowBytes = BK1 * 2;  // 64 B = 4 chunks; chunk c of row r sits in slot c ^ swz(r)
+    auto swz = [](int row) { return ((row >> 2) & 1) | ((((row >> 1) ^ (row >> 3)) & 1) << 1); };
+    char* lds_c = reinterpret_cast<char*>(lds_raw);
+    const char* a_base = static_cast<const char*>(prm.a);
+    const char* b_base = static_cast<const char*>(prm.w);
+    // A wave-load writes 64 consecutive 16-byte slots of LDS (lane l -> slot l): 16 tile rows x 4 slots. The lane
+    // fetches the global chunk that belongs in its slot.
+    uint32_t a_off[A_LD], b_off[B_LD];
+    if constexpr (MODE != kDw) b_base += (int64_t)expert * prm.w_expert_stride * 2;
+#pragma unroll
+    for (int t = 0; t < A_LD; ++t) {
+      const int r = (wave * A_LD + t) * 16 + (lane >> 2);
+      const int c = (lane & 3) ^ swz(r);
+      int64_t row;
+      if constexpr (MODE == kDw) {
+        row = min(m0 + r, (int64_t)prm.M - 1);
+      } else {
+        int64_t p = m0 + r;
+        if (p >= valid_end) p = valid_end - 1;  // pad rows re-read a valid row; their results are never stored
+        row = prm.a_gather_div > 0 ? (int64_t)(prm.row_slot[p] / prm.a_gather_div) : p;
+      }
+      a_off[t] = (uint32_t)((row * prm.lda + k_begin) * 2 + c * 16);
+    }
+#pragma unroll
+    for (int t = 0; t < B_LD; ++t) {
+      const int j = (wave * B_LD + t) * 16 + (lane >> 2);  // row of the LDS B tile
+      const int c = (lane & 3) ^ swz(j);
+      int64_t n;
+      if constexpr (MODE == kSwiglu) {
+        const int half = (j % WN) / (WN / 2);
+        const int within = (j / WN) * (WN / 2) + (j % (WN / 2));
+        n = (int64_t)half * prm.I + min((int64_t)nt * (BN / 2) + within, (int64_t)prm.I - 1);
+      } else {
+        n = min((int64_t)nt * BN + j, (int64_t)prm.N - 1);
+      }
+      b_off[t] = (uint32_t)((n * prm.ldw + k_begin) * 2 + c * 16);
+    }
+    const int nk = k_len / BK1;
+    // loads of K step `step` into stage step % 4; steps past the end re-fetch the last one (never read) so that the
+    // number of loads in flight is the same at every wait
+    // One wave-load: global -> LDS, no registers in between. Issued as inline asm so that the compiler's wait-count
+    // pass does not serialise the pipeline behind it; the waits for these loads are the explicit ones below.
+    auto dma16 = [&](const char* src, uint32_t lds_addr) {
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(src) : "m0");
+    };
+    const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds_c;
+    const uint32_t wave_a = __builtin_amdgcn_readfirstlane(lds_base + wave * A_LD * 1024);
+    const uint32_t wave_b = __builtin_amdgcn_readfirstlane(lds_base + BM * kRowBytes + wave * B_LD * 1024);
+    constexpr int kLoadsPerStep = A_LD + B_LD, kReads = MI + NI, kMfma = MI * NI;
+    // load number `g` (0 .. kLoadsPerStep) of K step `step` into stage step % 4; steps past the end re-fetch the last
+    // one (never read) so that the number of loads in flight is the same at every wait
+    auto issue_one = [&](int step, int g) {
+      const int64_t kb = (CK_ABLATE & 16) ? (int64_t)0 : (int64_t)min(step, nk - 1) * kRowBytes;  // 16: always K step 0
+      const uint32_t st = (uint32_t)((step & (NSTAGE - 1)) * kStageBytes);
+      if (g < A_LD) dma16(a_base + kb + a_off[g], wave_a + st + g * 1024);
+      else dma16(b_base + kb + b_off[g - A_LD], wave_b + st + (g - A_LD) * 1024);
+    };
+    auto issue = [&](int step) {
+#pragma unroll
+      for (int g = 0; g < kLoadsPerStep; ++g) issue_one(step, g);
+    };
+    typedef typename Mfma<T>::frag frag_t;
+    const int fsw = swz(lane & 31), fh = lane >> 5;
+    int slice_off[KS];
+#pragma unroll
+    for (int sl = 0; sl < KS; ++sl) slice_off[sl] = (((2 * sl + fh) ^ fsw) * 16);
+    const int fa_row = (wm * WM + (lane & 31)) * kRowBytes;
+    const int fb_row = BM * kRowBytes + (wn * WN + (lane & 31)) * kRowBytes;
+    frag_t fa[2][MI], fb[2][NI];
+    // fragment `g` of a slice: g < MI -> A block g, else B block g - MI
+    auto read_one = [&](int stage, int sl, int buf, int g) {
+      const char* st = lds_c + stage * kStageBytes + slice_off[sl];
+      if (g < MI) fa[buf][g] = *reinterpret_cast<const frag_t*>(st + fa_row + g * 32 * kRowBytes);
+      else fb[buf][g - MI] = *reinterpret_cast<const frag_t*>(st + fb_row + (g - MI) * 32 * kRowBytes);
+    };
+    auto mfma_range = [&](int buf, int first, int last) {
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+          if (i * NI + j >= first && i * NI + j < last) acc[i][j] = Mfma<T>::run(fa[buf][i], fb[buf][j], acc[i][j]);
+    };
+    // wait until at most `pending` of this wave's loads are in flight, then meet the other waves
+    auto wait_and_barrier = [&](auto pending) {
+      constexpr int kPending = decltype(pending)::value;
+      if constexpr (!(CK_ABLATE & 8)) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kPending) : "memory");
+      if constexpr (!(CK_ABLATE & 1)) asm volatile("s_barrier" ::: "memory");
+    };
+    // fragment read order: A0, then every B block, then the remaining A blocks -- the order the MFMAs need them in
+    auto read_nth = [&](int stage, int sl, int buf, int n) {
+      const int g = n == 0 ? 0 : (n <= NI ? MI + n - 1 : n - NI);
+      if constexpr (!(CK_ABLATE & 4)) read_one(stage, sl, buf, g);
+    };
+    constexpr int kPerGroup = kMfma / kReads;  // MFMAs per fragment read
+    if (nk > 0) {
+      issue(0);
+      issue(1);
+      issue(2);
+      wait_and_barrier(std::integral_constant<int, 2 * kLoadsPerStep>{});  // step 0 has landed, for every wave
+#pragma unroll
+      for (int g = 0; g < kReads; ++g) read_one(0, 0, 0, g);
+      for (int kt = 0; kt < nk; ++kt) {
+        // first half: MFMAs of slice 0 from fragment buffer 0, the fragment reads of slice 1 between them
+#pragma unroll
+        for (int g = 0; g < kReads; ++g) {
+          read_nth(kt & (NSTAGE - 1), 1, 1, g);
+          mfma_range(0, g * kPerGroup, (g + 1) * kPerGroup);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        // Step kt + 1 has landed for every wave (only step kt + 2 may still be in flight). The barrier also orders
+        // the overwrite below: stage (kt + 3) % 4 was last read as slice 1 of step kt - 1, and every wave consumed
+        // those fragments (so its reads completed) before arriving here.
+        wait_and_barrier(std::integral_constant<int, kLoadsPerStep>{});
+        // second half: MFMAs of slice 1 from buffer 1; between them the loads of step kt + 3 and the slice-0 fragment
+        // reads of step kt + 1
+#pragma unroll
+        for (int g = 0; g < kReads; ++g) {
+          if constexpr (!(CK_ABLATE & 2))
+            if (g < kLoadsPerStep) issue_one(kt + 3, g);
+          read_nth((kt + 1) & (NSTAGE - 1), 0, 0, g);
+          mfma_range(1, g * kPerGroup, (g + 1) * kPerGroup);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        static_assert(kLoadsPerStep <= kReads, "every load of a step has a slot in the second half");
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the re-fetches before LDS is reused or released
+    }
   }
 
   // ---- epilogue. Lane holds, per 32x32 block and q in 0..3, rows 8q + 4*(lane/32) + 0..3 of column lane%32.
@@ -430,28 +575,36 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
   }
 }
 
-template <int BM, int BN>
+template <int BM, int BN, int PIPE>
 constexpr size_t lds_bytes() {
-  return (size_t)2 * (BM + BN) * kLdsStride * 2;
+  return PIPE == 0 ? (size_t)2 * (BM + BN) * kLdsStride * 2 : (size_t)4 * (BM + BN) * 32 * 2;
 }
 
-template <typename T, int BM, int BN, int MODE>
-int launch(const GemmParams& prm, unsigned blocks, hipStream_t s, const char* name) {
-  auto kernel = grouped_gemm_kernel<T, BM, BN, MODE>;
+template <typename T, int BM, int BN, int MODE, int PIPE>
+int launch_pipe(const GemmParams& prm, unsigned blocks, hipStream_t s, const char* name) {
+  auto kernel = grouped_gemm_kernel<T, BM, BN, MODE, PIPE>;
   static bool attr_set = false;  // per instantiation; the attribute is idempotent, a race only repeats the call
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)lds_bytes<BM, BN>());
+                                       (int)lds_bytes<BM, BN, PIPE>());
     if (e != hipSuccess) {
-      set_error("%s: cannot reserve %zu bytes of LDS: %s", name, lds_bytes<BM, BN>(), hipGetErrorString(e));
+      set_error("%s: cannot reserve %zu bytes of LDS: %s", name, lds_bytes<BM, BN, PIPE>(), hipGetErrorString(e));
       return CK_ERR_LAUNCH;
     }
     attr_set = true;
   }
-  constexpr size_t kLds = lds_bytes<BM, BN>();
+  constexpr size_t kLds = lds_bytes<BM, BN, PIPE>();
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kThreads), kLds, s, prm);
   CK_CHECK_LAUNCH(name);
   return CK_OK;
+}
+
+// the direct-to-LDS pipeline whenever the contraction length allows it
+template <typename T, int BM, int BN, int MODE>
+int launch(const GemmParams& prm, unsigned blocks, hipStream_t s, const char* name) {
+  const bool dma = (MODE == kDw) || (prm.K % 32 == 0);
+  if (dma && !g_force_pipe0) return launch_pipe<T, BM, BN, MODE, 1>(prm, blocks, s, name);
+  return launch_pipe<T, BM, BN, MODE, 0>(prm, blocks, s, name);
 }
 
 template <typename T, int MODE>

@@ -156,6 +156,59 @@ __global__ __launch_bounds__(kBlock) void group_rows_padded_kernel(
   store_tile_transposed<T>(tile, grouped_t, ld_t, p0, h0, min(kTile, H - h0), p0 + kTile);
 }
 
+// SwiGLU backward over padded grouped rows, with the transposed copy the weight-gradient GEMM consumes:
+//   d_pre[p, :] = swiglu_bwd(pre[p, :], d_act[p, :]) for valid rows;  d_pre_t = d_pre^T with zeros in pad rows.
+// grid: (ceil(I / 64), max_rows / 64); pre / d_pre are [max_rows, 2I] packed [up | gate], d_act is [max_rows, I].
+template <typename T>
+__global__ __launch_bounds__(kBlock) void swiglu_bwd_grouped_kernel(
+    const T* __restrict__ pre, const T* __restrict__ d_act, int I, const int32_t* __restrict__ seg_starts,
+    const uint32_t* __restrict__ counts, const int32_t* __restrict__ tile_expert, int align, T* __restrict__ d_pre,
+    T* __restrict__ d_pre_t, int64_t ld_t) {
+  __shared__ T tile_up[kTile][kTileStride];
+  __shared__ T tile_gate[kTile][kTileStride];
+  const int64_t p0 = (int64_t)blockIdx.y * kTile;
+  const int e = tile_expert[p0 / align];
+  if (e < 0) return;
+  const int64_t valid_end = (int64_t)seg_starts[e] + counts[e];
+  const int c0 = blockIdx.x * kTile;
+  const int64_t two_i = 2 * (int64_t)I;
+#pragma unroll
+  for (int q = 0; q < (kTile * kTile / 8) / kBlock; ++q) {
+    const int chunk = q * kBlock + threadIdx.x;
+    const int r = chunk >> 3, cc = chunk & 7;
+    const int64_t p = p0 + r;
+    const int c = c0 + cc * 8;
+    Pack16<T> du, dg;
+    du.v = zero16();
+    dg.v = zero16();
+    if (p < valid_end && c < I) {
+      Pack16<T> u, g, dy;
+      u.v = load16(pre + p * two_i + c);
+      g.v = load16(pre + p * two_i + I + c);
+      dy.v = load16(d_act + p * I + c);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float gf = Elem<T>::up(g.e[i]), uf = Elem<T>::up(u.e[i]), dyf = Elem<T>::up(dy.e[i]);
+        const float sg = sigmoid_f32(gf);
+        const float gsg = gf * sg;
+        dg.e[i] = Elem<T>::down(dyf * uf * (sg + gsg * (1.0f - sg)));
+        du.e[i] = Elem<T>::down(dyf * gsg);
+      }
+      store16(d_pre + p * two_i + c, du.v);
+      store16(d_pre + p * two_i + I + c, dg.v);
+    }
+    if (d_pre_t != nullptr) {
+      fill_tile_chunk(tile_up, r, cc, du.v);
+      fill_tile_chunk(tile_gate, r, cc, dg.v);
+    }
+  }
+  if (d_pre_t == nullptr) return;
+  __syncthreads();
+  const int cols_ok = min(kTile, I - c0);
+  store_tile_transposed<T>(tile_up, d_pre_t, ld_t, p0, c0, cols_ok, p0 + kTile);
+  store_tile_transposed<T>(tile_gate, d_pre_t, ld_t, p0, (int64_t)I + c0, cols_ok, p0 + kTile);
+}
+
 // dst[b, c, r] = src[b, r, c]; grid: (ceil(cols/64), ceil(rows/64), batch); rows % 8 == 0 and cols % 8 == 0
 template <typename T>
 __global__ __launch_bounds__(kBlock) void transpose_batched_kernel(const T* __restrict__ src, int rows, int cols,
@@ -263,6 +316,32 @@ extern "C" int ck_group_rows_padded(const void* src, const void* coeff, int32_t 
                        static_cast<scalar_t*>(grouped_t), ld_t);
   });
   CK_CHECK_LAUNCH("ck_group_rows_padded");
+  return CK_OK;
+}
+
+extern "C" int ck_swiglu_bwd_grouped(const void* pre, const void* d_act, int32_t I, const int32_t* seg_starts,
+                                     const uint32_t* counts, const int32_t* tile_expert, int32_t align,
+                                     int64_t max_rows, void* d_pre, void* d_pre_t, int64_t ld_t, int32_t dtype,
+                                     void* stream) {
+  CK_REQUIRE(I >= 8 && I % 8 == 0, "ck_swiglu_bwd_grouped: I=%d must be a positive multiple of 8", I);
+  CK_REQUIRE(align >= kTile && align % kTile == 0, "ck_swiglu_bwd_grouped: align=%d must be a multiple of %d", align, kTile);
+  CK_REQUIRE(max_rows >= 0 && max_rows % align == 0, "ck_swiglu_bwd_grouped: max_rows=%lld is not a multiple of align",
+             (long long)max_rows);
+  if (max_rows == 0) return CK_OK;
+  CK_REQUIRE(pre && d_act && d_pre && seg_starts && counts && tile_expert, "ck_swiglu_bwd_grouped: NULL argument");
+  CK_REQUIRE(d_pre_t == nullptr || (ld_t >= max_rows && ld_t % 8 == 0),
+             "ck_swiglu_bwd_grouped: ld_t=%lld must be >= max_rows and a multiple of 8", (long long)ld_t);
+  CK_REQUIRE(aligned16(pre) && aligned16(d_act) && aligned16(d_pre) && (!d_pre_t || aligned16(d_pre_t)),
+             "ck_swiglu_bwd_grouped: pointers must be 16-byte aligned");
+  CK_REQUIRE(max_rows / kTile <= 65535, "ck_swiglu_bwd_grouped: too many rows for one launch");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)ceil_div(I, kTile), (unsigned)(max_rows / kTile));
+  CK_DISPATCH_HALF(dtype, "ck_swiglu_bwd_grouped", {
+    hipLaunchKernelGGL((swiglu_bwd_grouped_kernel<scalar_t>), grid, dim3(kBlock), 0, s,
+                       static_cast<const scalar_t*>(pre), static_cast<const scalar_t*>(d_act), (int)I, seg_starts, counts,
+                       tile_expert, (int)align, static_cast<scalar_t*>(d_pre), static_cast<scalar_t*>(d_pre_t), ld_t);
+  });
+  CK_CHECK_LAUNCH("ck_swiglu_bwd_grouped");
   return CK_OK;
 }
 

@@ -51,6 +51,10 @@ _SIGNATURES = {
         c_int32,
         [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_int64, c_int32, c_void_p],
     ),
+    "ck_swiglu_bwd_grouped": (
+        c_int32,
+        [c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_int64, c_int32, c_void_p],
+    ),
     "ck_transpose_batched": (c_int32, [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_int32, c_void_p]),
     "ck_grouped_gemm": (
         c_int32,

@@ -443,12 +443,23 @@ class _SwigluExperts(torch.autograd.Function):
             del d_y_t
 
         if need_x or need_fc:
-            # d_act = d_y @ w_proj, SwiGLU backward in the epilogue -> d_pre (+ transpose for d_w_fc)
+            # d_act = d_y @ w_proj with the leanest epilogue, then one streaming pass for the SwiGLU backward and the
+            # transpose d_w_fc needs. (The GEMM can also do this in its epilogue, CK_EPI_SWIGLU_BWD, but with one
+            # workgroup per CU the epilogue is time the MFMA units idle, while the streaming pass runs at HBM speed.)
             w_proj_t = _transpose_weights(w_proj)  # [E, I, H]
+            d_act = torch.empty(seg.max_rows, I, dtype=dt, device=dev)
+            _gemm(d_y, 0, w_proj_t, seg, _C.CK_EPI_GROUPED, d_act)
+            del w_proj_t, d_y
             d_pre = torch.empty(seg.max_rows, two_i, dtype=dt, device=dev)
             d_pre_t = torch.empty(two_i, seg.ld_t, dtype=dt, device=dev) if need_fc else None
-            _gemm(d_y, 0, w_proj_t, seg, _C.CK_EPI_SWIGLU_BWD, d_pre, y_t=d_pre_t, aux_in=pre)
-            del w_proj_t, d_y
+            with torch.cuda.device(dev):
+                _C.check(
+                    _C.lib().ck_swiglu_bwd_grouped(
+                        _C.ptr(pre), _C.ptr(d_act), I, _C.ptr(seg.seg_starts), _C.ptr(seg.counts), _C.ptr(seg.tile_expert),
+                        seg.align, seg.max_rows, _C.ptr(d_pre), _C.ptr(d_pre_t), seg.ld_t, _C.dtype_code(dt), _C.stream(),
+                    )
+                )
+            del d_act
             if need_fc:
                 _, x_t = _group_rows(x, None, k, seg, False, True)
                 d_w_fc = torch.empty_like(w_fc)

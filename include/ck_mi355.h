@@ -115,6 +115,13 @@ int ck_group_rows_padded(const void* src, const void* coeff, int32_t fan_out, in
                          const int32_t* seg_starts, const uint32_t* counts, const int32_t* tile_expert,
                          int32_t align, int64_t max_rows, void* grouped, void* grouped_t, int64_t ld_t,
                          int32_t dtype, void* stream);
+/* SwiGLU backward over padded grouped rows (formula: cute_kernels/kernels/swiglu/cuda_implementation/backward.cu:27-41),
+ * writing what the weight-gradient GEMM consumes in the same pass:
+ *   pre [max_rows, 2I] packed [up | gate], d_act [max_rows, I]  ->  d_pre [max_rows, 2I] (valid rows only) and
+ *   d_pre_t [2I, ld_t] = d_pre^T with zeros in the pad rows of live tiles (may be NULL). I % 8 == 0. 16-bit dtypes. */
+int ck_swiglu_bwd_grouped(const void* pre, const void* d_act, int32_t I, const int32_t* seg_starts,
+                          const uint32_t* counts, const int32_t* tile_expert, int32_t align, int64_t max_rows,
+                          void* d_pre, void* d_pre_t, int64_t ld_t, int32_t dtype, void* stream);
 /* Batched 2-D transpose: dst[b, c, r] = src[b, r, c]; src [batch, rows, cols]. 16-bit dtypes only. */
 int ck_transpose_batched(const void* src, int64_t batch, int32_t rows, int32_t cols, void* dst, int32_t dtype,
                          void* stream);

@@ -120,6 +120,21 @@ def test_grouped_gemm_swiglu_epilogues(device, dtype, align, K, I):
     torch.testing.assert_close(d_pre.float().cpu()[valid], pre_c.grad[valid], rtol=2e-2, atol=2e-2)
     assert torch.equal(d_pre_t.cpu()[:, :live], (d_pre.cpu()[:live] * valid[:live, None]).t())
 
+    # the same backward as a plain GEMM followed by the streaming SwiGLU-backward pass (what the layer uses)
+    d_act_gpu = torch.zeros(seg.max_rows, I, dtype=dtype, device=device)
+    scattermoe._gemm(d_y.to(device), 0, w_proj_t.to(device), seg, _C.CK_EPI_GROUPED, d_act_gpu)
+    d_pre2 = torch.zeros(seg.max_rows, 2 * I, dtype=dtype, device=device)
+    d_pre2_t = torch.full((2 * I, seg.ld_t), 7.0, dtype=dtype, device=device)
+    _C.check(
+        _C.lib().ck_swiglu_bwd_grouped(
+            pre.data_ptr(), d_act_gpu.data_ptr(), I, seg.seg_starts.data_ptr(), seg.counts.data_ptr(),
+            seg.tile_expert.data_ptr(), seg.align, seg.max_rows, d_pre2.data_ptr(), d_pre2_t.data_ptr(), seg.ld_t,
+            _C.dtype_code(dtype), torch.cuda.current_stream().cuda_stream,
+        )
+    )
+    torch.testing.assert_close(d_pre2.float().cpu()[valid], pre_c.grad[valid], rtol=2e-2, atol=2e-2)
+    assert torch.equal(d_pre2_t.cpu()[:, :live], (d_pre2.cpu()[:live] * valid[:live, None]).t())
+
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("align", [128, 256])
