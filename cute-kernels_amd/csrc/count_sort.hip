@@ -8,6 +8,8 @@
 //         [bin][segment]; the last block scans that flattened table, which is exactly the destination of the first id of
 //         every (bin, segment) pair in a stable sort, and derives counts / offsets / tile-aligned segment starts /
 //         tile->expert table. (2) every wave re-reads its segment in order and ranks ids 64 at a time with bit-ballots.
+#include <stdlib.h>
+
 #include "ck_common.h"
 
 namespace ck {
@@ -54,8 +56,12 @@ __device__ uint32_t block_exclusive_scan(uint32_t* data, int n, uint32_t* tmp) {
 
 // Returns true in every thread of exactly one block: the last one to arrive. Blocks must have made their global
 // writes before calling; the caller may read other blocks' writes after a true return.
+// FENCE = false is for blocks that publish their data only through device-scope atomics: those are coherent across the
+// XCDs by themselves and are complete once the barrier below has drained the wave's memory counters, so the L2
+// write-back + invalidate of a full fence (about 0.2 us per block, serialised) is not needed.
+template <bool FENCE>
 __device__ bool last_block_ticket(uint32_t* ticket, uint32_t* lds_flag) {
-  __threadfence();
+  if constexpr (FENCE) __threadfence();
   __syncthreads();
   if (threadIdx.x == 0) {
     const uint32_t prev = atomicAdd(ticket, 1u);
@@ -63,7 +69,7 @@ __device__ bool last_block_ticket(uint32_t* ticket, uint32_t* lds_flag) {
   }
   __syncthreads();
   const bool last = (*lds_flag != 0u);
-  if (last) __threadfence();
+  if (FENCE && last) __threadfence();
   return last;
 }
 
@@ -91,10 +97,12 @@ struct RegCounters {
   }
 };
 
-// REG_BINS > 0: wave-uniform register counters via ballot (num_bins <= REG_BINS). REG_BINS == 0: LDS atomics.
+// REG_BINS > 0: wave-uniform register counters via ballot (num_bins <= REG_BINS): a handful of bins would make every
+//               lane of an LDS atomic hit the same few addresses.
+// REG_BINS == 0: LDS atomics on per-wave copies of the histogram.
 template <typename id_t, int REG_BINS>
 __global__ __launch_bounds__(kBlock) void count_kernel(const id_t* __restrict__ ids, int64_t n, int num_bins,
-                                                        int lds_copies, uint32_t* __restrict__ counts,
+                                                        int lds_copies, int replicas, uint32_t* __restrict__ counts,
                                                         uint32_t* __restrict__ ends, uint32_t* __restrict__ starts,
                                                         uint32_t* __restrict__ ws) {
   extern __shared__ uint32_t lds[];  // [lds_copies][num_bins] then kWavesPerBlock + 1 words of scan scratch
@@ -179,12 +187,19 @@ __global__ __launch_bounds__(kBlock) void count_kernel(const id_t* __restrict__ 
     __syncthreads();
   }
 
+  // Blocks merge into one of `replicas` global accumulators (thousands of atomics on one cache line would serialise in a
+  // single L2 channel); the last block adds the replicas up and puts them back to zero.
   uint32_t* acc = ws + 1;
   if (gridDim.x > 1) {
+    uint32_t* my_acc = acc + (size_t)(blockIdx.x % replicas) * num_bins;
     for (int e = t; e < num_bins; e += kBlock)
-      if (hist[e]) atomicAdd(&acc[e], hist[e]);
-    if (!last_block_ticket(ws, tmp + kWavesPerBlock)) return;
-    for (int e = t; e < num_bins; e += kBlock) hist[e] = atomicExch(&acc[e], 0u);  // read and restore the zero
+      if (hist[e]) atomicAdd(&my_acc[e], hist[e]);
+    if (!last_block_ticket<false>(ws, tmp + kWavesPerBlock)) return;
+    for (int e = t; e < num_bins; e += kBlock) {
+      uint32_t s = 0;
+      for (int r = 0; r < replicas; ++r) s += atomicExch(&acc[(size_t)r * num_bins + e], 0u);  // read, restore the zero
+      hist[e] = s;
+    }
     if (t == 0) ws[0] = 0u;
     __syncthreads();
   }
@@ -247,7 +262,7 @@ __global__ __launch_bounds__(kBlock) void sort_hist_kernel(const id_t* __restric
 
   const int table_words = E * S;
   uint32_t* tmp = lds + max(kWavesPerBlock * E, table_words + E + 1);
-  if (!last_block_ticket(ws, tmp + kWavesPerBlock)) return;
+  if (!last_block_ticket<true>(ws, tmp + kWavesPerBlock)) return;
 
   // ---- last block: scan the flattened bin-major table in LDS
   uint32_t* tab = lds;
@@ -334,7 +349,15 @@ __global__ __launch_bounds__(kBlock) void sort_scatter_kernel(const id_t* __rest
 
 using namespace ck;
 
-extern "C" int64_t ck_count_workspace_words(int32_t num_bins) { return 1 + (int64_t)(num_bins > 0 ? num_bins : 0); }
+// global accumulator replicas: as many as fit in 16384 words, at most 32
+static int count_replicas(int num_bins) {
+  int r = kMaxCountBins / (num_bins > 0 ? num_bins : 1);
+  return r < 1 ? 1 : (r > 32 ? 32 : r);
+}
+
+extern "C" int64_t ck_count_workspace_words(int32_t num_bins) {
+  return 1 + (int64_t)(num_bins > 0 ? num_bins : 0) * count_replicas(num_bins);
+}
 
 extern "C" int ck_count_offsets(const void* ids, int32_t ids_are_i64, int64_t n, int32_t num_bins, uint32_t* counts,
                                 uint32_t* ends, uint32_t* starts, uint32_t* workspace, void* stream) {
@@ -350,14 +373,19 @@ extern "C" int ck_count_offsets(const void* ids, int32_t ids_are_i64, int64_t n,
   // 4 vectors per thread per trip; enough blocks to fill 256 CUs a few times over, one block for small inputs
   int64_t blocks = ceil_div(n, (int64_t)kBlock * vec * 4 * 4);
   if (blocks < 1) blocks = 1;
-  if (blocks > 2048) blocks = 2048;
+  if (blocks > 1024) blocks = 1024;  // 4 per CU: 16 waves per CU keep HBM busy, and the merge stays short
+  if (const char* env = getenv("CK_COUNT_BLOCKS")) {  // tuning knob for measurements
+    const long v = atol(env);
+    if (v >= 1 && v <= 65535) blocks = v;
+  }
   const int reg_bins = num_bins <= 8 ? 8 : (num_bins <= 16 ? 16 : 0);
-  const int copies = reg_bins ? 1 : (num_bins <= 1024 ? kWavesPerBlock : 1);
+  const int copies = reg_bins > 0 ? 1 : (num_bins <= 1024 ? kWavesPerBlock : 1);
   const size_t lds_bytes = ((size_t)copies * num_bins + kWavesPerBlock + 2) * sizeof(uint32_t);
   hipStream_t s = static_cast<hipStream_t>(stream);
 #define CK_LAUNCH_COUNT(ID_T, RB)                                                                              \
   hipLaunchKernelGGL((count_kernel<ID_T, RB>), dim3((unsigned)blocks), dim3(kBlock), lds_bytes, s,            \
-                     static_cast<const ID_T*>(ids), n, (int)num_bins, copies, counts, ends, starts, workspace)
+                     static_cast<const ID_T*>(ids), n, (int)num_bins, copies, count_replicas(num_bins), counts, ends,   \
+                     starts, workspace)
   if (ids_are_i64) {
     if (reg_bins == 8) CK_LAUNCH_COUNT(int64_t, 8);
     else if (reg_bins == 16) CK_LAUNCH_COUNT(int64_t, 16);

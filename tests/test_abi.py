@@ -48,7 +48,8 @@ def test_argument_validation_returns_error_and_message():
 
 def test_host_side_size_helpers():
     lib = _C.lib()
-    assert lib.ck_count_workspace_words(64) == 65
+    assert lib.ck_count_workspace_words(64) == 1 + 64 * 32
+    assert lib.ck_count_workspace_words(16384) == 1 + 16384
     # sum_e round_up(c_e, align) <= R + E*(align-1), rounded to whole tiles
     assert lib.ck_sort_max_rows(32768, 8, 256) == 34816
     assert lib.ck_sort_max_rows(0, 8, 128) % 128 == 0
