@@ -25,6 +25,16 @@ for _p in (ROOT, os.path.join(ROOT, "cute-kernels_amd")):
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E
 
+# Bytes per launch between L2 and the fabric (fetched + written) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
+# this same command, FETCH_SIZE scaled x2.0 and WRITE_SIZE x1.0 against transpose_batched_kernel (known size);
+# summary and commands: profiles/grouped_gemm_c3_moe_fwd_bwd.md. Not measurable from inside this process.
+TRAFFIC_BYTES_PER_LAUNCH = {
+    "grouped_gemm<scatter>": 13.9e9 + 0.27e9,
+    "grouped_gemm<dw>": 10.0e9 + 1.41e9,
+    "grouped_gemm<swiglu>": 19.5e9 + 4.92e9,
+    "grouped_gemm<grouped>": 9.5e9 + 0.94e9,
+}
+
 # workload: configs[2] of the baseline, the configuration its headline metric (MoE fwd+bwd TFLOP/s) is quoted on
 T, H, E, TOP_K, I = 16384, 4096, 8, 2, 14336
 SEED = 42
@@ -123,11 +133,24 @@ def secondary_hbm_kernels(dev):
         torch.cuda.synchronize()
         return s.elapsed_time(e) / iters * 1e-3
 
+    from cute_kernels import _C
+
     out = {}
     g = torch.Generator().manual_seed(SEED)
-    for n in (1 << 16, 1 << 28):
-        ids = torch.randint(0, 64, (n,), generator=g, dtype=torch.int32).to(dev) if n <= (1 << 20) else torch.randint(0, 64, (n,), dtype=torch.int32, device=dev)
-        dt = timed(lambda: cute_kernels.continuous_count_and_offsets_cute(ids, 64))
+    lib = _C.lib()
+    for n in (1 << 16, 1 << 22, 1 << 28):
+        ids = torch.randint(0, 64, (n,), generator=g, dtype=torch.int32).to(dev) if n <= (1 << 22) else torch.randint(0, 64, (n,), dtype=torch.int32, device=dev)
+        # straight through the C ABI with caller-owned outputs, as a C caller would (no Python-side allocation in the loop)
+        counts, ends, starts = (torch.empty(64, dtype=torch.uint32, device=dev) for _ in range(3))
+        ws = torch.zeros(lib.ck_count_workspace_words(64), dtype=torch.int32, device=dev)
+        stream = torch.cuda.current_stream().cuda_stream
+
+        def count():
+            _C.check(lib.ck_count_offsets(ids.data_ptr(), 0, n, 64, counts.data_ptr(), ends.data_ptr(), starts.data_ptr(),
+                                          ws.data_ptr(), stream))
+
+        dt = timed(count, iters=200 if n <= (1 << 22) else 20)
+        assert int(ends[-1]) == n
         b = 4 * n + 8 * 64 + 4 * 64
         out[f"count_offsets_N{n}_E64"] = {"us": dt * 1e6, "GB/s": b / dt / 1e9, "frac_hbm": b / dt / 1e9 / PEAK_HBM_GBS}
         del ids
@@ -156,6 +179,35 @@ def secondary_hbm_kernels(dev):
     return out
 
 
+def gemm_only(dev, launches: int):
+    """Just the c_fc-forward-shape grouped GEMM (grouped epilogue) at the C3 shape: the target of counter runs."""
+    import numpy as np
+    import torch
+
+    import cute_kernels
+    from cute_kernels import _C, scattermoe
+
+    R = T * TOP_K
+    p = 1.0 / np.arange(1, E + 1)
+    ids = torch.from_numpy(np.random.default_rng(SEED).choice(E, size=R, p=p / p.sum())).to(torch.int32)
+    seg = cute_kernels.sort_by_expert(ids.to(dev), E, 256)
+    x = torch.randn(T, H, device=dev, dtype=torch.bfloat16)
+    w = torch.randn(E, 2 * I, H, device=dev, dtype=torch.bfloat16) * 0.02
+    y = torch.empty(seg.max_rows, 2 * I, device=dev, dtype=torch.bfloat16)
+    for _ in range(2):
+        scattermoe._gemm(x, TOP_K, w, seg, _C.CK_EPI_GROUPED, y)
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(launches):
+        scattermoe._gemm(x, TOP_K, w, seg, _C.CK_EPI_GROUPED, y)
+    e.record()
+    torch.cuda.synchronize()
+    ms = s.elapsed_time(e) / launches
+    flops = 4.0 * R * H * I
+    print(json.dumps({"kernel": "grouped_gemm<grouped>", "shape": [R, 2 * I, H], "avg_launch_ms": ms,
+                      "TFLOP/s": flops / ms / 1e9, "frac_mfma": flops / ms / 1e9 / PEAK_BF16_TFLOPS}))
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -163,6 +215,11 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--skip-cpu-baseline", action="store_true")
     ap.add_argument("--skip-secondary", action="store_true")
+    ap.add_argument("--only-gemm", type=int, default=0, metavar="LAUNCHES",
+                    help="run only the c_fc-forward-shape grouped GEMM this many times (for rocprofv3 --pmc runs)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one 1 GiB device copy (outside the timed region): the known-size kernel that "
+                    "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build uses no second GPU (no collectives, no sharding); run with --gpus 1",
@@ -175,8 +232,18 @@ def main() -> int:
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
+    if args.only_gemm > 0:
+        gemm_only(dev, args.only_gemm)
+        return 0
     moe, x, grad_out, freq, zipf_c = build_layer(dev)
     x.requires_grad_()
+
+    if args.copy_calibration:
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).random_(0, 255)
+        dst = torch.empty_like(src)
+        dst.copy_(src)  # reads 2^30 B, writes 2^30 B
+        torch.cuda.synchronize()
+        del src, dst
 
     for _ in range(args.warmup):
         step(moe, x, grad_out)
@@ -212,7 +279,7 @@ def main() -> int:
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
         "frac": achieved / PEAK_BF16_TFLOPS,
-        "traffic": None,
+        "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(dominant),
         "avg_launch_ms": d["ms"] / d["launches"],
         "flops_per_launch": d["flops"] / d["launches"],
     }

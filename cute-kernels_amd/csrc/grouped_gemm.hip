@@ -8,6 +8,8 @@
 // Workgroup = 256 threads = 4 waves in a 2x2 grid; wave tile (BM/2)x(BN/2) built from 32x32 MFMA blocks; K step 64
 // staged through double-buffered LDS (rows padded to 72 elements so 16 lanes x 16 bytes cover all banks); the global
 // loads of step k+1 are in flight while step k is multiplied.
+#include <stdlib.h>
+
 #include <type_traits>
 
 #include "ck_common.h"
@@ -44,7 +46,11 @@ struct Mfma<f16_t> {
 #define CK_ABLATE 0  // measurement builds only: 1 no barrier, 2 no loads in the loop, 4 no fragment reads, 8 no load wait
 #endif
 
-bool g_force_pipe0 = false;  // set from the environment (CK_GEMM_PIPE=0) for A/B measurements
+// CK_GEMM_PIPE=0 in the environment forces the register-staged pipeline (A/B measurements)
+const bool g_force_pipe0 = [] {
+  const char* env = getenv("CK_GEMM_PIPE");
+  return env != nullptr && env[0] == '0';
+}();
 
 struct GemmParams {
   const void* a;      // forward modes: [*, K]; dW: a_t [M, ld_t]
