@@ -52,6 +52,12 @@ const bool g_force_pipe0 = [] {
   return env != nullptr && env[0] == '0';
 }();
 
+// CK_GEMM_WAVES=4 in the environment selects the 4-wave variant of the direct-to-LDS pipeline (default: 8 waves)
+const bool g_eight_waves = [] {
+  const char* env = getenv("CK_GEMM_WAVES");
+  return !(env != nullptr && env[0] == '4');
+}();
+
 struct GemmParams {
   const void* a;      // forward modes: [*, K]; dW: a_t [M, ld_t]
   const void* w;      // forward modes: [E, N, K]; dW: b_t [N, ld_t]
@@ -122,9 +128,14 @@ __device__ inline void grouped_order(int r, int a_count, int b_count, int& a, in
 // PIPE 0: K step 64, global -> registers -> padded LDS, two stages (any K % 8 == 0).
 // PIPE 1: K step 32, global -> LDS directly (no register staging), four XOR-swizzled stages, loads three steps ahead
 //         (needs K % 32 == 0).
-template <typename T, int BM, int BN, int MODE, int PIPE>
-__global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams prm) {
-  constexpr int WM = BM / 2, WN = BN / 2;    // wave tile
+// WGM: waves along M (2 or 4), always 2 along N: 4 waves = one per SIMD with 128x128 wave tiles at BM = BN = 256;
+//      8 waves = two per SIMD with 64x128 wave tiles, so that one wave's memory instructions issue under the other's
+//      MFMAs (PIPE 1 only).
+template <typename T, int BM, int BN, int MODE, int PIPE, int WGM>
+__global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmParams prm) {
+  static_assert(PIPE == 1 || WGM == 2, "the register-staged pipeline is written for 4 waves");
+  constexpr int NW = WGM * 2;                // waves per workgroup
+  constexpr int WM = BM / WGM, WN = BN / 2;  // wave tile
   constexpr int MI = WM / 32, NI = WN / 32;  // 32x32 blocks per wave tile
   constexpr int A_CH = BM / 32, B_CH = BN / 32;  // 16-byte chunks per thread per stage
   constexpr int kStageElems = (BM + BN) * kLdsStride;
@@ -338,7 +349,8 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
   } else {
     // ---- PIPE 1: direct-to-LDS pipeline
     constexpr int BK1 = 32, NSTAGE = 4, KS = BK1 / 16;
-    constexpr int A_LD = BM / 64, B_LD = BN / 64;  // 1 KiB wave-loads per wave per step and operand
+    constexpr int A_LD = BM / (16 * NW), B_LD = BN / (16 * NW);  // 1 KiB wave-loads per wave per step and operand
+    static_assert(A_LD >= 1 && B_LD >= 1, "tile too small for this many waves");
     constexpr int kStageBytes = (BM + BN) * BK1 * 2;
     constexpr int kRowBytes = BK1 * 2;  // 64 B = 4 chunks; chunk c of row r sits in slot c ^ swz(r)
     auto swz = [](int row) { return ((row >> 2) & 1) | ((((row >> 1) ^ (row >> 3)) & 1) << 1); };
@@ -383,7 +395,10 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
     // One wave-load: global -> LDS, no registers in between. Issued as inline asm so that the compiler's wait-count
     // pass does not serialise the pipeline behind it; the waits for these loads are the explicit ones below.
     auto dma16 = [&](const char* src, uint32_t lds_addr) {
-      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(src) : "m0");
+#ifndef CK_LOAD_MOD
+#define CK_LOAD_MOD ""
+#endif
+      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" CK_LOAD_MOD ::"s"(lds_addr), "v"(src) : "m0");
     };
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds_c;
     const uint32_t wave_a = __builtin_amdgcn_readfirstlane(lds_base + wave * A_LD * 1024);
@@ -416,6 +431,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
       else fb[buf][g - MI] = *reinterpret_cast<const frag_t*>(st + fb_row + (g - MI) * 32 * kRowBytes);
     };
     auto mfma_range = [&](int buf, int first, int last) {
+      if constexpr ((CK_ABLATE & 64) != 0) return;  // measurement builds: loads and fragment reads only
 #pragma unroll
       for (int i = 0; i < MI; ++i)
 #pragma unroll
@@ -433,7 +449,8 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
       const int g = n == 0 ? 0 : (n <= NI ? MI + n - 1 : n - NI);
       if constexpr (!(CK_ABLATE & 4)) read_one(stage, sl, buf, g);
     };
-    constexpr int kPerGroup = kMfma / kReads;  // MFMAs per fragment read
+    // MFMAs [mfma_begin(g), mfma_begin(g + 1)) follow fragment read g
+    auto mfma_begin = [](int g) { return g * kMfma / kReads; };
     if (nk > 0) {
       issue(0);
       issue(1);
@@ -446,7 +463,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
 #pragma unroll
         for (int g = 0; g < kReads; ++g) {
           read_nth(kt & (NSTAGE - 1), 1, 1, g);
-          mfma_range(0, g * kPerGroup, (g + 1) * kPerGroup);
+          mfma_range(0, mfma_begin(g), mfma_begin(g + 1));
           __builtin_amdgcn_sched_barrier(0);
         }
         // Step kt + 1 has landed for every wave (only step kt + 2 may still be in flight). The barrier also orders
@@ -460,7 +477,7 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
           if constexpr (!(CK_ABLATE & 2))
             if (g < kLoadsPerStep) issue_one(kt + 3, g);
           read_nth((kt + 1) & (NSTAGE - 1), 0, 0, g);
-          mfma_range(1, g * kPerGroup, (g + 1) * kPerGroup);
+          mfma_range(1, mfma_begin(g), mfma_begin(g + 1));
           __builtin_amdgcn_sched_barrier(0);
         }
         static_assert(kLoadsPerStep <= kReads, "every load of a step has a slot in the second half");
@@ -473,6 +490,151 @@ __global__ __launch_bounds__(kThreads) void grouped_gemm_kernel(const GemmParams
   // static_for keeps every accumulator index a compile-time constant (the accumulators live in AGPRs).
   const int col_in_block = lane & 31;
   const int row_quad = (lane >> 5) * 4;
+  if constexpr ((CK_ABLATE & 32) != 0) {  // measurement builds: no epilogue (keep the accumulators alive)
+    float keep = 0.f;
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+      for (int j = 0; j < NI; ++j) keep += acc[i][j][0];
+    if (keep == 123.456f) static_cast<float*>(prm.y)[0] = keep;
+    return;
+  }
+  if constexpr (BM == 256 && BN == 256 && MODE != kSwigluBwd && !(CK_ABLATE & 128)) {
+    // ---- staged epilogue (256x256 tiles): the tile leaves through LDS so that global stores are 16 bytes per lane
+    // and 64+ contiguous bytes per row. A slab = 128 tile columns (2 of each wave's 4 column blocks), kept transposed,
+    // S[col][row]: the accumulator layout (4 consecutive rows of one column per lane) writes it with 8-byte stores,
+    // row-major outputs come back out through ds_read_b64_tr_b16 (a lane ends up with 8 consecutive columns of one
+    // row), transposed outputs through plain 16-byte reads.
+    typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4;
+    constexpr int NT = 64 * NW;
+    constexpr int kSlabCols = 128, kSlabLd = BM + 4;  // 520-byte rows: 8-byte aligned and spread over the banks
+    T* slab = lds;                                    // the pipeline stages are dead by now
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave is done with the stages
+
+    // write this wave's blocks (i, jb..jb+1) of a value source into the slab
+    auto stage_blocks = [&](auto&& value /* (i, jj, q, s) -> T */) {
+      static_for<MI>([&](auto i) {
+        static_for<2>([&](auto jj) {
+          static_for<4>([&](auto q) {
+            const int r = wm * WM + i * 32 + 8 * q + row_quad;
+            const int c = wn * 64 + jj * 32 + col_in_block;
+            store4(slab + c * kSlabLd + r, value(i, jj, q, std::integral_constant<int, 0>{}),
+                   value(i, jj, q, std::integral_constant<int, 1>{}), value(i, jj, q, std::integral_constant<int, 2>{}),
+                   value(i, jj, q, std::integral_constant<int, 3>{}));
+          });
+        });
+      });
+    };
+    // slab column -> column of the block tile, for pass `pass` (which pair of each wave's column blocks is staged)
+    auto tile_col = [&](int sc, int pass) { return (sc >> 6) * WN + pass * 64 + (sc & 63); };
+    // row-major readout: out_ptr(row, tile column) must return the address of 8 consecutive output columns or nullptr
+    auto drain_rows = [&](auto&& out_ptr) {
+      const int l16 = tid & 15, grp = tid >> 4;
+      const int tq = l16 & 3, tj = l16 >> 2;  // as a source lane: which slab column this lane points at
+      const int oq = l16 >> 2, oe = l16 & 3;  // as a destination lane: 8 columns oq of row oe of the 4 x 32 block
+      constexpr int kBlocks = (BM / 4) * (kSlabCols / 32);
+#pragma unroll 4
+      for (int b = grp; b < kBlocks; b += NT / 16) {
+        const int rb = b >> 2, cb = b & 3;
+        const T* src = slab + (cb * 32 + 8 * tq + tj) * kSlabLd + rb * 4;
+        const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(src));
+        const s16x4 hi =
+            __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(src + 4 * kSlabLd));
+        T* dst = out_ptr(rb * 4 + oe, cb * 32 + 8 * oq);
+        if (dst != nullptr) {
+          vec16 v;
+          v.w[0] = (uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
+          v.w[1] = (uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
+          v.w[2] = (uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
+          v.w[3] = (uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16);
+          store16(dst, v);
+        }
+      }
+    };
+    // transposed readout: out_ptr(slab column, row) -> address of 8 consecutive rows of that column, or nullptr
+    auto drain_cols = [&](auto&& out_ptr) {
+      constexpr int kChunks = kSlabCols * (BM / 8);
+#pragma unroll 4
+      for (int ch = tid; ch < kChunks; ch += NT) {
+        const int c = ch / (BM / 8), r = (ch % (BM / 8)) * 8;
+        T* dst = out_ptr(c, r);
+        if (dst != nullptr) store16(dst, load16(slab + c * kSlabLd + r));
+      }
+    };
+    auto sync_slab = [&]() { __syncthreads(); };
+    const T kZero = Elem<T>::down(0.f);
+
+    if constexpr (MODE == kDw) {
+      T* dw = static_cast<T*>(prm.y) + (int64_t)expert * prm.M * prm.N;
+      static_for<2>([&](auto pass) {
+        stage_blocks([&](auto i, auto jj, auto q, auto sidx) { return Elem<T>::down(acc[i][pass * 2 + jj][4 * q + sidx]); });
+        sync_slab();
+        drain_rows([&](int r, int sc) -> T* {
+          const int64_t m = m0 + r, n = (int64_t)nt * BN + tile_col(sc, pass);
+          return (m < prm.M && n < prm.N) ? dw + m * prm.N + n : nullptr;
+        });
+        sync_slab();
+      });
+    } else if constexpr (MODE == kGrouped || MODE == kScatter) {
+      T* y = static_cast<T*>(prm.y);
+      T* y_t = static_cast<T*>(prm.y_t);
+      static_for<2>([&](auto pass) {
+        // pad rows are staged as zeros: the transposed copy must hold zeros there
+        stage_blocks([&](auto i, auto jj, auto q, auto sidx) {
+          const int64_t p = m0 + wm * WM + i * 32 + 8 * q + row_quad + sidx;
+          return p < valid_end ? Elem<T>::down(acc[i][pass * 2 + jj][4 * q + sidx]) : kZero;
+        });
+        sync_slab();
+        drain_rows([&](int r, int sc) -> T* {
+          const int64_t p = m0 + r, n = (int64_t)nt * BN + tile_col(sc, pass);
+          if (p >= valid_end || n >= prm.N) return nullptr;
+          const int64_t row = (MODE == kScatter) ? (int64_t)prm.row_slot[p] : p;
+          return y + row * prm.N + n;
+        });
+        if (MODE == kGrouped && y_t != nullptr) {
+          drain_cols([&](int sc, int r) -> T* {
+            const int64_t n = (int64_t)nt * BN + tile_col(sc, pass);
+            return n < prm.N ? y_t + n * prm.ld_t + m0 + r : nullptr;
+          });
+        }
+        sync_slab();
+      });
+    } else {  // kSwiglu: blocks j = 0, 1 are up, j = 2, 3 are gate of the same activation columns
+      T* pre = static_cast<T*>(prm.y);
+      T* act = static_cast<T*>(prm.aux);
+      T* act_t = static_cast<T*>(prm.y_t);
+      const int64_t two_i = 2 * (int64_t)prm.I;
+      // activation column of slab column sc (64 per wave column)
+      auto act_col = [&](int sc) { return (int64_t)nt * (BN / 2) + (sc >> 6) * (WN / 2) + (sc & 63); };
+      static_for<3>([&](auto pass) {  // 0: up half of the pre-activation, 1: gate half, 2: activation
+        stage_blocks([&](auto i, auto jj, auto q, auto sidx) {
+          const int64_t p = m0 + wm * WM + i * 32 + 8 * q + row_quad + sidx;
+          const T up = Elem<T>::down(acc[i][jj][4 * q + sidx]);
+          const T gate = Elem<T>::down(acc[i][jj + 2][4 * q + sidx]);
+          if (pass == 0) return up;
+          if (pass == 1) return gate;
+          const float gf = Elem<T>::up(gate);
+          return p < valid_end ? Elem<T>::down(Elem<T>::up(up) * gf * sigmoid_fast(gf)) : kZero;
+        });
+        sync_slab();
+        drain_rows([&](int r, int sc) -> T* {
+          const int64_t p = m0 + r, col = act_col(sc);
+          if (p >= valid_end || col >= prm.I) return nullptr;
+          if (pass == 0) return pre + p * two_i + col;
+          if (pass == 1) return pre + p * two_i + prm.I + col;
+          return act + p * prm.I + col;
+        });
+        if (pass == 2 && act_t != nullptr) {
+          drain_cols([&](int sc, int r) -> T* {
+            const int64_t col = act_col(sc);
+            return col < prm.I ? act_t + col * prm.ld_t + m0 + r : nullptr;
+          });
+        }
+        sync_slab();
+      });
+    }
+    return;
+  }
   if constexpr (MODE == kDw) {
     T* dw = static_cast<T*>(prm.y) + (int64_t)expert * prm.M * prm.N;
     static_for<MI>([&](auto i) {
@@ -586,9 +748,9 @@ constexpr size_t lds_bytes() {
   return PIPE == 0 ? (size_t)2 * (BM + BN) * kLdsStride * 2 : (size_t)4 * (BM + BN) * 32 * 2;
 }
 
-template <typename T, int BM, int BN, int MODE, int PIPE>
+template <typename T, int BM, int BN, int MODE, int PIPE, int WGM>
 int launch_pipe(const GemmParams& prm, unsigned blocks, hipStream_t s, const char* name) {
-  auto kernel = grouped_gemm_kernel<T, BM, BN, MODE, PIPE>;
+  auto kernel = grouped_gemm_kernel<T, BM, BN, MODE, PIPE, WGM>;
   static bool attr_set = false;  // per instantiation; the attribute is idempotent, a race only repeats the call
   if (!attr_set) {
     hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
@@ -600,7 +762,7 @@ int launch_pipe(const GemmParams& prm, unsigned blocks, hipStream_t s, const cha
     attr_set = true;
   }
   constexpr size_t kLds = lds_bytes<BM, BN, PIPE>();
-  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(kThreads), kLds, s, prm);
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(64 * WGM * 2), kLds, s, prm);
   CK_CHECK_LAUNCH(name);
   return CK_OK;
 }
@@ -609,8 +771,11 @@ int launch_pipe(const GemmParams& prm, unsigned blocks, hipStream_t s, const cha
 template <typename T, int BM, int BN, int MODE>
 int launch(const GemmParams& prm, unsigned blocks, hipStream_t s, const char* name) {
   const bool dma = (MODE == kDw) || (prm.K % 32 == 0);
-  if (dma && !g_force_pipe0) return launch_pipe<T, BM, BN, MODE, 1>(prm, blocks, s, name);
-  return launch_pipe<T, BM, BN, MODE, 0>(prm, blocks, s, name);
+  if (dma && !g_force_pipe0) {
+    if (g_eight_waves) return launch_pipe<T, BM, BN, MODE, 1, 4>(prm, blocks, s, name);
+    return launch_pipe<T, BM, BN, MODE, 1, 2>(prm, blocks, s, name);
+  }
+  return launch_pipe<T, BM, BN, MODE, 0, 2>(prm, blocks, s, name);
 }
 
 template <typename T, int MODE>

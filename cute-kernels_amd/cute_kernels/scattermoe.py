@@ -124,8 +124,10 @@ class ExpertSegments:
 
 
 def choose_align(num_rows: int, num_experts: int) -> int:
-    """Tile height of the padded layout: 256-row tiles once experts average at least 2048 rows, else 128."""
-    return 256 if num_rows >= 2048 * num_experts else 128
+    """Tile height of the padded layout: 256-row tiles once experts average at least 512 rows (measured at the
+    fine-grained shape, 1024 rows per expert: 256-row tiles run the forward GEMMs 30 % faster than 128-row ones despite
+    the extra padding), else 128."""
+    return 256 if num_rows >= 512 * num_experts else 128
 
 
 @torch.no_grad()
