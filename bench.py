@@ -125,6 +125,7 @@ def secondary_hbm_kernels(dev):
     def timed(fn, iters=20):
         for _ in range(3):
             fn()
+        torch.cuda.synchronize()
         s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         s.record()
         for _ in range(iters):
@@ -154,15 +155,29 @@ def secondary_hbm_kernels(dev):
         b = 4 * n + 8 * 64 + 4 * 64
         out[f"count_offsets_N{n}_E64"] = {"us": dt * 1e6, "GB/s": b / dt / 1e9, "frac_hbm": b / dt / 1e9 / PEAK_HBM_GBS}
         del ids
-    # C2 routing bookkeeping: logits [16384, 64] bf16, top-2 -> ids, gates, sort, offsets
-    logits = torch.randn(16384, 64, generator=g).to(torch.bfloat16).to(dev)
+    # C2 routing bookkeeping: logits [16384, 64] bf16, top-2 -> ids, gates, stable sort, counts / offsets.
+    # Straight through the C ABI with caller-owned outputs (three launches: route, sort histogram + scan, sort scatter).
+    Tr, Er, kr = 16384, 64, 2
+    Rr = Tr * kr
+    logits = torch.randn(Tr, Er, generator=g).to(torch.bfloat16).to(dev)
+    i32 = dict(dtype=torch.int32, device=dev)
+    sel, gates = torch.empty(Tr, kr, **i32), torch.empty(Tr, kr, dtype=torch.float32, device=dev)
+    max_rows = lib.ck_sort_max_rows(Rr, Er, 128)
+    se, ss = torch.empty(Rr, **i32), torch.empty(Rr, **i32)
+    cnt, en, st = (torch.empty(Er, dtype=torch.uint32, device=dev) for _ in range(3))
+    seg_starts, row_slot, tile_expert = torch.empty(Er + 1, **i32), torch.empty(max_rows, **i32), torch.empty(max_rows // 128, **i32)
+    ws2 = torch.zeros(lib.ck_sort_workspace_words(Rr, Er), **i32)
+    stream = torch.cuda.current_stream().cuda_stream
 
     def routing():
-        sel, gates, _ = cute_kernels.route_topk_softmax_raw(logits, 2)
-        cute_kernels.sort_by_expert(sel, 64)
+        _C.check(lib.ck_route_topk_softmax(logits.data_ptr(), _C.CK_BF16, Tr, Er, kr, sel.data_ptr(), gates.data_ptr(), None, stream))
+        _C.check(lib.ck_sort_by_expert(sel.data_ptr(), 0, Rr, Er, 128, se.data_ptr(), ss.data_ptr(), cnt.data_ptr(), en.data_ptr(),
+                                       st.data_ptr(), seg_starts.data_ptr(), row_slot.data_ptr(), tile_expert.data_ptr(),
+                                       ws2.data_ptr(), stream))
 
-    dt = timed(routing)
-    b = 2 * 16384 * 64 + 4 * 4 * 32768 + 8 * 64
+    dt = timed(routing, iters=200)
+    assert int(en[-1]) == Rr
+    b = 2 * Tr * Er + 4 * 4 * Rr + 8 * Er
     out["route_sort_C2"] = {"us": dt * 1e6, "GB/s": b / dt / 1e9, "frac_hbm": b / dt / 1e9 / PEAK_HBM_GBS}
     # row gather / gated combine at the C3 shape
     R = T * TOP_K

@@ -195,10 +195,15 @@ __global__ __launch_bounds__(kBlock) void count_kernel(const id_t* __restrict__ 
     for (int e = t; e < num_bins; e += kBlock)
       if (hist[e]) atomicAdd(&my_acc[e], hist[e]);
     if (!last_block_ticket<false>(ws, tmp + kWavesPerBlock)) return;
-    for (int e = t; e < num_bins; e += kBlock) {
-      uint32_t s = 0;
-      for (int r = 0; r < replicas; ++r) s += atomicExch(&acc[(size_t)r * num_bins + e], 0u);  // read, restore the zero
-      hist[e] = s;
+    // Sum the replicas that were used and put them back to zero. Device-scope atomic loads read the values where the
+    // other blocks' atomics left them; the loads of one thread are independent, so their latencies overlap.
+    const int used = min(replicas, (int)gridDim.x);
+    for (int e = t; e < num_bins; e += kBlock) hist[e] = 0;
+    __syncthreads();
+    for (int idx = t; idx < used * num_bins; idx += kBlock) {  // (replica, bin) pairs spread over the whole block
+      const uint32_t v = __hip_atomic_load(&acc[idx], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      acc[idx] = 0u;  // visible to the next launch at the kernel boundary; nobody reads it before
+      if (v) atomicAdd(&hist[idx % num_bins], v);
     }
     if (t == 0) ws[0] = 0u;
     __syncthreads();
