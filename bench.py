@@ -191,6 +191,47 @@ def secondary_hbm_kernels(dev):
     dt = timed(lambda: scattermoe._combine(expanded, gates, T, TOP_K, H))
     b = R * H * 2 + T * H * 2 + 2 * R
     out["combine_rows_C3"] = {"us": dt * 1e6, "GB/s": b / dt / 1e9, "frac_hbm": b / dt / 1e9 / PEAK_HBM_GBS}
+    del src, idx, expanded, gates
+
+    # stand-alone SwiGLU (packed, C3 rows x 2I) and RMSNorm (C5 rows: 65,536 x 4,096), forward and backward
+    def rec(name, dt, b):
+        out[name] = {"us": dt * 1e6, "GB/s": b / dt / 1e9, "frac_hbm": b / dt / 1e9 / PEAK_HBM_GBS}
+
+    xp = torch.randn(R, 2 * I, device=dev, dtype=torch.bfloat16, requires_grad=True)
+    rec("swiglu_packed_fwd_C3", timed(lambda: cute_kernels.swiglu_packed_cute(xp.detach())), 3 * R * I * 2)
+    yp = cute_kernels.swiglu_packed_cute(xp)
+    gy = torch.randn_like(yp)
+    rec("swiglu_packed_bwd_C3", timed(lambda: torch.autograd.grad(yp, xp, gy, retain_graph=True)), 5 * R * I * 2)
+    del xp, yp, gy
+    Bn, Hn = 65536, 4096
+    xn = torch.randn(Bn, Hn, device=dev, dtype=torch.bfloat16, requires_grad=True)
+    wn = torch.ones(Hn, device=dev, dtype=torch.bfloat16, requires_grad=True)
+    rec("rmsnorm_fwd_C5", timed(lambda: cute_kernels.rmsnorm_cute(xn.detach(), wn.detach(), 1e-6)), 2 * Bn * Hn * 2 + 4 * Bn)
+    yn = cute_kernels.rmsnorm_cute(xn, wn, 1e-6)
+    gn = torch.randn_like(yn)
+    rec("rmsnorm_bwd_C5", timed(lambda: torch.autograd.grad(yn, (xn, wn), gn, retain_graph=True)), 3 * Bn * Hn * 2 + 4 * Bn)
+    del xn, wn, yn, gn
+    torch.cuda.empty_cache()
+
+    # C4: fine-grained MoE fwd+bwd behind an RMSNorm prologue (T=8192, H=2048, E=64, top-8, I=1408, uniform routing)
+    T4, H4, E4, K4, I4 = 8192, 2048, 64, 8, 1408
+    torch.manual_seed(SEED)
+    moe4 = cute_kernels.MoE(E4, K4, H4, I4, cute_kernels.swiglu_packed_cute, True, False, 0.02).to(torch.bfloat16).to(dev)
+    w4 = (1 + 0.02 * torch.randn(H4, device=dev)).to(torch.bfloat16).requires_grad_()
+    x4 = torch.randn(T4, H4, device=dev, dtype=torch.bfloat16, requires_grad=True)
+    g4 = torch.randn(T4, H4, device=dev, dtype=torch.bfloat16)
+
+    def step4():
+        for p_ in moe4.parameters():
+            p_.grad = None
+        x4.grad = None
+        w4.grad = None
+        y4, _ = moe4(cute_kernels.rmsnorm_cute(x4, w4, 1e-6))
+        y4.backward(g4)
+
+    dt = timed(step4, iters=10)
+    f4 = 18.0 * T4 * K4 * H4 * I4
+    out["C4_moe_fwd_bwd"] = {"ms": dt * 1e3, "TFLOP/s": f4 / dt / 1e12, "frac_mfma": f4 / dt / 1e12 / PEAK_BF16_TFLOPS}
     return out
 
 

@@ -1,0 +1,101 @@
+// Pieces shared by the grouped GEMM kernels (bf16 / f16 in grouped_gemm.hip, fp8 e4m3 in grouped_gemm_fp8.hip).
+#pragma once
+
+#include <type_traits>
+
+#include "ck_common.h"
+
+namespace ck {
+namespace {
+
+constexpr int kXcds = 8;
+
+enum Mode { kGrouped = CK_EPI_GROUPED, kScatter = CK_EPI_SCATTER, kSwiglu = CK_EPI_SWIGLU, kSwigluBwd = CK_EPI_SWIGLU_BWD, kDw = 4 };
+
+struct GemmParams {
+  const void* a;      // forward modes: [*, K]; dW: a_t [M, ld_t]
+  const void* w;      // forward modes: [E, N, K]; dW: b_t [N, ld_t]
+  int64_t lda;        // row stride of a (elements)
+  int64_t ldw;        // row stride of w (elements)
+  int64_t w_expert_stride;
+  int a_gather_div;   // > 0: A row p comes from a[row_slot[p] / div]
+  int M;              // dW only: rows of a_t
+  int N;              // output columns of the GEMM (2I for kSwiglu)
+  int K;              // contraction length (forward modes)
+  int I;              // kSwiglu / kSwigluBwd: intermediate size
+  int n_tiles;        // tiles along N
+  int m_tiles;        // dW only: tiles along M
+  int align;          // rows per M tile (== BM) in the padded layout
+  int num_experts;
+  const int32_t* seg_starts;
+  const uint32_t* counts;
+  const int32_t* tile_expert;
+  const int32_t* row_slot;
+  void* y;
+  void* y_t;
+  int64_t ld_t;
+  void* aux;
+  const void* aux_in;
+  const float* a_scale;  // fp8 only: per-row dequantisation scale of a (indexed like the rows of a)
+  const float* w_scale;  // fp8 only: per-output-channel scale of w, [E, N]
+};
+
+// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant expression
+template <int N, typename F>
+__device__ inline void static_for(F&& f) {
+  if constexpr (N > 0) {
+    static_for<N - 1>(f);
+    f(std::integral_constant<int, N - 1>{});
+  }
+}
+
+template <typename T>
+__device__ inline uint16_t bits16(T v) {
+  union {
+    T t;
+    uint16_t u;
+  } c;
+  c.t = v;
+  return c.u;
+}
+
+// 4 consecutive 16-bit values as one 8-byte store
+template <typename T>
+__device__ inline void store4(T* p, T v0, T v1, T v2, T v3) {
+  uint2 u;
+  u.x = (uint32_t)bits16(v0) | ((uint32_t)bits16(v1) << 16);
+  u.y = (uint32_t)bits16(v2) | ((uint32_t)bits16(v3) << 16);
+  *reinterpret_cast<uint2*>(p) = u;
+}
+
+// Tile order inside a run of tiles: groups of 8 along `a` (the side with a_count tiles), then `b`, with `a` fastest
+// inside a group -- 32 consecutive tiles form an 8 x 4 block that shares 8 + 4 operand panels.
+__device__ inline void grouped_order(int r, int a_count, int b_count, int& a, int& b) {
+  constexpr int GROUP = 8;
+  const int group_sz = GROUP * b_count;
+  const int g = r / group_sz;
+  const int first = g * GROUP;
+  const int in_group = min(GROUP, a_count - first);
+  const int q = r - g * group_sz;
+  b = q / in_group;
+  a = first + (q - b * in_group);
+}
+
+
+// XOR swizzle of the 64-byte LDS rows of the direct-to-LDS pipeline: 16-byte chunk c of row r sits in slot
+// c ^ lds_swizzle(r). Found by exhaustive search: fragment reads (32 consecutive rows, same chunk) are free of bank
+// conflicts both for 8 lanes over 32 banks and for 16 lanes over 64 banks.
+__device__ inline int lds_swizzle(int row) { return ((row >> 2) & 1) | ((((row >> 1) ^ (row >> 3)) & 1) << 1); }
+
+inline int check_segments(const ck_segments* seg, const char* name) {
+  CK_REQUIRE(seg != nullptr, "%s: seg is NULL", name);
+  CK_REQUIRE(seg->seg_starts && seg->counts && seg->tile_expert && seg->row_slot, "%s: NULL table in seg", name);
+  CK_REQUIRE(seg->align == 128 || seg->align == 256, "%s: align=%d must be 128 or 256", name, seg->align);
+  CK_REQUIRE(seg->num_experts >= 1, "%s: num_experts=%d", name, seg->num_experts);
+  CK_REQUIRE(seg->max_rows >= 0 && seg->max_rows % seg->align == 0, "%s: max_rows=%lld is not a multiple of align", name,
+             (long long)seg->max_rows);
+  return CK_OK;
+}
+
+}  // namespace
+}  // namespace ck

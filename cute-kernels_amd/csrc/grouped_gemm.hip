@@ -10,9 +10,7 @@
 // loads of step k+1 are in flight while step k is multiplied.
 #include <stdlib.h>
 
-#include <type_traits>
-
-#include "ck_common.h"
+#include "gemm_common.h"
 
 namespace ck {
 namespace {
@@ -21,9 +19,7 @@ constexpr int kThreads = 256;
 constexpr int BK = 64;            // K elements per stage
 constexpr int kLdsStride = 72;    // elements per LDS row (64 + 8 pad)
 constexpr int kChunksPerRow = 8;  // 16-byte chunks per 64-element row
-constexpr int kXcds = 8;
 
-enum Mode { kGrouped = CK_EPI_GROUPED, kScatter = CK_EPI_SCATTER, kSwiglu = CK_EPI_SWIGLU, kSwigluBwd = CK_EPI_SWIGLU_BWD, kDw = 4 };
 
 template <typename T>
 struct Mfma;
@@ -57,73 +53,6 @@ const bool g_eight_waves = [] {
   const char* env = getenv("CK_GEMM_WAVES");
   return !(env != nullptr && env[0] == '4');
 }();
-
-struct GemmParams {
-  const void* a;      // forward modes: [*, K]; dW: a_t [M, ld_t]
-  const void* w;      // forward modes: [E, N, K]; dW: b_t [N, ld_t]
-  int64_t lda;        // row stride of a (elements)
-  int64_t ldw;        // row stride of w (elements)
-  int64_t w_expert_stride;
-  int a_gather_div;   // > 0: A row p comes from a[row_slot[p] / div]
-  int M;              // dW only: rows of a_t
-  int N;              // output columns of the GEMM (2I for kSwiglu)
-  int K;              // contraction length (forward modes)
-  int I;              // kSwiglu / kSwigluBwd: intermediate size
-  int n_tiles;        // tiles along N
-  int m_tiles;        // dW only: tiles along M
-  int align;          // rows per M tile (== BM) in the padded layout
-  int num_experts;
-  const int32_t* seg_starts;
-  const uint32_t* counts;
-  const int32_t* tile_expert;
-  const int32_t* row_slot;
-  void* y;
-  void* y_t;
-  int64_t ld_t;
-  void* aux;
-  const void* aux_in;
-};
-
-// f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant expression
-template <int N, typename F>
-__device__ inline void static_for(F&& f) {
-  if constexpr (N > 0) {
-    static_for<N - 1>(f);
-    f(std::integral_constant<int, N - 1>{});
-  }
-}
-
-template <typename T>
-__device__ inline uint16_t bits16(T v) {
-  union {
-    T t;
-    uint16_t u;
-  } c;
-  c.t = v;
-  return c.u;
-}
-
-// 4 consecutive 16-bit values as one 8-byte store
-template <typename T>
-__device__ inline void store4(T* p, T v0, T v1, T v2, T v3) {
-  uint2 u;
-  u.x = (uint32_t)bits16(v0) | ((uint32_t)bits16(v1) << 16);
-  u.y = (uint32_t)bits16(v2) | ((uint32_t)bits16(v3) << 16);
-  *reinterpret_cast<uint2*>(p) = u;
-}
-
-// Tile order inside a run of tiles: groups of 8 along `a` (the side with a_count tiles), then `b`, with `a` fastest
-// inside a group -- 32 consecutive tiles form an 8 x 4 block that shares 8 + 4 operand panels.
-__device__ inline void grouped_order(int r, int a_count, int b_count, int& a, int& b) {
-  constexpr int GROUP = 8;
-  const int group_sz = GROUP * b_count;
-  const int g = r / group_sz;
-  const int first = g * GROUP;
-  const int in_group = min(GROUP, a_count - first);
-  const int q = r - g * group_sz;
-  b = q / in_group;
-  a = first + (q - b * in_group);
-}
 
 // PIPE 0: K step 64, global -> registers -> padded LDS, two stages (any K % 8 == 0).
 // PIPE 1: K step 32, global -> LDS directly (no register staging), four XOR-swizzled stages, loads three steps ahead
@@ -353,7 +282,7 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
     static_assert(A_LD >= 1 && B_LD >= 1, "tile too small for this many waves");
     constexpr int kStageBytes = (BM + BN) * BK1 * 2;
     constexpr int kRowBytes = BK1 * 2;  // 64 B = 4 chunks; chunk c of row r sits in slot c ^ swz(r)
-    auto swz = [](int row) { return ((row >> 2) & 1) | ((((row >> 1) ^ (row >> 3)) & 1) << 1); };
+    auto swz = [](int row) { return lds_swizzle(row); };
     char* lds_c = reinterpret_cast<char*>(lds_raw);
     const char* a_base = static_cast<const char*>(prm.a);
     const char* b_base = static_cast<const char*>(prm.w);
@@ -783,16 +712,6 @@ int launch_by_tile(const GemmParams& prm, int align, unsigned blocks_256, unsign
                    const char* name) {
   if (align == 256) return launch<T, 256, 256, MODE>(prm, blocks_256, s, name);
   return launch<T, 128, 128, MODE>(prm, blocks_128, s, name);
-}
-
-int check_segments(const ck_segments* seg, const char* name) {
-  CK_REQUIRE(seg != nullptr, "%s: seg is NULL", name);
-  CK_REQUIRE(seg->seg_starts && seg->counts && seg->tile_expert && seg->row_slot, "%s: NULL table in seg", name);
-  CK_REQUIRE(seg->align == 128 || seg->align == 256, "%s: align=%d must be 128 or 256", name, seg->align);
-  CK_REQUIRE(seg->num_experts >= 1, "%s: num_experts=%d", name, seg->num_experts);
-  CK_REQUIRE(seg->max_rows >= 0 && seg->max_rows % seg->align == 0, "%s: max_rows=%lld is not a multiple of align", name,
-             (long long)seg->max_rows);
-  return CK_OK;
 }
 
 }  // namespace

@@ -232,13 +232,25 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const T* __restrict
   }
 }
 
+// d_weight[h] = sum over the partial rows, in a fixed order. A block owns 64 columns; its 4 waves each sum a quarter of
+// the rows (reads are 256-byte coalesced), then the quarters are added through LDS.
 __global__ __launch_bounds__(kBlock) void rmsnorm_dw_reduce_kernel(const float* __restrict__ partial, int64_t workers,
                                                                     int H, float* __restrict__ d_weight) {
-  const int h = blockIdx.x * kBlock + threadIdx.x;
-  if (h >= H) return;
+  __shared__ float part[kBlock / kWave][kWave];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int h = blockIdx.x * kWave + lane;
   float s = 0.f;
-  for (int64_t w = 0; w < workers; ++w) s += partial[w * H + h];
-  d_weight[h] = s;
+  if (h < H) {
+    for (int64_t w = wave; w < workers; w += kBlock / kWave) s += partial[w * H + h];
+  }
+  part[wave][lane] = s;
+  __syncthreads();
+  if (wave == 0 && h < H) {
+    float t = 0.f;
+#pragma unroll
+    for (int g = 0; g < kBlock / kWave; ++g) t += part[g][lane];
+    d_weight[h] = t;
+  }
 }
 
 constexpr int64_t kMaxWorkers = 2048;
@@ -339,7 +351,7 @@ extern "C" int ck_rmsnorm_bwd(const void* x, const void* weight, const void* d_o
              "ck_rmsnorm_bwd: weight, d_weight and d_weight_partial must be given together");
   if (B == 0) {
     if (d_weight != nullptr) {  // no rows: the sum over zero partial rows is zero
-      hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3((unsigned)ceil_div(H, kBlock)), dim3(kBlock), 0,
+      hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3((unsigned)ceil_div(H, kWave)), dim3(kBlock), 0,
                          static_cast<hipStream_t>(stream), d_weight_partial, (int64_t)0, (int)H, d_weight);
       CK_CHECK_LAUNCH("ck_rmsnorm_bwd");
     }
@@ -355,7 +367,7 @@ extern "C" int ck_rmsnorm_bwd(const void* x, const void* weight, const void* d_o
     const int64_t blocks = workers / rows_per_block;
     CK_RMS_DISPATCH(CK_RMS_BWD, 0);
     if (d_weight != nullptr) {
-      hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3((unsigned)ceil_div(H, kBlock)), dim3(kBlock), 0, s,
+      hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3((unsigned)ceil_div(H, kWave)), dim3(kBlock), 0, s,
                          d_weight_partial, workers, (int)H, d_weight);
     }
   });

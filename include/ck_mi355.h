@@ -172,6 +172,24 @@ int ck_grouped_gemm_dw(const void* a_t, const void* b_t, int64_t ld_t, int32_t M
                        void* dw, int32_t dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------------------------------
+ * (c, fp8) quantised-expert forward path: e4m3 operands (OCP e4m3fn, the gfx950 format), fp32 accumulation
+ * No counterpart in the reference (it has no fp8 code): the semantics are those of the same layer evaluated on the
+ * de-quantised operands, cute_kernels/kernels/scattermoe/torch_implementation.py:137-169.
+ * ------------------------------------------------------------------------------------------------------------- */
+/* Per-row quantisation: scales[r] = max|x[r, :]| / 448 (1 for an all-zero row), q[r, c] = e4m3(x[r, c] * (448 / max)),
+ * round to nearest even. x [rows, cols] bf16 / f16, q [rows, cols] bytes, cols % 16 == 0. Used per token for
+ * activations and per output channel ([E * out, in] rows) for expert weights. */
+int ck_quant_rows_e4m3(const void* x, int64_t rows, int32_t cols, void* q, float* scales, int32_t dtype, void* stream);
+/* Y = (A_e * diag(a_scale)) * (W[e] * diag(w_scale[e]))^T over tile-aligned expert segments (align must be 256).
+ * a8: e4m3 rows [*, K], gathered like ck_grouped_gemm (a_gather_div); a_scale is indexed by the row of a8 that is read.
+ * w8 [E, N, K] e4m3, w_scale [E, N]. K % 64 == 0. Epilogues: CK_EPI_GROUPED (y [max_rows, N]), CK_EPI_SCATTER
+ * (y [R, N]), CK_EPI_SWIGLU (N = 2I packed [up | gate]; only the activation is written, to aux [max_rows, I]).
+ * Outputs have `out_dtype` (bf16 / f16). */
+int ck_grouped_gemm_fp8(const void* a8, const float* a_scale, int32_t a_gather_div, const void* w8,
+                        const float* w_scale, int32_t N, int32_t K, const ck_segments* seg, int32_t epilogue, void* y,
+                        void* aux, int32_t out_dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------------
  * SwiGLU, stand-alone
  * Replaces: swiglu_forward_cuda / swiglu_backward_cuda -- cute_kernels/kernels/swiglu/cuda_implementation/ops.cpp:7-22,
  *           forward.cu:18-94, backward.cu:18-129 (and the strided Triton variants used for the packed form).

@@ -124,3 +124,43 @@ class MoEOracle(nn.Module):
         hidden_states = hidden_states * batch_gates.unsqueeze(-1)                 # :163
         zeros = torch.zeros((total_q, self.hidden_size), dtype=hidden_states.dtype, device=hidden_states.device)
         return zeros.index_add(0, fan_in_index, hidden_states)                    # :164-165
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# fp8 (e4m3) quantised-expert forward. The reference has NO fp8 code or tests: PARITY UNPINNED upstream. This is the
+# specification this build gives itself: the reference layer (torch_implementation.py:137-169) evaluated on
+# de-quantised operands, with the roundings a 16-bit tensor between the two expert linears implies.
+# ---------------------------------------------------------------------------------------------------------------
+E4M3_MAX = 448.0
+
+
+def quantize_rows_e4m3_torch(x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """q = e4m3fn(x * (448 / amax_row)) (round to nearest even), scale = amax_row / 448 (1 for an all-zero row)."""
+    xf = x.float()
+    amax = xf.abs().amax(dim=-1, keepdim=True)
+    nz = amax > 0
+    inv = torch.where(nz, torch.tensor(E4M3_MAX) / amax, torch.ones_like(amax))
+    scale = torch.where(nz, amax / torch.tensor(E4M3_MAX), torch.ones_like(amax))
+    return (xf * inv).to(torch.float8_e4m3fn), scale.squeeze(-1)
+
+
+def moe_e4m3_forward_oracle(moe: "MoEOracle", x: torch.Tensor, selected: torch.Tensor, gates: torch.Tensor) -> torch.Tensor:
+    """Packed-SwiGLU MoE forward with e4m3 operands, per token; x [T, H] in a 16-bit dtype, gates in x.dtype."""
+    dt = x.dtype
+    w1q, w1s = quantize_rows_e4m3_torch(moe.c_fc.weight.detach().flatten(0, 1))
+    w2q, w2s = quantize_rows_e4m3_torch(moe.c_proj.weight.detach().flatten(0, 1))
+    E = moe.num_experts
+    w1 = (w1q.float() * w1s[:, None]).view(E, -1, x.size(-1))
+    w2 = (w2q.float() * w2s[:, None]).view(E, x.size(-1), -1)
+    xq, xs = quantize_rows_e4m3_torch(x)
+    xd = xq.float() * xs[:, None]
+    out = torch.zeros(x.shape, dtype=torch.float32)
+    for t in range(x.size(0)):
+        for j in range(selected.size(1)):
+            e = int(selected[t, j])
+            pre = (w1[e] @ xd[t]).to(dt)  # the pre-activation a 16-bit tensor would hold
+            act = swiglu_packed_torch(pre)
+            aq, a_s = quantize_rows_e4m3_torch(act[None])
+            y = (w2[e] @ (aq.float()[0] * a_s)).to(dt)
+            out[t] += gates[t, j].float() * y.float()
+    return out.to(dt)

@@ -1,0 +1,117 @@
+"""GPU parity for the fp8 (e4m3) quantised-expert forward path, through the C ABI.
+
+The reference has no fp8 code: parity is UNPINNED upstream. These tests check the kernels against the specification in
+oracle/moe_oracle.py (the reference layer on de-quantised operands). Quantisation is bit-exact; GEMM results are held to
+rtol 5e-2 / atol 5e-2 on 16-bit outputs (stated tolerance for fp8; e4m3 carries 3 mantissa bits = 6 % steps)."""
+
+import numpy as np
+import pytest
+import torch
+
+import cute_kernels
+from cute_kernels import _C, fp8
+from oracle import moe_oracle as mo
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("rows,cols", [(1, 16), (37, 64), (300, 4096), (5, 1536)])
+def test_quantize_rows_is_bit_exact(device, dtype, rows, cols):
+    g = torch.Generator().manual_seed(rows + cols)
+    x = (torch.randn(rows, cols, generator=g) * 3).to(dtype)
+    x[0, : min(cols, 16)] = 0  # zeros inside a row
+    if rows > 2:
+        x[2] = 0  # an all-zero row: scale 1, q 0
+    q, scale = cute_kernels.quantize_rows_e4m3(x.to(device))
+    oq, oscale = mo.quantize_rows_e4m3_torch(x)
+    assert q.dtype == torch.float8_e4m3fn and scale.dtype == torch.float32
+    assert torch.equal(scale.cpu(), oscale)
+    assert torch.equal(q.cpu().view(torch.uint8), oq.view(torch.uint8))
+    # round trip: within half an e4m3 step of the row maximum
+    back = q.cpu().float() * scale.cpu()[:, None]
+    assert float((back - x.float()).abs().max()) <= float(x.float().abs().max()) * 2.0**-4 + 1e-6
+
+
+def _segments(device, T, k, E, seed, empty=()):
+    g = torch.Generator().manual_seed(seed)
+    ids = torch.randint(0, E, (T * k,), generator=g, dtype=torch.int32)
+    for e in empty:
+        ids[ids == e] = 0
+    return g, ids, cute_kernels.sort_by_expert(ids.to(device), E, 256)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("K,N", [(64, 128), (256, 264), (1024, 512)])
+def test_grouped_gemm_fp8_grouped_and_scatter(device, dtype, K, N):
+    T, k, E = 300, 2, 5
+    g, ids, seg = _segments(device, T, k, E, seed=K + N, empty=(3,))
+    x = torch.randn(T, K, generator=g).to(dtype)
+    w = (0.1 * torch.randn(E, N, K, generator=g)).to(dtype)
+    x8, xs = cute_kernels.quantize_rows_e4m3(x.to(device))
+    w8, ws = cute_kernels.quantize_expert_weights_e4m3(w.to(device))
+    xd = x8.cpu().float() * xs.cpu()[:, None]
+    wd = w8.cpu().float() * ws.cpu()[:, :, None]
+    seg_starts, counts, row_slot = seg.seg_starts.cpu().numpy(), seg.counts.cpu().numpy(), seg.row_slot.cpu().numpy()
+
+    y = torch.zeros(seg.max_rows, N, dtype=dtype, device=device)
+    fp8._gemm_fp8(x8, xs, k, w8, ws, seg, _C.CK_EPI_GROUPED, y, None, dtype)
+    expect = torch.zeros(seg.max_rows, N)
+    for e in range(E):
+        s, c = int(seg_starts[e]), int(counts[e])
+        if c:
+            rows = torch.stack([xd[int(row_slot[p]) // k] for p in range(s, s + c)])
+            expect[s : s + c] = rows @ wd[e].t()
+    live = int(seg_starts[E])
+    torch.testing.assert_close(y.float().cpu()[:live], expect[:live], rtol=1e-2, atol=1e-2)  # same operands: tight
+
+    # grouped-in / scatter-out with the grouped result re-quantised per row
+    a = torch.randn(seg.max_rows, K, generator=g).to(dtype)
+    a8, a_s = cute_kernels.quantize_rows_e4m3(a.to(device))
+    ad = a8.cpu().float() * a_s.cpu()[:, None]
+    out = torch.full((T * k, N), float("nan"), dtype=dtype, device=device)
+    fp8._gemm_fp8(a8, a_s, 0, w8, ws, seg, _C.CK_EPI_SCATTER, out, None, dtype)
+    expect2 = torch.zeros(T * k, N)
+    for e in range(E):
+        for p in range(int(seg_starts[e]), int(seg_starts[e]) + int(counts[e])):
+            expect2[int(row_slot[p])] = wd[e] @ ad[p]
+    assert not torch.isnan(out.float()).any()
+    torch.testing.assert_close(out.float().cpu(), expect2, rtol=1e-2, atol=1e-2)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,E,k,H,I", [(257, 8, 2, 128, 256), (33, 4, 4, 64, 192), (700, 16, 8, 256, 320)])
+def test_moe_e4m3_layer_forward(device, dtype, T, E, k, H, I):
+    torch.manual_seed(E + k)
+    moe = cute_kernels.MoE(E, k, H, I, cute_kernels.swiglu_packed_cute, True, False, 0.02).to(dtype)
+    oracle = mo.MoEOracle(E, k, H, I, mo.swiglu_packed_torch, True, False, 0.02).to(dtype)
+    oracle.load_state_dict(moe.state_dict())
+    q = cute_kernels.MoE_E4M3(moe.to(device))
+    x = torch.randn(T, H).to(dtype)
+    y, logits = q(x.to(device))
+    assert y.shape == x.shape and y.dtype == dtype and logits.shape == (T, E)
+    # route the oracle as the GPU did; gates from its own logits
+    sel = cute_kernels.route_topk_softmax_raw(logits, k)[0].long().cpu()
+    lo = oracle.gate(x)
+    gates = torch.softmax(lo.gather(-1, sel).float(), dim=-1).to(dtype)
+    expect = mo.moe_e4m3_forward_oracle(oracle, x, sel, gates)
+    # stated fp8 tolerance: rtol 5e-2 / atol 5e-2 (here far inside it: both sides quantise identically)
+    torch.testing.assert_close(y.float().cpu(), expect.float(), rtol=5e-2, atol=5e-2)
+    # and fp8 stays close to the 16-bit layer itself
+    with torch.no_grad():
+        y16, _ = moe(x.to(device))
+    rel = float((y.float() - y16.float()).norm() / y16.float().norm())
+    assert rel < 0.08, rel
+
+
+def test_fp8_rejects_unsupported(device):
+    g, ids, seg128 = None, None, cute_kernels.sort_by_expert(torch.zeros(64, dtype=torch.int32, device=device), 2, 128)
+    x8 = torch.zeros(64, 64, dtype=torch.float8_e4m3fn, device=device)
+    s = torch.ones(64, device=device)
+    w8 = torch.zeros(2, 64, 64, dtype=torch.float8_e4m3fn, device=device)
+    ws = torch.ones(2, 64, device=device)
+    y = torch.zeros(seg128.max_rows, 64, dtype=torch.bfloat16, device=device)
+    with pytest.raises(RuntimeError, match="256"):
+        fp8._gemm_fp8(x8, s, 1, w8, ws, seg128, _C.CK_EPI_GROUPED, y, None, torch.bfloat16)
+    with pytest.raises(RuntimeError, match="multiple of 16"):
+        _C.check(_C.lib().ck_quant_rows_e4m3(1, 4, 24, 1, 1, _C.CK_BF16, None))
