@@ -22,6 +22,7 @@ for _p in (ROOT, os.path.join(ROOT, "cute-kernels_amd")):
     if _p not in sys.path:
         sys.path.insert(0, _p)
 
+PEAK_FP8_TFLOPS = 5000.0
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E
 
@@ -232,6 +233,43 @@ def secondary_hbm_kernels(dev):
     dt = timed(step4, iters=10)
     f4 = 18.0 * T4 * K4 * H4 * I4
     out["C4_moe_fwd_bwd"] = {"ms": dt * 1e3, "TFLOP/s": f4 / dt / 1e12, "frac_mfma": f4 / dt / 1e12 / PEAK_BF16_TFLOPS}
+    del moe4, w4, x4, g4
+    torch.cuda.empty_cache()
+
+    # C5: quantised-expert forward (e4m3 weights, per-channel scales; activations e4m3 per token) behind an RMSNorm
+    # prologue: T=65,536, H=4,096, E=128, top-8, I=1,536, Zipf(0.8) load, forward only
+    T5, H5, E5, K5, I5 = 65536, 4096, 128, 8, 1536
+    torch.manual_seed(SEED)
+    moe5 = cute_kernels.MoE(E5, K5, H5, I5, cute_kernels.swiglu_packed_cute, True, False, 0.02).to(torch.bfloat16).to(dev)
+    x5 = torch.randn(T5, H5, device=dev, dtype=torch.bfloat16)
+    w5 = (1 + 0.02 * torch.randn(H5, device=dev)).to(torch.bfloat16)
+    with torch.no_grad():
+        bias5, freq5, c5 = zipf_bias(moe5.gate(cute_kernels.rmsnorm_cute(x5[:16384], w5, 1e-6)), K5, 0.8)
+    bias5 = bias5.to(torch.bfloat16)
+    moe5.gate.register_forward_hook(lambda mod, inp, o: o + bias5)
+    q5 = cute_kernels.MoE_E4M3(moe5)
+    moe5.c_fc.weight.data = torch.empty(0, device=dev)  # the 16-bit expert weights are not part of the fp8 layer
+    moe5.c_proj.weight.data = torch.empty(0, device=dev)
+    torch.cuda.empty_cache()
+
+    def step5():
+        with torch.no_grad():
+            q5(cute_kernels.rmsnorm_cute(x5, w5, 1e-6))
+
+    dt = timed(step5, iters=5)
+    timer = scattermoe.LaunchTimer()
+    scattermoe.launch_timer = timer
+    step5()
+    scattermoe.launch_timer = None
+    torch.cuda.synchronize()
+    f5 = 6.0 * T5 * K5 * H5 * I5
+    launches = {}
+    for name, dims, s_, e_ in timer.records:
+        ms = s_.elapsed_time(e_)
+        fl = 2.0 * T5 * K5 * dims[0] * dims[1]
+        launches[name] = {"N_K": list(dims), "ms": ms, "TFLOP/s": fl / ms / 1e9, "frac_mfma_fp8": fl / ms / 1e9 / PEAK_FP8_TFLOPS}
+    out["C5_moe_e4m3_fwd"] = {"ms": dt * 1e3, "TFLOP/s": f5 / dt / 1e12, "frac_mfma_fp8": f5 / dt / 1e12 / PEAK_FP8_TFLOPS,
+                              "zipf_c": c5, "max_expert_share": max(freq5.tolist()), "launches": launches}
     return out
 
 

@@ -4,11 +4,15 @@
 //
 // Same machinery as the 16-bit kernel (tile-aligned expert segments, 256x256 tile, 8 waves, global -> LDS direct loads,
 // four XOR-swizzled 64-byte-row stages, hand-ordered load / fragment-read / MFMA stream, LDS-staged epilogue), with one
-// byte per element: a K step is 64 elements = four 16-wide slices of v_mfma_f32_32x32x16_fp8_fp8, fragments are 8 bytes
-// per lane, and every byte fetched from L2 carries twice the FLOPs.
+// byte per element: a K step is 64 elements = one v_mfma_f32_32x32x64_f8f6f4 per 32 x 32 block (twice the rate of the
+// 16-bit MFMA), fragments are 32 bytes per lane, and every byte fetched from L2 carries twice the FLOPs.
 #include <stdlib.h>
 
 #include "gemm_common.h"
+
+#ifndef CK_ABLATE
+#define CK_ABLATE 0  // measurement builds only: 2 no loads in the loop, 4 no fragment reads, 32 no epilogue, 64 no MFMA, 128 no main loop
+#endif
 
 namespace ck {
 namespace {
@@ -17,12 +21,17 @@ constexpr int BM = 256, BN = 256;
 constexpr int WGM = 4, NW = WGM * 2, NT = 64 * NW;  // 8 waves: 4 along M, 2 along N
 constexpr int WM = BM / WGM, WN = BN / 2;           // 64 x 128 wave tile
 constexpr int MI = WM / 32, NI = WN / 32;
-constexpr int BK = 64, KS = BK / 16, NSTAGE = 4;
+constexpr int BK = 64, NSTAGE = 4;
 constexpr int kRowBytes = 64;
 constexpr int kStageBytes = (BM + BN) * kRowBytes;
 constexpr int A_LD = BM / (16 * NW), B_LD = BN / (16 * NW);
-constexpr int kLoadsPerStep = A_LD + B_LD, kReads = MI + NI, kMfma = MI * NI;
-constexpr size_t kLdsBytes = (size_t)NSTAGE * kStageBytes;
+constexpr int kLoadsPerStep = A_LD + B_LD;
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x8 __attribute__((ext_vector_type(8)));
+constexpr int kMetaOffset = NSTAGE * kStageBytes;  // after the stages: a_scale of the tile's rows, w_scale of its columns,
+constexpr int kMetaBytes = (BM + BN + BM) * 4;      // and the output row of every tile row (scatter epilogue)
+constexpr size_t kLdsBytes = (size_t)kMetaOffset + kMetaBytes;
+static_assert(NT == BM + BN, "one thread per tile row / tile column fetches the epilogue's scales");
 
 template <typename TO, int MODE>
 __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams prm) {
@@ -44,6 +53,15 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
   const int64_t m0 = (int64_t)mt * BM;
   const int64_t valid_end = (int64_t)prm.seg_starts[expert] + prm.counts[expert];
 
+#if (CK_ABLATE & 256)
+  auto stamp = [&](int i) {
+    __builtin_amdgcn_s_waitcnt(0);
+    if (prm.y_t != nullptr && tid == 0) static_cast<uint64_t*>(prm.y_t)[(size_t)blockIdx.x * 8 + i] = wall_clock64();
+  };
+#else
+  auto stamp = [&](int) {};
+#endif
+  stamp(0);
   f32x16 acc[MI][NI];
 #pragma unroll
   for (int i = 0; i < MI; ++i)
@@ -79,7 +97,30 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
     }
     b_off[t] = (uint32_t)(n * prm.ldw + c * 16);
   }
-  const int nk = prm.K / BK;
+  const int nk = (CK_ABLATE & 128) ? 0 : prm.K / BK;  // 128: no main loop at all
+
+  // ---- what the epilogue needs from global memory is fetched now and parked in LDS after the main loop: thread t < BM
+  // takes tile row t (its de-quantisation scale and, for the scatter epilogue, its output row), thread BM + j column j
+  float meta_scale = 0.f;
+  int meta_row = -1;
+  if (tid < BM) {
+    const int64_t p = m0 + tid;
+    if (p < valid_end) {
+      const int slot = (prm.a_gather_div > 0 || MODE == kScatter) ? prm.row_slot[p] : 0;
+      meta_scale = prm.a_scale[prm.a_gather_div > 0 ? (int64_t)(slot / prm.a_gather_div) : p];
+      meta_row = (MODE == kScatter) ? slot : tid;
+    }
+  } else {
+    const int j = tid - BM;
+    const float* w_scale = prm.w_scale + (int64_t)expert * prm.N;
+    if constexpr (MODE == kSwiglu) {  // columns 0 .. 127: up scales of the tile's activation columns; 128 .. 255: gate
+      const int64_t col = (int64_t)nt * (BN / 2) + (j & (BN / 2 - 1));
+      if (col < prm.I) meta_scale = w_scale[(j < BN / 2 ? 0 : prm.I) + col];
+    } else {
+      const int64_t n = (int64_t)nt * BN + j;
+      if (n < prm.N) meta_scale = w_scale[n];
+    }
+  }
 
   auto dma16 = [&](const char* src, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(src) : "m0");
@@ -90,6 +131,9 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
   auto issue_one = [&](int step, int g) {
     const int64_t kb = (int64_t)min(step, nk - 1) * kRowBytes;  // past the end: re-fetch the last step (never read)
     const uint32_t st = (uint32_t)((step & (NSTAGE - 1)) * kStageBytes);
+    if constexpr ((CK_ABLATE & 2) != 0) {
+      if (step >= NSTAGE - 1) return;
+    }
     if (g < A_LD) dma16(a_base + kb + a_off[g], wave_a + st + g * 1024);
     else dma16(b_base + kb + b_off[g - A_LD], wave_b + st + (g - A_LD) * 1024);
   };
@@ -98,65 +142,84 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
     for (int g = 0; g < kLoadsPerStep; ++g) issue_one(step, g);
   };
 
-  // ---- fragments: slice sl of a row is its 16-byte chunk sl; lanes 0-31 take its first 8 bytes, lanes 32-63 the rest
+  // ---- fragments for v_mfma_f32_32x32x64_f8f6f4: lane l holds 32 bytes of row l % 32 -- 16-byte chunks 2h and 2h + 1 of
+  // the 64-byte row, h = l / 32. Both operands use the same byte -> k assignment, which is all a dot product needs.
   const int fsw = lds_swizzle(lane & 31), fh = lane >> 5;
-  int slice_off[KS];
-#pragma unroll
-  for (int sl = 0; sl < KS; ++sl) slice_off[sl] = ((sl ^ fsw) * 16) + fh * 8;
+  const int chunk_lo = ((2 * fh) ^ fsw) * 16, chunk_hi = ((2 * fh + 1) ^ fsw) * 16;
   const int fa_row = (wm * WM + (lane & 31)) * kRowBytes;
   const int fb_row = BM * kRowBytes + (wn * WN + (lane & 31)) * kRowBytes;
-  long fa[2][MI], fb[2][NI];
-  auto read_one = [&](int stage, int sl, int buf, int g) {
-    const char* st = lds_c + stage * kStageBytes + slice_off[sl];
-    if (g < MI) fa[buf][g] = *reinterpret_cast<const long*>(st + fa_row + g * 32 * kRowBytes);
-    else fb[buf][g - MI] = *reinterpret_cast<const long*>(st + fb_row + (g - MI) * 32 * kRowBytes);
+  i32x8 fa[MI], fb[NI];
+  auto read_frag = [&](int stage, int g) {  // g < MI: A block g; else B block g - MI
+    if constexpr ((CK_ABLATE & 4) != 0) {
+      if (stage != 0) return;
+    }
+    const char* row = lds_c + stage * kStageBytes + (g < MI ? fa_row + g * 32 * kRowBytes : fb_row + (g - MI) * 32 * kRowBytes);
+    const i32x4 lo = *reinterpret_cast<const i32x4*>(row + chunk_lo);
+    const i32x4 hi = *reinterpret_cast<const i32x4*>(row + chunk_hi);
+    const i32x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+    if (g < MI) fa[g] = v;
+    else fb[g - MI] = v;
   };
-  auto read_nth = [&](int stage, int sl, int buf, int n) {  // A0, every B block, then the remaining A blocks
-    const int g = n == 0 ? 0 : (n <= NI ? MI + n - 1 : n - NI);
-    read_one(stage, sl, buf, g);
+  auto mfma = [&](int i, int j) {
+    if constexpr ((CK_ABLATE & 64) != 0) {
+      asm volatile("" ::"v"(fa[i]), "v"(fb[j]));
+      return;
+    }
+    // scale operands 0: the compiler emits the unscaled v_mfma_f32_32x32x64_f8f6f4 (both operands e4m3: cbsz = blgp = 0)
+    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], 0, 0, 0, 0, 0, 0);
   };
-  auto mfma_range = [&](int buf, int first, int last) {
-#pragma unroll
-    for (int i = 0; i < MI; ++i)
-#pragma unroll
-      for (int j = 0; j < NI; ++j)
-        if (i * NI + j >= first && i * NI + j < last)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(fa[buf][i], fb[buf][j], acc[i][j], 0, 0, 0);
-  };
-  auto mfma_begin = [](int g) { return g * kMfma / kReads; };
-  static_assert(kLoadsPerStep <= kReads, "every load of a step has a slot in the last slice");
+  static_assert(MI == 2 && NI == 4 && kLoadsPerStep == 4, "the hand schedule below is written for a 64 x 128 wave tile");
 
+  stamp(1);
   if (nk > 0) {
     issue(0);
     issue(1);
     issue(2);
     asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * kLoadsPerStep) : "memory");  // step 0 landed, all waves
 #pragma unroll
-    for (int g = 0; g < kReads; ++g) read_one(0, 0, 0, g);
-    for (int kt = 0; kt < nk; ++kt) {
-      const int stage = kt & (NSTAGE - 1);
-      // slices 0 .. KS-2: their MFMAs hide the fragment reads of the next slice
-#pragma unroll
-      for (int sl = 0; sl + 1 < KS; ++sl) {
-#pragma unroll
-        for (int g = 0; g < kReads; ++g) {
-          read_nth(stage, sl + 1, (sl + 1) & 1, g);
-          mfma_range(sl & 1, mfma_begin(g), mfma_begin(g + 1));
-          __builtin_amdgcn_sched_barrier(0);
-        }
-      }
-      // step kt + 1 has landed for every wave (only step kt + 2 may be in flight); the barrier also orders the
-      // overwrite of stage (kt + 3) % 4, last read in step kt - 1
-      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kLoadsPerStep) : "memory");
-      // last slice: hides the loads of step kt + 3 and the slice-0 fragment reads of step kt + 1
-#pragma unroll
-      for (int g = 0; g < kReads; ++g) {
-        if (g < kLoadsPerStep) issue_one(kt + 3, g);
-        read_nth((kt + 1) & (NSTAGE - 1), 0, 0, g);
-        mfma_range((KS - 1) & 1, mfma_begin(g), mfma_begin(g + 1));
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
+    for (int g = 0; g < MI + NI; ++g) read_frag(0, g);
+    // One 64-byte K step per iteration = one MFMA per 32 x 32 block. Fragments are single-buffered and rotate: as soon
+    // as the last MFMA that needs a fragment has issued, the same registers are reloaded from the next step's stage.
+    // phase 0: steady state (prefetch step kt + 3, steps kt + 1 and kt + 2 in flight); phase 1: step nk - 3 (nothing left
+    // to prefetch, same wait); phase 2: the last two steps (at most one step in flight: wait for everything)
+    auto k_step = [&](int kt, auto phase) {
+      constexpr bool kTail = decltype(phase)::value > 0;
+      constexpr bool kWaitAll = decltype(phase)::value > 1;
+      const int next = (kt + 1) & (NSTAGE - 1);
+      mfma(0, 0);
+      mfma(0, 1);
+      mfma(0, 2);
+      mfma(0, 3);
+      __builtin_amdgcn_sched_barrier(0);
+      // step kt + 1 has landed for every wave (only step kt + 2 may be in flight); every fragment read of stage
+      // (kt + 3) % 4 was consumed before the barrier of step kt - 1, so its overwrite below is ordered too
+      if constexpr (kWaitAll) asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kLoadsPerStep) : "memory");
+      read_frag(next, 0);
+      if constexpr (!kTail) issue_one(kt + 3, 0);
+      mfma(1, 0);
+      __builtin_amdgcn_sched_barrier(0);
+      read_frag(next, MI + 0);
+      if constexpr (!kTail) issue_one(kt + 3, 1);
+      mfma(1, 1);
+      __builtin_amdgcn_sched_barrier(0);
+      read_frag(next, MI + 1);
+      if constexpr (!kTail) issue_one(kt + 3, 2);
+      mfma(1, 2);
+      __builtin_amdgcn_sched_barrier(0);
+      read_frag(next, MI + 2);
+      if constexpr (!kTail) issue_one(kt + 3, 3);
+      mfma(1, 3);
+      __builtin_amdgcn_sched_barrier(0);
+      read_frag(next, MI + 3);
+      read_frag(next, 1);
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    // a prefetch past the end would only re-fetch the last step and waste L2 bandwidth
+    int kt = 0;
+    for (; kt + 3 < nk; ++kt) k_step(kt, std::integral_constant<int, 0>{});
+    if (kt + 3 == nk) k_step(kt++, std::integral_constant<int, 1>{});
+    for (; kt < nk; ++kt) k_step(kt, std::integral_constant<int, 2>{});
   }
 
   // ---- epilogue through LDS (see the 16-bit kernel): slab S[col][row] of 128 tile columns, 8-byte writes from the
@@ -164,25 +227,31 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
   typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4;
   constexpr int kSlabCols = 128, kSlabLd = BM + 4;
   TO* slab = reinterpret_cast<TO*>(lds_raw);
+  stamp(2);
+  float* meta_f = reinterpret_cast<float*>(lds_c + kMetaOffset);    // [0, BM): a scales; [BM, BM + BN): w scales
+  int* meta_rows = reinterpret_cast<int*>(lds_c + kMetaOffset) + BM + BN;  // [BM]: output row, -1 for a pad row
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  meta_f[tid] = meta_scale;
+  if (tid < BM) meta_rows[tid] = meta_row;
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  stamp(3);
   const int col_in_block = lane & 31;
   const int row_quad = (lane >> 5) * 4;
-  const TO kZero = Elem<TO>::down(0.f);
 
-  // dequantisation scales of the rows this lane holds
+  // de-quantisation scales of the rows this lane holds (0 for pad rows)
   float rs[MI][4][4];
 #pragma unroll
   for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int q = 0; q < 4; ++q)
-#pragma unroll
-      for (int s = 0; s < 4; ++s) {
-        const int64_t p = m0 + wm * WM + i * 32 + 8 * q + row_quad + s;
-        float v = 0.f;
-        if (p < valid_end) v = prm.a_scale[prm.a_gather_div > 0 ? (int64_t)(prm.row_slot[p] / prm.a_gather_div) : p];
-        rs[i][q][s] = v;
-      }
+    for (int q = 0; q < 4; ++q) {
+      const float4 v = *reinterpret_cast<const float4*>(meta_f + wm * WM + i * 32 + 8 * q + row_quad);
+      rs[i][q][0] = v.x;
+      rs[i][q][1] = v.y;
+      rs[i][q][2] = v.z;
+      rs[i][q][3] = v.w;
+    }
 
+  stamp(4);
   auto stage_blocks = [&](auto&& value) {
     static_for<MI>([&](auto i) {
       static_for<2>([&](auto jj) {
@@ -218,35 +287,38 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
       }
     }
   };
-  const float* w_scale = prm.w_scale + (int64_t)expert * prm.N;
+  const float* w_sc = meta_f + BM;
 
-  if constexpr (MODE == kGrouped || MODE == kScatter) {
+  if constexpr ((CK_ABLATE & 32) != 0) {
+    float sum = 0.f;
+    static_for<MI>([&](auto i) { static_for<NI>([&](auto j) { static_for<16>([&](auto r) { sum += acc[i][j][(int)r]; }); }); });
+    if (sum == 12345.678f) static_cast<TO*>(prm.y ? prm.y : prm.aux)[tid] = Elem<TO>::down(sum + rs[0][0][0]);
+  } else if constexpr (MODE == kGrouped || MODE == kScatter) {
     TO* y = static_cast<TO*>(prm.y);
     static_for<2>([&](auto pass) {
       float cs[2];
-      static_for<2>([&](auto jj) {
-        const int64_t n = (int64_t)nt * BN + wn * WN + (pass * 2 + jj) * 32 + col_in_block;
-        cs[jj] = n < prm.N ? w_scale[n] : 0.f;
-      });
+      static_for<2>([&](auto jj) { cs[jj] = w_sc[wn * WN + (pass * 2 + jj) * 32 + col_in_block]; });
       stage_blocks([&](auto i, auto jj, auto q, auto s) {
         return Elem<TO>::down(acc[i][pass * 2 + jj][4 * q + s] * rs[i][q][s] * cs[jj]);
       });
       __syncthreads();
+      if constexpr (pass == 0) stamp(6);
       drain_rows([&](int r, int sc) -> TO* {
-        const int64_t p = m0 + r, n = (int64_t)nt * BN + (sc >> 6) * WN + pass * 64 + (sc & 63);
-        if (p >= valid_end || n >= prm.N) return nullptr;
-        const int64_t row = (MODE == kScatter) ? (int64_t)prm.row_slot[p] : p;
+        const int64_t n = (int64_t)nt * BN + (sc >> 6) * WN + pass * 64 + (sc & 63);
+        const int out_row = meta_rows[r];
+        if (out_row < 0 || n >= prm.N) return nullptr;
+        const int64_t row = (MODE == kScatter) ? (int64_t)out_row : m0 + r;
         return y + row * prm.N + n;
       });
+      if constexpr (pass == 0) stamp(7);
       __syncthreads();
     });
   } else {  // kSwiglu: blocks 0, 1 = up, blocks 2, 3 = gate of the same activation columns; only the activation is kept
     TO* act = static_cast<TO*>(prm.aux);
     float cs_up[2], cs_gate[2];
     static_for<2>([&](auto jj) {
-      const int64_t col = (int64_t)nt * (BN / 2) + wn * (WN / 2) + jj * 32 + col_in_block;
-      cs_up[jj] = col < prm.I ? w_scale[col] : 0.f;
-      cs_gate[jj] = col < prm.I ? w_scale[prm.I + col] : 0.f;
+      cs_up[jj] = w_sc[wn * (WN / 2) + jj * 32 + col_in_block];
+      cs_gate[jj] = w_sc[BN / 2 + wn * (WN / 2) + jj * 32 + col_in_block];
     });
     stage_blocks([&](auto i, auto jj, auto q, auto s) {
       // rounded to the output type first, like a pre-activation tensor would be
@@ -262,7 +334,7 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
       return act + p * prm.I + col;
     });
   }
-  (void)kZero;
+  stamp(5);
 }
 
 template <typename TO, int MODE>
@@ -386,6 +458,9 @@ extern "C" int ck_grouped_gemm_fp8(const void* a8, const float* a_scale, int32_t
   prm.aux = aux;
   prm.a_scale = a_scale;
   prm.w_scale = w_scale;
+#if (CK_ABLATE & 256)
+  if (const char* t = getenv("CK_TRACE_PTR")) prm.y_t = reinterpret_cast<void*>(strtoull(t, nullptr, 16));
+#endif
   int out_cols = N;
   if (epilogue == CK_EPI_SWIGLU) {
     CK_REQUIRE(N % 16 == 0 && aux != nullptr, "%s: the SwiGLU epilogue needs N = 2*I with I %% 8 == 0 and aux", name);

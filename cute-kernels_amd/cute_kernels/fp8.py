@@ -13,6 +13,7 @@ import torch
 import torch.nn as nn
 
 from . import _C
+from . import scattermoe
 from .scattermoe import ExpertSegments, _combine, route_topk_softmax, sort_by_expert
 
 
@@ -47,13 +48,20 @@ def quantize_expert_weights_e4m3(weight: torch.Tensor) -> tuple[torch.Tensor, to
 def _gemm_fp8(a8, a_scale, gather_div, w8, w_scale, seg: ExpertSegments, epilogue, y, aux, out_dtype):
     E, N, K = w8.shape
     cs = seg.c_struct()
-    with torch.cuda.device(w8.device):
-        _C.check(
-            _C.lib().ck_grouped_gemm_fp8(
-                _C.ptr(a8), _C.ptr(a_scale), gather_div, _C.ptr(w8), _C.ptr(w_scale), N, K, ctypes.byref(cs), epilogue,
-                _C.ptr(y), _C.ptr(aux), _C.dtype_code(out_dtype), _C.stream(),
+
+    def launch():
+        with torch.cuda.device(w8.device):
+            _C.check(
+                _C.lib().ck_grouped_gemm_fp8(
+                    _C.ptr(a8), _C.ptr(a_scale), gather_div, _C.ptr(w8), _C.ptr(w_scale), N, K, ctypes.byref(cs),
+                    epilogue, _C.ptr(y), _C.ptr(aux), _C.dtype_code(out_dtype), _C.stream(),
+                )
             )
-        )
+
+    if scattermoe.launch_timer is None:
+        launch()
+    else:
+        scattermoe.launch_timer.time("fp8_" + scattermoe._EPILOGUE_NAMES[epilogue], (N, K), launch)
 
 
 @torch.no_grad()
