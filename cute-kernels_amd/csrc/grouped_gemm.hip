@@ -60,6 +60,16 @@ const bool g_eight_waves = [] {
 // WGM: waves along M (2 or 4), always 2 along N: 4 waves = one per SIMD with 128x128 wave tiles at BM = BN = 256;
 //      8 waves = two per SIMD with 64x128 wave tiles, so that one wave's memory instructions issue under the other's
 //      MFMAs (PIPE 1 only).
+// pipeline stages, then one int per tile row: the output row of the scatter epilogue (-1 for a pad row)
+template <int BM, int BN, int PIPE>
+constexpr size_t stage_bytes() {
+  return PIPE == 0 ? (size_t)2 * (BM + BN) * kLdsStride * 2 : (size_t)4 * (BM + BN) * 32 * 2;
+}
+template <int BM, int BN, int PIPE>
+constexpr size_t lds_bytes() {
+  return stage_bytes<BM, BN, PIPE>() + (size_t)BM * 4;
+}
+
 template <typename T, int BM, int BN, int MODE, int PIPE, int WGM>
 __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmParams prm) {
   static_assert(PIPE == 1 || WGM == 2, "the register-staged pipeline is written for 4 waves");
@@ -114,6 +124,12 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
 
   int64_t valid_end = 0;  // forward modes: first pad row of this expert's segment
   if constexpr (MODE != kDw) valid_end = (int64_t)prm.seg_starts[expert] + prm.counts[expert];
+  // scatter epilogue: the output row of tile row `tid`, fetched now and parked in LDS once the main loop is over
+  int scatter_row = -1;
+  if constexpr (MODE == kScatter) {
+    for (int r = threadIdx.x; r < BM; r += 64 * WGM * 2)  // at most one trip per thread: BM <= threads
+      if (m0 + r < valid_end) scatter_row = prm.row_slot[m0 + r];
+  }
 
   f32x16 acc[MI][NI];
 #pragma unroll
@@ -387,7 +403,10 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
       wait_and_barrier(std::integral_constant<int, 2 * kLoadsPerStep>{});  // step 0 has landed, for every wave
 #pragma unroll
       for (int g = 0; g < kReads; ++g) read_one(0, 0, 0, g);
-      for (int kt = 0; kt < nk; ++kt) {
+      // phase 0: steady state (prefetch step kt + 3; steps kt + 1, kt + 2 in flight); phase 1: step nk - 3 (nothing left
+      // to prefetch, same wait); phase 2: the last two steps (at most one step in flight: wait for all of it)
+      auto k_step = [&](int kt, auto phase) {
+        constexpr int kPhase = decltype(phase)::value;
         // first half: MFMAs of slice 0 from fragment buffer 0, the fragment reads of slice 1 between them
 #pragma unroll
         for (int g = 0; g < kReads; ++g) {
@@ -398,20 +417,25 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
         // Step kt + 1 has landed for every wave (only step kt + 2 may still be in flight). The barrier also orders
         // the overwrite below: stage (kt + 3) % 4 was last read as slice 1 of step kt - 1, and every wave consumed
         // those fragments (so its reads completed) before arriving here.
-        wait_and_barrier(std::integral_constant<int, kLoadsPerStep>{});
+        wait_and_barrier(std::integral_constant<int, kPhase == 2 ? 0 : kLoadsPerStep>{});
         // second half: MFMAs of slice 1 from buffer 1; between them the loads of step kt + 3 and the slice-0 fragment
         // reads of step kt + 1
 #pragma unroll
         for (int g = 0; g < kReads; ++g) {
-          if constexpr (!(CK_ABLATE & 2))
+          if constexpr (!(CK_ABLATE & 2) && kPhase == 0)
             if (g < kLoadsPerStep) issue_one(kt + 3, g);
           read_nth((kt + 1) & (NSTAGE - 1), 0, 0, g);
           mfma_range(1, mfma_begin(g), mfma_begin(g + 1));
           __builtin_amdgcn_sched_barrier(0);
         }
         static_assert(kLoadsPerStep <= kReads, "every load of a step has a slot in the second half");
-      }
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // drain the re-fetches before LDS is reused or released
+      };
+      // a prefetch past the end would only re-fetch the last step and waste L2 bandwidth
+      int kt = 0;
+      for (; kt + 3 < nk; ++kt) k_step(kt, std::integral_constant<int, 0>{});
+      if (kt + 3 == nk) k_step(kt++, std::integral_constant<int, 1>{});
+      for (; kt < nk; ++kt) k_step(kt, std::integral_constant<int, 2>{});
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // short contractions: the prologue fetched past the end
     }
   }
 
@@ -438,6 +462,10 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
     constexpr int NT = 64 * NW;
     constexpr int kSlabCols = 128, kSlabLd = BM + 4;  // 520-byte rows: 8-byte aligned and spread over the banks
     T* slab = lds;                                    // the pipeline stages are dead by now
+    int* scatter_rows = reinterpret_cast<int*>(lds_raw + stage_bytes<BM, BN, PIPE>());
+    if constexpr (MODE == kScatter) {
+      if (tid < BM) scatter_rows[tid] = scatter_row;
+    }
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave is done with the stages
 
     // write this wave's blocks (i, jb..jb+1) of a value source into the slab
@@ -517,7 +545,7 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
         drain_rows([&](int r, int sc) -> T* {
           const int64_t p = m0 + r, n = (int64_t)nt * BN + tile_col(sc, pass);
           if (p >= valid_end || n >= prm.N) return nullptr;
-          const int64_t row = (MODE == kScatter) ? (int64_t)prm.row_slot[p] : p;
+          const int64_t row = (MODE == kScatter) ? (int64_t)scatter_rows[r] : p;
           return y + row * prm.N + n;
         });
         if (MODE == kGrouped && y_t != nullptr) {
@@ -670,11 +698,6 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
       });
     });
   }
-}
-
-template <int BM, int BN, int PIPE>
-constexpr size_t lds_bytes() {
-  return PIPE == 0 ? (size_t)2 * (BM + BN) * kLdsStride * 2 : (size_t)4 * (BM + BN) * 32 * 2;
 }
 
 template <typename T, int BM, int BN, int MODE, int PIPE, int WGM>

@@ -44,6 +44,27 @@ struct Vec {
   }
 };
 
+// Residual-add fusion (both optional, all-null = plain RMSNorm).
+// forward: added = round(round(x * multiplier) + residual) is written out and normalised (multiplier == 1: no scaling);
+// backward: d_added_total = d(norm input) + d_added; d_residual = d_added_total, d_x = d_added_total * multiplier.
+template <typename T>
+struct FwdFuse {
+  const T* residual;
+  T* added;
+  float multiplier;
+};
+template <typename T>
+struct BwdFuse {
+  const T* d_added;
+  T* d_residual;
+  float multiplier;
+};
+
+template <typename T>
+__device__ inline float round_to(float v) {
+  return Elem<T>::up(Elem<T>::down(v));
+}
+
 template <int TPR>
 __device__ inline float row_sum(float v, float* scratch) {
   if constexpr (TPR == kWave) return wave_sum(v);
@@ -54,7 +75,8 @@ __device__ inline float row_sum(float v, float* scratch) {
 template <typename T, int P, int TPR, int NC>
 __global__ __launch_bounds__(kBlock) void rmsnorm_fwd_kernel(const T* __restrict__ x, const T* __restrict__ weight,
                                                               float eps, int64_t B, int H, int chunks,
-                                                              T* __restrict__ out, float* __restrict__ rstd_out) {
+                                                              T* __restrict__ out, float* __restrict__ rstd_out,
+                                                              const FwdFuse<T> fuse) {
   __shared__ float scratch[kBlock / kWave];
   constexpr int ROWS = kBlock / TPR;
   const int lane = threadIdx.x % TPR;
@@ -64,6 +86,23 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_fwd_kernel(const T* __restrict
   for (int64_t row = (int64_t)blockIdx.x * ROWS + threadIdx.x / TPR; row < B; row += row_stride) {
     const T* xr = x + row * H;
     T* yr = out + row * H;
+    const T* rr = fuse.residual ? fuse.residual + row * H : nullptr;
+    T* ar = fuse.residual ? fuse.added + row * H : nullptr;
+    // the row to normalise: x, or the freshly written sum with the residual stream
+    auto load_x = [&](int ch) {
+      Vec<T, P> v = Vec<T, P>::load(xr + (int64_t)ch * P);
+      if (rr != nullptr) {
+        const Vec<T, P> r = Vec<T, P>::load(rr + (int64_t)ch * P);
+#pragma unroll
+        for (int i = 0; i < P; ++i) {
+          float t = v.f[i];
+          if (fuse.multiplier != 1.0f) t = round_to<T>(t * fuse.multiplier);
+          v.f[i] = round_to<T>(t + r.f[i]);
+        }
+        v.store(ar + (int64_t)ch * P);
+      }
+      return v;
+    };
     float ss = 0.f;
     if constexpr (NC > 0) {
       Vec<T, P> xv[NC];
@@ -71,7 +110,7 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_fwd_kernel(const T* __restrict
       for (int c = 0; c < NC; ++c) {
         const int ch = c * TPR + lane;
         if (ch < chunks) {
-          xv[c] = Vec<T, P>::load(xr + (int64_t)ch * P);
+          xv[c] = load_x(ch);
 #pragma unroll
           for (int i = 0; i < P; ++i) ss += xv[c].f[i] * xv[c].f[i];
         }
@@ -92,15 +131,16 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_fwd_kernel(const T* __restrict
       }
     } else {
       for (int ch = lane; ch < chunks; ch += TPR) {
-        const Vec<T, P> v = Vec<T, P>::load(xr + (int64_t)ch * P);
+        const Vec<T, P> v = load_x(ch);
 #pragma unroll
         for (int i = 0; i < P; ++i) ss += v.f[i] * v.f[i];
       }
       ss = row_sum<TPR>(ss, scratch);
       const float rs = rsqrtf(ss * inv_h + eps);
       if (rstd_out != nullptr && lane == 0) rstd_out[row] = rs;
+      const T* again = rr != nullptr ? ar : xr;  // this lane's own writes, or x (L1 / L2 serve the second read)
       for (int ch = lane; ch < chunks; ch += TPR) {
-        const Vec<T, P> v = Vec<T, P>::load(xr + (int64_t)ch * P);
+        const Vec<T, P> v = Vec<T, P>::load(again + (int64_t)ch * P);
         const Vec<T, P> wv = weight ? Vec<T, P>::load(weight + (int64_t)ch * P) : Vec<T, P>::ones();
         Vec<T, P> y;
 #pragma unroll
@@ -117,7 +157,8 @@ template <typename T, int P, int TPR, int NC>
 __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const T* __restrict__ x, const T* __restrict__ weight,
                                                               const T* __restrict__ d_out, const float* __restrict__ rstd,
                                                               float eps, int64_t B, int H, int chunks,
-                                                              T* __restrict__ d_x, float* __restrict__ partial) {
+                                                              T* __restrict__ d_x, float* __restrict__ partial,
+                                                              const BwdFuse<T> fuse) {
   __shared__ float scratch[kBlock / kWave];
   constexpr int ROWS = kBlock / TPR;
   const int lane = threadIdx.x % TPR;
@@ -144,6 +185,20 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const T* __restrict
     const T* xr = x + row * H;
     const T* gr = d_out + row * H;
     T* dxr = d_x + row * H;
+    // o = gradient w.r.t. the normalised row; with the fusion add the residual stream's gradient, emit both outputs
+    auto finish = [&](Vec<T, P>& o, int ch) {
+      if (fuse.d_added != nullptr) {
+        const Vec<T, P> a = Vec<T, P>::load(fuse.d_added + row * H + (int64_t)ch * P);
+#pragma unroll
+        for (int i = 0; i < P; ++i) o.f[i] += a.f[i];
+      }
+      if (fuse.d_residual != nullptr) o.store(fuse.d_residual + row * H + (int64_t)ch * P);
+      if (fuse.multiplier != 1.0f) {
+#pragma unroll
+        for (int i = 0; i < P; ++i) o.f[i] = round_to<T>(o.f[i]) * fuse.multiplier;
+      }
+      o.store(dxr + (int64_t)ch * P);
+    };
     float dot = 0.f, ss = 0.f;
     if constexpr (NC > 0) {
       Vec<T, P> xv[NC], gv[NC];  // gv holds d_y * w
@@ -181,7 +236,7 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const T* __restrict
             o.f[i] = rs * gv[c].f[i] * wv.f[i] - coef * xv[c].f[i];
             dw[c].f[i] += gv[c].f[i] * xv[c].f[i] * rs;
           }
-          o.store(dxr + (int64_t)ch * P);
+          finish(o, ch);
         }
       }
     } else {
@@ -214,7 +269,7 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const T* __restrict
           o.f[i] = rs * gv.f[i] * wv.f[i] - coef * xv.f[i];
           if (my_partial != nullptr) my_partial[(int64_t)ch * P + i] += gv.f[i] * xv.f[i] * rs;  // lane-private slots
         }
-        o.store(dxr + (int64_t)ch * P);
+        finish(o, ch);
       }
     }
   }
@@ -232,23 +287,35 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const T* __restrict
   }
 }
 
-// d_weight[h] = sum over the partial rows, in a fixed order. A block owns 64 columns; its 4 waves each sum a quarter of
-// the rows (reads are 256-byte coalesced), then the quarters are added through LDS.
-__global__ __launch_bounds__(kBlock) void rmsnorm_dw_reduce_kernel(const float* __restrict__ partial, int64_t workers,
-                                                                    int H, float* __restrict__ d_weight) {
-  __shared__ float part[kBlock / kWave][kWave];
+// d_weight[h] = sum over the partial rows, in a fixed order. A block owns 64 columns; its 16 waves each sum a sixteenth
+// of the rows (256-byte coalesced reads, 8 independent partial sums so that 8 loads are in flight per wave), then the
+// sixteen results are added through LDS.
+constexpr int kReduceBlock = 1024, kReduceWaves = kReduceBlock / kWave, kReduceUnroll = 8;
+__global__ __launch_bounds__(kReduceBlock) void rmsnorm_dw_reduce_kernel(const float* __restrict__ partial, int64_t workers,
+                                                                          int H, float* __restrict__ d_weight) {
+  __shared__ float part[kReduceWaves][kWave];
   const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
   const int h = blockIdx.x * kWave + lane;
   float s = 0.f;
   if (h < H) {
-    for (int64_t w = wave; w < workers; w += kBlock / kWave) s += partial[w * H + h];
+    float acc[kReduceUnroll];
+#pragma unroll
+    for (int u = 0; u < kReduceUnroll; ++u) acc[u] = 0.f;
+    int64_t w = wave;
+    for (; w + (kReduceUnroll - 1) * kReduceWaves < workers; w += kReduceUnroll * kReduceWaves) {
+#pragma unroll
+      for (int u = 0; u < kReduceUnroll; ++u) acc[u] += partial[(w + u * kReduceWaves) * H + h];
+    }
+    for (; w < workers; w += kReduceWaves) acc[0] += partial[w * H + h];
+#pragma unroll
+    for (int u = 0; u < kReduceUnroll; ++u) s += acc[u];
   }
   part[wave][lane] = s;
   __syncthreads();
   if (wave == 0 && h < H) {
     float t = 0.f;
 #pragma unroll
-    for (int g = 0; g < kBlock / kWave; ++g) t += part[g][lane];
+    for (int g = 0; g < kReduceWaves; ++g) t += part[g][lane];
     d_weight[h] = t;
   }
 }
@@ -312,65 +379,101 @@ using namespace ck;
 #define CK_RMS_FWD(PP, TPR, NC, dummy)                                                                              \
   hipLaunchKernelGGL((rmsnorm_fwd_kernel<scalar_t, PP, TPR, NC>), dim3((unsigned)blocks), dim3(kBlock), 0, s,        \
                      static_cast<const scalar_t*>(x), static_cast<const scalar_t*>(weight), eps, B, (int)H,          \
-                     plan.chunks, static_cast<scalar_t*>(out), rstd)
+                     plan.chunks, static_cast<scalar_t*>(out), rstd, fuse)
 
-extern "C" int ck_rmsnorm_fwd(const void* x, const void* weight, float eps, int64_t B, int32_t H, void* out,
-                              float* rstd, int32_t dtype, void* stream) {
-  CK_REQUIRE(B >= 0 && H >= 1, "ck_rmsnorm_fwd: bad sizes B=%lld H=%d", (long long)B, H);
+static int rmsnorm_fwd_impl(const char* name, const void* x, const void* residual, const void* weight, float eps,
+                            float multiplier, int64_t B, int32_t H, void* out, void* added, float* rstd, int32_t dtype,
+                            void* stream) {
+  CK_REQUIRE(B >= 0 && H >= 1, "%s: bad sizes B=%lld H=%d", name, (long long)B, H);
   if (B == 0) return CK_OK;
-  CK_REQUIRE(x && out, "ck_rmsnorm_fwd: NULL argument");
+  CK_REQUIRE(x && out, "%s: NULL argument", name);
+  CK_REQUIRE((residual == nullptr) == (added == nullptr), "%s: residual and added must be given together", name);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  CK_DISPATCH_FLOAT(dtype, "ck_rmsnorm_fwd", {
-    const bool aligned = aligned16(x) && aligned16(out) && (weight == nullptr || aligned16(weight));
+  CK_DISPATCH_FLOAT(dtype, name, {
+    const bool aligned = aligned16(x) && aligned16(out) && (weight == nullptr || aligned16(weight)) &&
+                         (residual == nullptr || (aligned16(residual) && aligned16(added)));
     const Plan plan = make_plan<scalar_t>(H, aligned);
     const int rows_per_block = kBlock / plan.tpr;
     int64_t blocks = ceil_div(B, rows_per_block);
     if (blocks > 8192) blocks = 8192;
+    const FwdFuse<scalar_t> fuse = {static_cast<const scalar_t*>(residual), static_cast<scalar_t*>(added), multiplier};
     CK_RMS_DISPATCH(CK_RMS_FWD, 0);
   });
-  CK_CHECK_LAUNCH("ck_rmsnorm_fwd");
+  CK_CHECK_LAUNCH(name);
   return CK_OK;
+}
+
+extern "C" int ck_rmsnorm_fwd(const void* x, const void* weight, float eps, int64_t B, int32_t H, void* out,
+                              float* rstd, int32_t dtype, void* stream) {
+  return rmsnorm_fwd_impl("ck_rmsnorm_fwd", x, nullptr, weight, eps, 1.0f, B, H, out, nullptr, rstd, dtype, stream);
+}
+
+extern "C" int ck_fused_residual_add_rmsnorm_fwd(const void* x, const void* residual, const void* weight, float eps,
+                                                 float multiplier, int64_t B, int32_t H, void* out, void* added,
+                                                 float* rstd, int32_t dtype, void* stream) {
+  const char* name = "ck_fused_residual_add_rmsnorm_fwd";
+  CK_REQUIRE(B == 0 || (residual && added), "%s: residual and added are required", name);
+  return rmsnorm_fwd_impl(name, x, residual, weight, eps, multiplier, B, H, out, added, rstd, dtype, stream);
 }
 
 #define CK_RMS_BWD(PP, TPR, NC, dummy)                                                                              \
   hipLaunchKernelGGL((rmsnorm_bwd_kernel<scalar_t, PP, TPR, NC>), dim3((unsigned)blocks), dim3(kBlock), 0, s,        \
                      static_cast<const scalar_t*>(x), static_cast<const scalar_t*>(weight),                          \
                      static_cast<const scalar_t*>(d_out), rstd, eps, B, (int)H, plan.chunks,                         \
-                     static_cast<scalar_t*>(d_x), d_weight_partial)
+                     static_cast<scalar_t*>(d_x), d_weight_partial, fuse)
 
 extern "C" int64_t ck_rmsnorm_bwd_partial_rows(int64_t B) {
   if (B <= 0) return 0;
   return round_up(B < kMaxWorkers ? B : kMaxWorkers, kBlock / kWave);
 }
 
-extern "C" int ck_rmsnorm_bwd(const void* x, const void* weight, const void* d_out, const float* rstd, float eps,
-                              int64_t B, int32_t H, void* d_x, float* d_weight_partial, float* d_weight, int32_t dtype,
-                              void* stream) {
-  CK_REQUIRE(B >= 0 && H >= 1, "ck_rmsnorm_bwd: bad sizes B=%lld H=%d", (long long)B, H);
+static int rmsnorm_bwd_impl(const char* name, const void* x, const void* weight, const void* d_out, const void* d_added,
+                            const float* rstd, float eps, float multiplier, int64_t B, int32_t H, void* d_x,
+                            void* d_residual, float* d_weight_partial, float* d_weight, int32_t dtype, void* stream) {
+  CK_REQUIRE(B >= 0 && H >= 1, "%s: bad sizes B=%lld H=%d", name, (long long)B, H);
   CK_REQUIRE((weight == nullptr) == (d_weight == nullptr) && (weight == nullptr) == (d_weight_partial == nullptr),
-             "ck_rmsnorm_bwd: weight, d_weight and d_weight_partial must be given together");
+             "%s: weight, d_weight and d_weight_partial must be given together", name);
   if (B == 0) {
     if (d_weight != nullptr) {  // no rows: the sum over zero partial rows is zero
-      hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3((unsigned)ceil_div(H, kWave)), dim3(kBlock), 0,
+      hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3((unsigned)ceil_div(H, kWave)), dim3(kReduceBlock), 0,
                          static_cast<hipStream_t>(stream), d_weight_partial, (int64_t)0, (int)H, d_weight);
-      CK_CHECK_LAUNCH("ck_rmsnorm_bwd");
+      CK_CHECK_LAUNCH(name);
     }
     return CK_OK;
   }
-  CK_REQUIRE(x && d_out && d_x, "ck_rmsnorm_bwd: NULL argument");
+  CK_REQUIRE(x && d_out && d_x, "%s: NULL argument", name);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  CK_DISPATCH_FLOAT(dtype, "ck_rmsnorm_bwd", {
-    const bool aligned = aligned16(x) && aligned16(d_out) && aligned16(d_x) && (weight == nullptr || aligned16(weight));
+  CK_DISPATCH_FLOAT(dtype, name, {
+    const bool aligned = aligned16(x) && aligned16(d_out) && aligned16(d_x) && (weight == nullptr || aligned16(weight)) &&
+                         (d_added == nullptr || aligned16(d_added)) && (d_residual == nullptr || aligned16(d_residual));
     const Plan plan = make_plan<scalar_t>(H, aligned);
     const int rows_per_block = kBlock / plan.tpr;
     const int64_t workers = workers_for(B, plan.tpr);
     const int64_t blocks = workers / rows_per_block;
+    const BwdFuse<scalar_t> fuse = {static_cast<const scalar_t*>(d_added), static_cast<scalar_t*>(d_residual), multiplier};
     CK_RMS_DISPATCH(CK_RMS_BWD, 0);
     if (d_weight != nullptr) {
-      hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3((unsigned)ceil_div(H, kWave)), dim3(kBlock), 0, s,
+      hipLaunchKernelGGL(rmsnorm_dw_reduce_kernel, dim3((unsigned)ceil_div(H, kWave)), dim3(kReduceBlock), 0, s,
                          d_weight_partial, workers, (int)H, d_weight);
     }
   });
-  CK_CHECK_LAUNCH("ck_rmsnorm_bwd");
+  CK_CHECK_LAUNCH(name);
   return CK_OK;
+}
+
+extern "C" int ck_rmsnorm_bwd(const void* x, const void* weight, const void* d_out, const float* rstd, float eps,
+                              int64_t B, int32_t H, void* d_x, float* d_weight_partial, float* d_weight, int32_t dtype,
+                              void* stream) {
+  return rmsnorm_bwd_impl("ck_rmsnorm_bwd", x, weight, d_out, nullptr, rstd, eps, 1.0f, B, H, d_x, nullptr,
+                          d_weight_partial, d_weight, dtype, stream);
+}
+
+extern "C" int ck_fused_residual_add_rmsnorm_bwd(const void* added, const void* weight, const void* d_out,
+                                                 const void* d_added, const float* rstd, float eps, float multiplier,
+                                                 int64_t B, int32_t H, void* d_x, void* d_residual,
+                                                 float* d_weight_partial, float* d_weight, int32_t dtype, void* stream) {
+  const char* name = "ck_fused_residual_add_rmsnorm_bwd";
+  CK_REQUIRE(B == 0 || d_residual != nullptr, "%s: d_residual is required", name);
+  return rmsnorm_bwd_impl(name, added, weight, d_out, d_added, rstd, eps, multiplier, B, H, d_x, d_residual,
+                          d_weight_partial, d_weight, dtype, stream);
 }

@@ -8,6 +8,7 @@ ahead-of-time built libck_mi355.so; there is no other backend and no CPU path.
 from .fp8 import MoE_E4M3, quantize_expert_weights_e4m3, quantize_rows_e4m3, swiglu_experts_e4m3
 from .continuous_count import continuous_count_and_offsets_cute, continuous_count_cute
 from .modules import Experts, MoE, MoE_Triton
+from .fused_residual_add_rmsnorm import fused_residual_add_rmsnorm_cute
 from .rmsnorm import rmsnorm_cute
 from .scattermoe import (
     ExpertSegments,

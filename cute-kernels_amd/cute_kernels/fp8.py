@@ -84,7 +84,7 @@ def swiglu_experts_e4m3(
     E, two_i, _ = w_fc8.shape
     I = two_i // 2
     x8, x_scale = quantize_rows_e4m3(x)  # per token
-    act = torch.zeros(seg.max_rows, I, dtype=x.dtype, device=x.device)  # pad rows stay zero for the row quantiser
+    act = torch.empty(seg.max_rows, I, dtype=x.dtype, device=x.device)  # pad rows: never written, quantised, never used
     _gemm_fp8(x8, x_scale, k, w_fc8, w_fc_scale, seg, _C.CK_EPI_SWIGLU, None, act, x.dtype)
     act8, act_scale = quantize_rows_e4m3(act)  # per routed row
     expanded = torch.empty(T * k, H, dtype=x.dtype, device=x.device)

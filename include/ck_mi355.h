@@ -220,6 +220,24 @@ int64_t ck_rmsnorm_bwd_partial_rows(int64_t B);
 int ck_rmsnorm_bwd(const void* x, const void* weight, const void* d_out, const float* rstd, float eps, int64_t B,
                    int32_t H, void* d_x, float* d_weight_partial, float* d_weight, int32_t dtype, void* stream);
 
+/* ---------------------------------------------------------------------------------------------------------------
+ * Residual add fused with RMSNorm (the step in front of an MoE block in a transformer layer)
+ * Replaces: fused_residual_add_rmsnorm_forward_triton / _backward_triton -- cute_kernels/kernels/
+ *           fused_residual_add_rmsnorm/triton_implementation/forward.py:14-104, backward.py:14-149; semantics of
+ *           fused_residual_add_rmsnorm_torch (torch_implementation.py:9-19).
+ * forward:  added = (x * multiplier) + residual, each step rounded to the tensor dtype (multiplier == 1: no scaling);
+ *           out = rmsnorm(added). x, residual, out, added [B, H]; rstd as above.
+ * backward: g = d rmsnorm(added)/d added applied to d_out, plus d_added (the gradient arriving through the residual
+ *           stream; NULL = none); d_residual = g, d_x = g * multiplier. `added` is the forward's output.
+ * ------------------------------------------------------------------------------------------------------------- */
+int ck_fused_residual_add_rmsnorm_fwd(const void* x, const void* residual, const void* weight, float eps,
+                                      float multiplier, int64_t B, int32_t H, void* out, void* added, float* rstd,
+                                      int32_t dtype, void* stream);
+int ck_fused_residual_add_rmsnorm_bwd(const void* added, const void* weight, const void* d_out, const void* d_added,
+                                      const float* rstd, float eps, float multiplier, int64_t B, int32_t H, void* d_x,
+                                      void* d_residual, float* d_weight_partial, float* d_weight, int32_t dtype,
+                                      void* stream);
+
 #ifdef __cplusplus
 }
 #endif
