@@ -96,8 +96,8 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_fwd_kernel(const T* __restrict
 #pragma unroll
         for (int i = 0; i < P; ++i) {
           float t = v.f[i];
-          if (fuse.multiplier != 1.0f) t = round_to<T>(t * fuse.multiplier);
-          v.f[i] = round_to<T>(t + r.f[i]);
+          if (fuse.multiplier != 1.0f) t = round_to<T>(__fmul_rn(t, fuse.multiplier));  // never contracted into an fma
+          v.f[i] = round_to<T>(__fadd_rn(t, r.f[i]));
         }
         v.store(ar + (int64_t)ch * P);
       }

@@ -41,6 +41,17 @@ def rmsnorm_torch(x: torch.Tensor, weight: torch.Tensor | None, eps: float | Non
     return F.rms_norm(x, (x.size(-1),), weight=weight, eps=eps)
 
 
+def fused_residual_add_rmsnorm_torch(
+    x: torch.Tensor, residual: torch.Tensor, weight: torch.Tensor | None, eps: float | None, multiplier: float | None = None
+) -> tuple[torch.Tensor, torch.Tensor]:
+    """cute_kernels/kernels/fused_residual_add_rmsnorm/torch_implementation.py:9-19: scale x (unless the multiplier is
+    None or 1), add the residual stream, return (rmsnorm of the sum, the sum)."""
+    if multiplier not in [None, 1]:
+        x = x * multiplier
+    x = x + residual
+    return rmsnorm_torch(x, weight, eps), x
+
+
 def topk_lowest_index_first(logits: torch.Tensor, k: int) -> tuple[torch.Tensor, torch.Tensor]:
     """Top-k with a fixed tie rule (equal logits: lowest expert index first). torch.topk's own tie order is
     unspecified (torch_implementation.py:195-201 just calls it); values are identical either way."""

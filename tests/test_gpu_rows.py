@@ -165,3 +165,56 @@ def test_rmsnorm_bf16_is_bit_exact_with_f_rms_norm_on_c4_rows(device):
     assert mismatch < 2e-3, mismatch  # rsqrt / summation-order differences flip at most a few roundings
     torch.testing.assert_close(z.cpu().float(), z_ref.float(), rtol=1e-2, atol=1e-2)
     assert cute_kernels.rmsnorm_cute(x.to(device), None, None).dtype == torch.bfloat16
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("has_weight", [True, False])
+@pytest.mark.parametrize("memory_efficient", [True, False])
+@pytest.mark.parametrize("multiplier", [None, 0.9])
+def test_fused_residual_add_rmsnorm_reference_grid(device, dtype, has_weight, memory_efficient, multiplier):
+    # reference grid fused_residual_add_rmsnorm_test.py:20-90 (fp32 there; bf16 added with bf16-sized bounds)
+    g = torch.Generator().manual_seed(42)
+    eps = 1e-5
+    for size in _rms_sizes():
+        x = torch.randn(size, generator=g).to(dtype)
+        r = torch.randn(size, generator=g).to(dtype)
+        w = torch.randn(size[-1], generator=g).to(dtype) if has_weight else None
+        xa, xc = x.clone().to(device).requires_grad_(), x.clone().requires_grad_()
+        ra, rc = r.clone().to(device).requires_grad_(), r.clone().requires_grad_()
+        wa = w.clone().to(device).requires_grad_() if has_weight else None
+        wc = w.clone().requires_grad_() if has_weight else None
+        z, added = cute_kernels.fused_residual_add_rmsnorm_cute(
+            x=xa, residual=ra, weight=wa, eps=eps, multiplier=multiplier, memory_efficient=memory_efficient
+        )
+        z_ref, added_ref = mo.fused_residual_add_rmsnorm_torch(xc, rc, wc, eps, multiplier)
+        # both outputs carry gradient, as in a transformer layer (the reference test does z * 2 + r * 3)
+        (z.float() * 2 + added.float() * 3).sum().backward()
+        (z_ref.float() * 2 + added_ref.float() * 3).sum().backward()
+        assert torch.equal(added.cpu(), added_ref)  # the residual stream is bit-exact: same roundings
+        if dtype == torch.float32:
+            torch.testing.assert_close(z.cpu(), z_ref, rtol=1.3e-6, atol=1e-5)
+            torch.testing.assert_close(xa.grad.cpu(), xc.grad, rtol=1e-4, atol=2e-4)
+            torch.testing.assert_close(ra.grad.cpu(), rc.grad, rtol=1e-4, atol=2e-4)
+            if has_weight:
+                torch.testing.assert_close(wa.grad.cpu(), wc.grad, rtol=1e-4, atol=4e-4 * max(1, size[0] if len(size) > 1 else 1) ** 0.5)
+        else:
+            torch.testing.assert_close(z.cpu(), z_ref, rtol=0, atol=6.3e-2)
+            torch.testing.assert_close(xa.grad.cpu(), xc.grad, rtol=2e-2, atol=0.72)
+            torch.testing.assert_close(ra.grad.cpu(), rc.grad, rtol=2e-2, atol=0.72)
+            if has_weight:
+                torch.testing.assert_close(wa.grad.cpu(), wc.grad, rtol=0.04, atol=1.0)
+
+
+def test_fused_residual_add_rmsnorm_without_residual_gradient(device):
+    # only the normalised output is used downstream: the residual-stream gradient is absent (None -> zeros)
+    g = torch.Generator().manual_seed(3)
+    x, r = torch.randn(64, 512, generator=g), torch.randn(64, 512, generator=g)
+    w = torch.randn(512, generator=g)
+    xa, ra, wa = (t.clone().to(device).requires_grad_() for t in (x, r, w))
+    xc, rc, wc = (t.clone().requires_grad_() for t in (x, r, w))
+    z, _ = cute_kernels.fused_residual_add_rmsnorm_cute(xa, ra, wa, 1e-6, 0.5)
+    z_ref, _ = mo.fused_residual_add_rmsnorm_torch(xc, rc, wc, 1e-6, 0.5)
+    z.square().sum().backward()
+    z_ref.square().sum().backward()
+    for ours, ref in ((xa, xc), (ra, rc), (wa, wc)):
+        torch.testing.assert_close(ours.grad.cpu(), ref.grad, rtol=1e-4, atol=1e-3)

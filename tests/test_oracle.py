@@ -224,3 +224,23 @@ def test_moe_oracle_state_dict_keys_and_shapes():
     assert sd["c_fc.weight"].shape == (4, 48, 16)  # 2*I rows when is_glu
     assert sd["c_proj.weight"].shape == (4, 16, 24)
     assert abs(float(sd["c_fc.weight"].std()) - 0.02) < 0.005
+
+
+def test_fused_residual_add_rmsnorm_closed_form():
+    g = torch.Generator().manual_seed(5)
+    x, r = torch.randn(7, 33, generator=g, dtype=torch.float64), torch.randn(7, 33, generator=g, dtype=torch.float64)
+    w = torch.randn(33, generator=g, dtype=torch.float64)
+    for mult in (None, 1, 0.9):
+        y, added = mo.fused_residual_add_rmsnorm_torch(x, r, w, 1e-5, mult)
+        a = x * (1.0 if mult is None else mult) + r  # written out, not through the oracle
+        torch.testing.assert_close(added, a, rtol=0, atol=0)
+        expect = a / torch.sqrt((a * a).mean(-1, keepdim=True) + 1e-5) * w
+        torch.testing.assert_close(y, expect, rtol=1e-12, atol=1e-12)
+    # a dropped multiplier or a swapped operand would show: y depends on x only through mult * x + r
+    y1, _ = mo.fused_residual_add_rmsnorm_torch(x, r, None, 1e-5, 0.5)
+    y2, _ = mo.fused_residual_add_rmsnorm_torch(0.5 * x, r, None, 1e-5, None)
+    torch.testing.assert_close(y1, y2, rtol=1e-12, atol=1e-12)
+    # the 16-bit path rounds the scaled x and the sum separately
+    xb, rb = x.to(torch.bfloat16), r.to(torch.bfloat16)
+    _, added_b = mo.fused_residual_add_rmsnorm_torch(xb, rb, None, 1e-5, 0.9)
+    assert torch.equal(added_b, ((xb.float() * 0.9).to(torch.bfloat16).float() + rb.float()).to(torch.bfloat16))
