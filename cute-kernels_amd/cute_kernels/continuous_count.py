@@ -10,6 +10,8 @@ import torch
 
 from . import _C
 
+_ops = None  # cute_kernels.compile_ops, set by the package once it is imported (used only while torch.compile traces)
+
 
 def _launch(x: torch.Tensor, size: int, want_offsets: bool):
     _C.require_gpu(x)
@@ -47,6 +49,8 @@ def continuous_count_cute(x: torch.Tensor, size: int) -> torch.Tensor:
     assert x.dim() == 1, "x should be 1-dimensional"
     assert x.dtype in [torch.int32, torch.long]
 
+    if torch.compiler.is_compiling():
+        return _ops.continuous_count(x, size)
     return _launch(x, size, want_offsets=False)[0]
 
 

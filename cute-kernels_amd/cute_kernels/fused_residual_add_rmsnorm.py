@@ -12,6 +12,8 @@ import torch
 from . import _C
 from .utils import get_num_elements_and_hidden_size
 
+_ops = None  # cute_kernels.compile_ops, set by the package once it is imported (used only while torch.compile traces)
+
 
 class _FusedResidualAddRMSNorm_Cute(torch.autograd.Function):
     @staticmethod
@@ -109,4 +111,16 @@ def fused_residual_add_rmsnorm_cute(
     Returns:
         tuple[torch.Tensor, torch.Tensor]: output activations, updated residual stream
     """
+    if torch.compiler.is_compiling():
+        if weight is not None:
+            assert weight.dim() == 1, "weight should be 1D"
+            assert weight.size(-1) == x.size(-1), "hidden size for x and weight tensor is different"
+            assert weight.dtype == x.dtype, "tensors weight and y should have same dtype"
+        assert residual.shape == x.shape and residual.dtype == x.dtype, "x and residual should match"
+        if eps is None:
+            eps = torch.finfo(x.dtype).eps
+        output, added_x_residual, _ = _ops.fused_residual_add_rmsnorm(
+            x, residual, weight, eps, 1.0 if multiplier is None else float(multiplier), memory_efficient
+        )
+        return output, added_x_residual
     return _FusedResidualAddRMSNorm_Cute.apply(x, residual, weight, eps, multiplier, memory_efficient)

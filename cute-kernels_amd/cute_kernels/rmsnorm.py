@@ -11,6 +11,8 @@ import torch
 from . import _C
 from .utils import get_num_elements_and_hidden_size
 
+_ops = None  # cute_kernels.compile_ops, set by the package once it is imported (used only while torch.compile traces)
+
 
 class _RMSNorm_Cute(torch.autograd.Function):
     @staticmethod
@@ -84,4 +86,12 @@ def rmsnorm_cute(
     Returns:
         torch.Tensor: output tensor
     """
+    if torch.compiler.is_compiling():
+        if weight is not None:
+            assert weight.dim() == 1, "weight should be 1D"
+            assert weight.size(-1) == x.size(-1), "hidden size for x and weight tensor is different"
+            assert weight.dtype == x.dtype, "tensors weight and y should have same dtype"
+        if eps is None:
+            eps = torch.finfo(x.dtype).eps
+        return _ops.rmsnorm(x, weight, eps, memory_efficient)[0]
     return _RMSNorm_Cute.apply(x, weight, eps, memory_efficient)

@@ -16,6 +16,8 @@ import torch
 
 from . import _C
 
+_ops = None  # cute_kernels.compile_ops, set by the package once it is imported (used only while torch.compile traces)
+
 
 # ---------------------------------------------------------------------------------------------------------------
 # routing
@@ -64,6 +66,9 @@ class _RouteTopKSoftmax(torch.autograd.Function):
 def route_topk_softmax(logits: torch.Tensor, k: int) -> tuple[torch.Tensor, torch.Tensor]:
     """Top-k over the logits and softmax over the k selected logits in fp32, cast back to logits.dtype
     (torch_implementation.py:122-135). Equal logits: the lowest expert index wins."""
+    if torch.compiler.is_compiling():
+        gates, selected = _ops.route_topk_softmax(logits, k)
+        return gates.to(logits.dtype), selected.long()
     return _RouteTopKSoftmax.apply(logits, k)
 
 
@@ -133,12 +138,18 @@ def choose_align(num_rows: int, num_experts: int) -> int:
 @torch.no_grad()
 def sort_by_expert(expert_ids: torch.Tensor, num_experts: int, align: int | None = None) -> ExpertSegments:
     """Stable sort of the flat (token, slot) expert ids, with counts / offsets and the tile-aligned segment tables."""
-    _C.require_gpu(expert_ids)
     assert expert_ids.dtype in (torch.int32, torch.long)
+    if align is None:
+        align = choose_align(expert_ids.numel(), num_experts)
+    if torch.compiler.is_compiling():
+        return _ops.sort_by_expert_segments(expert_ids, num_experts, align)
+    return _sort_by_expert_eager(expert_ids, num_experts, align)
+
+
+def _sort_by_expert_eager(expert_ids: torch.Tensor, num_experts: int, align: int) -> ExpertSegments:
+    _C.require_gpu(expert_ids)
     ids = expert_ids.contiguous().view(-1)
     R = ids.numel()
-    if align is None:
-        align = choose_align(R, num_experts)
     lib = _C.lib()
     dev = ids.device
     max_rows = lib.ck_sort_max_rows(R, num_experts, align)
@@ -376,14 +387,23 @@ class _ExpertsDown(torch.autograd.Function):
 
 
 def experts_up(x: torch.Tensor, weight: torch.Tensor, seg: ExpertSegments, k: int) -> torch.Tensor:
-    _C.require_gpu(x, weight)
     _check_expert_dtypes(x, weight)
+    if torch.compiler.is_compiling():
+        return _ops.experts_up(
+            x, weight, seg.seg_starts, seg.counts, seg.tile_expert, seg.row_slot, seg.max_rows, seg.num_experts, seg.align, k
+        )
+    _C.require_gpu(x, weight)
     return _ExpertsUp.apply(x, weight, seg, k)
 
 
 def experts_down(h: torch.Tensor, weight: torch.Tensor, gates: torch.Tensor, seg: ExpertSegments) -> torch.Tensor:
-    _C.require_gpu(h, weight, gates)
     _check_expert_dtypes(h, weight)
+    if torch.compiler.is_compiling():
+        return _ops.experts_down(
+            h, weight, gates.to(h.dtype), seg.seg_starts, seg.counts, seg.tile_expert, seg.row_slot, seg.max_rows,
+            seg.num_experts, seg.align,
+        )[0]
+    _C.require_gpu(h, weight, gates)
     return _ExpertsDown.apply(h, weight, gates.to(h.dtype), seg)
 
 
@@ -479,7 +499,14 @@ def swiglu_experts(
     x: torch.Tensor, w_fc: torch.Tensor, w_proj: torch.Tensor, gates: torch.Tensor, seg: ExpertSegments
 ) -> torch.Tensor:
     """Fused expert block for `activation_function = swiglu_packed_cute`, `is_glu=True` (c_fc columns [up | gate])."""
-    _C.require_gpu(x, w_fc, w_proj, gates)
     _check_expert_dtypes(x, w_fc, w_proj)
     assert w_fc.size(1) % 16 == 0, "intermediate size should be a multiple of 8"
+    if torch.compiler.is_compiling():
+        grad = torch.is_grad_enabled()
+        return _ops.swiglu_experts(
+            x, w_fc, w_proj, gates.to(x.dtype), seg.seg_starts, seg.counts, seg.tile_expert, seg.row_slot, seg.max_rows,
+            seg.num_experts, seg.align, grad and x.requires_grad, grad and w_fc.requires_grad,
+            grad and w_proj.requires_grad, grad and gates.requires_grad,
+        )[0]
+    _C.require_gpu(x, w_fc, w_proj, gates)
     return _SwigluExperts.apply(x, w_fc, w_proj, gates.to(x.dtype), seg)

@@ -10,6 +10,8 @@ import torch
 from . import _C
 from .utils import divide_if_divisible
 
+_ops = None  # cute_kernels.compile_ops, set by the package once it is imported (used only while torch.compile traces)
+
 
 def _rows_cols(x: torch.Tensor) -> tuple[int, int]:
     cols = x.size(-1) if x.dim() > 0 else 1
@@ -109,6 +111,10 @@ def swiglu_cute(
     Returns:
         torch.Tensor: output tensor
     """
+    if torch.compiler.is_compiling():
+        assert gate.size() == up.size(), "tensors gate and up should have same shape"
+        assert gate.dtype == up.dtype, "tensors gate and up should have same dtype"
+        return _ops.swiglu(gate, up)
     return _Swiglu_Cute.apply(gate, up)
 
 
@@ -122,4 +128,7 @@ def swiglu_packed_cute(x: torch.Tensor) -> torch.Tensor:
     Returns:
         torch.Tensor: output tensor
     """
+    if torch.compiler.is_compiling():
+        divide_if_divisible(x.size(-1), 2)
+        return _ops.swiglu_packed(x)
     return _SwigluPacked_Cute.apply(x)

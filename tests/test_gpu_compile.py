@@ -1,0 +1,71 @@
+"""Compiled (torch.compile, fullgraph=True) versus eager, on the GPU: same kernels behind registered ops, so results are
+bit-identical. Backend "aot_eager": the graph is captured and partitioned by AOT autograd, nothing is re-generated
+(the reference's tests compile every op with fullgraph=True, e.g. scattermoe_test.py:80-81, rmsnorm_test.py:34)."""
+
+import pytest
+import torch
+
+import cute_kernels as ck
+
+pytestmark = pytest.mark.gpu
+
+
+def _compile(fn):
+    return torch.compile(fn, fullgraph=True, backend="aot_eager")
+
+
+def test_count_compiled(device):
+    ids = torch.randint(0, 64, (65536,), dtype=torch.int32, device=device)
+    out = _compile(lambda i: ck.continuous_count_cute(i, 64))(ids)
+    assert out.dtype == torch.uint32 and torch.equal(out.cpu().long(), torch.bincount(ids.cpu().long(), minlength=64))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu_and_norms_compiled(device, dtype):
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn(300, 512, generator=g).to(dtype).to(device)
+    y = torch.randn(300, 512, generator=g).to(dtype).to(device)
+    w = torch.randn(512, generator=g).to(dtype).to(device)
+    cases = {
+        "swiglu": (lambda a, b, c: ck.swiglu_cute(a, b), 2),
+        "swiglu_packed": (lambda a, b, c: ck.swiglu_packed_cute(a), 1),
+        "rmsnorm": (lambda a, b, c: ck.rmsnorm_cute(a, c, 1e-5), 3),
+        "rmsnorm_me": (lambda a, b, c: ck.rmsnorm_cute(a, None, None, memory_efficient=True), 1),
+        "frn": (lambda a, b, c: sum(t.float() for t in ck.fused_residual_add_rmsnorm_cute(a, b, c, 1e-5, 0.9)), 3),
+        "frn_me": (lambda a, b, c: ck.fused_residual_add_rmsnorm_cute(a, b, None, 1e-5, None, True)[0], 2),
+    }
+    for name, (fn, _) in cases.items():
+        eager_in = [t.clone().requires_grad_() for t in (x, y, w)]
+        comp_in = [t.clone().requires_grad_() for t in (x, y, w)]
+        z = fn(*eager_in)
+        zc = _compile(fn)(*comp_in)
+        assert torch.equal(z, zc), name
+        z.float().square().sum().backward()
+        zc.float().square().sum().backward()
+        for a, b in zip(eager_in, comp_in):
+            assert (a.grad is None) == (b.grad is None), name
+            if a.grad is not None:
+                assert torch.equal(a.grad, b.grad), name
+
+
+@pytest.mark.parametrize("act,is_glu", [(ck.swiglu_packed_cute, True), (torch.nn.GLU(), True), (torch.nn.GELU("tanh"), False)])
+def test_moe_layer_compiled(device, act, is_glu):
+    torch.manual_seed(1)
+    moe = ck.MoE(8, 2, 128, 256, act, is_glu, False, 0.02).to(torch.bfloat16).to(device)
+    x = torch.randn(512, 128, dtype=torch.bfloat16, device=device)
+    xe, xc = x.clone().requires_grad_(), x.clone().requires_grad_()
+    y, logits = moe(xe)
+    y.float().square().sum().backward()
+    eager_grads = {n: p.grad.clone() for n, p in moe.named_parameters()}
+    for p in moe.parameters():
+        p.grad = None
+    compiled = _compile(moe)
+    yc, logits_c = compiled(xc)
+    yc.float().square().sum().backward()
+    assert torch.equal(y, yc) and torch.equal(logits, logits_c)
+    assert torch.equal(xe.grad, xc.grad)
+    for n, p in moe.named_parameters():
+        assert torch.equal(eager_grads[n], p.grad), n
+    # inference: nothing is saved, nothing breaks
+    with torch.no_grad():
+        assert torch.equal(compiled(x)[0], moe(x)[0])
