@@ -144,7 +144,7 @@ __global__ __launch_bounds__(kBlock) void count_kernel(const id_t* __restrict__ 
     for (int u = 0; u < UNROLL; ++u) {
       const int64_t vi = (it * UNROLL + u) * gthreads + gtid;
       ok[u] = vi < nvec;
-      v[u] = ok[u] ? load16(body + vi * VEC) : zero16();
+      v[u] = ok[u] ? load16_nt(body + vi * VEC) : zero16();  // ids are read once
     }
 #pragma unroll
     for (int u = 0; u < UNROLL; ++u) {
@@ -375,15 +375,19 @@ extern "C" int ck_count_offsets(const void* ids, int32_t ids_are_i64, int64_t n,
   CK_REQUIRE((reinterpret_cast<uintptr_t>(ids) & (esz - 1)) == 0, "ck_count_offsets: ids is not element-aligned");
 
   const int64_t vec = 16 / (int64_t)esz;
-  // 4 vectors per thread per trip; enough blocks to fill 256 CUs a few times over, one block for small inputs
+  // 4 vectors per thread per trip; one block for small inputs. Large inputs: 2 blocks per CU stream fastest with the LDS
+  // path (6.5 TB/s at 512 blocks, 6.1 at 1024, 3.7 at 256); the ballot path is VALU-heavier and wants 4 per CU.
   int64_t blocks = ceil_div(n, (int64_t)kBlock * vec * 4 * 4);
   if (blocks < 1) blocks = 1;
-  if (blocks > 1024) blocks = 1024;  // 4 per CU: 16 waves per CU keep HBM busy, and the merge stays short
+  const int64_t max_blocks = num_bins <= 8 ? 1024 : 512;
+  if (blocks > max_blocks) blocks = max_blocks;
   if (const char* env = getenv("CK_COUNT_BLOCKS")) {  // tuning knob for measurements
     const long v = atol(env);
     if (v >= 1 && v <= 65535) blocks = v;
   }
-  const int reg_bins = num_bins <= 8 ? 8 : (num_bins <= 16 ? 16 : 0);
+  // up to 8 bins: ballot counters in registers (5.8 TB/s; LDS atomics on so few addresses serialise: 2.1-5.1 TB/s);
+  // more bins: LDS atomics (6.3-6.5 TB/s; 16 register counters measured 3.3 TB/s)
+  const int reg_bins = num_bins <= 8 ? 8 : 0;  // 16 register counters measured slower (3.3 TB/s) than LDS atomics (5.6)
   const int copies = reg_bins > 0 ? 1 : (num_bins <= 1024 ? kWavesPerBlock : 1);
   const size_t lds_bytes = ((size_t)copies * num_bins + kWavesPerBlock + 2) * sizeof(uint32_t);
   hipStream_t s = static_cast<hipStream_t>(stream);
@@ -393,11 +397,9 @@ extern "C" int ck_count_offsets(const void* ids, int32_t ids_are_i64, int64_t n,
                      starts, workspace)
   if (ids_are_i64) {
     if (reg_bins == 8) CK_LAUNCH_COUNT(int64_t, 8);
-    else if (reg_bins == 16) CK_LAUNCH_COUNT(int64_t, 16);
     else CK_LAUNCH_COUNT(int64_t, 0);
   } else {
     if (reg_bins == 8) CK_LAUNCH_COUNT(int32_t, 8);
-    else if (reg_bins == 16) CK_LAUNCH_COUNT(int32_t, 16);
     else CK_LAUNCH_COUNT(int32_t, 0);
   }
 #undef CK_LAUNCH_COUNT

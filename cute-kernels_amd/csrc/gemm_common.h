@@ -6,7 +6,6 @@
 #include "ck_common.h"
 
 namespace ck {
-namespace {
 
 constexpr int kXcds = 8;
 
@@ -38,6 +37,30 @@ struct GemmParams {
   const void* aux_in;
   const float* a_scale;  // fp8 only: per-row dequantisation scale of a (indexed like the rows of a)
   const float* w_scale;  // fp8 only: per-output-channel scale of w, [E, N]
+};
+
+// The 256 x 384 tile variant of the 16-bit kernel (grouped_gemm_wide.hip): modes kGrouped, kScatter, kSwiglu, kDw.
+// The caller fills `prm` for these tile dimensions (n_tiles, m_tiles) and sizes the grid accordingly.
+constexpr int kWideBM = 256, kWideBN = 384;
+int launch_wide(const GemmParams& prm, int mode, int dtype, unsigned blocks, hipStream_t stream, const char* name);
+
+namespace {
+
+template <typename T>
+struct Mfma;
+template <>
+struct Mfma<bf16_t> {
+  typedef bf16x8 frag;
+  __device__ static inline f32x16 run(const frag& a, const frag& b, const f32x16& c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <>
+struct Mfma<f16_t> {
+  typedef f16x8 frag;
+  __device__ static inline f32x16 run(const frag& a, const frag& b, const f32x16& c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+  }
 };
 
 // f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant expression

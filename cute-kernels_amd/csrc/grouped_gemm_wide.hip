@@ -1,0 +1,422 @@
+// 256 x 384 tile variant of the scattered grouped GEMM (bf16 / f16 inputs, fp32 accumulation).
+//
+// Why a wider tile: the 256 x 256 kernel is bound by L2 -> LDS load throughput, and a tile's FLOPs per loaded byte are
+// BM*BN / (BM + BN): 128 at 256 x 256, 153.6 here. The accumulators (384 fp32 registers per lane) only fit with one wave
+// per SIMD, so the workgroup is 4 waves in a 2 x 2 grid with 128 x 192 wave tiles = 4 x 6 v_mfma_f32_32x32x16 blocks.
+//
+// Pipeline: K step 32 (64-byte LDS rows, XOR-swizzled), operands go global -> LDS directly (global_load_lds_dwordx4),
+// four stages of 40 KiB = the whole 160 KiB of LDS, loads issued 2.5 steps ahead and never past the last step. Fragments
+// are single-buffered and rotate: a register set is reloaded for the next 16-wide K slice as soon as the last MFMA that
+// reads it has issued (A row blocks free up one by one, B column blocks during the last A row block).
+#include <stdlib.h>
+
+#include "gemm_common.h"
+
+namespace ck {
+namespace {
+
+constexpr int BM = kWideBM, BN = kWideBN;
+#ifndef CK_WIDE_WGM
+#define CK_WIDE_WGM 4
+#endif
+constexpr int WGM = CK_WIDE_WGM;           // waves along M (always 2 along N)
+constexpr int NW = 2 * WGM, NT = 64 * NW;
+constexpr int WM = BM / WGM, WN = BN / 2;  // wave tile
+constexpr int MI = WM / 32, NI = WN / 32;
+constexpr int BK = 32, KS = BK / 16, NSTAGE = 4;
+constexpr int kRowBytes = BK * 2;
+constexpr int kStageBytes = (BM + BN) * kRowBytes;
+constexpr int A_LD = BM / (16 * NW), B_LD = BN / (16 * NW);  // 1 KiB wave-loads per wave and K step
+constexpr int kLoadsPerStep = A_LD + B_LD;
+constexpr size_t kLdsBytes = (size_t)NSTAGE * kStageBytes;
+// epilogue: slab of half the tile's columns (3 of each wave's 6 column blocks), kept transposed S[col][row]
+constexpr int kSlabBlocks = NI / 2, kSlabCols = 2 * kSlabBlocks * 32, kSlabLd = BM + 4;
+constexpr int kMetaOffset = kSlabCols * kSlabLd * 2;  // after the slab: output row of every tile row (scatter)
+static_assert(kLdsBytes == 160 * 1024, "four stages fill the LDS of a CU");
+static_assert(kMetaOffset % 16 == 0 && kMetaOffset + BM * 4 <= (int)kLdsBytes, "slab and row table fit in the dead stages");
+static_assert(kLoadsPerStep <= (MI > 2 ? (MI - 2) * NI : NI), "every load of a step has an MFMA to hide behind");
+
+template <typename T, int MODE>
+__global__ __launch_bounds__(NT) void grouped_gemm_wide_kernel(const GemmParams prm) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
+  char* lds_c = reinterpret_cast<char*>(lds_raw);
+  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // ---- which tile (same XCD-aware orders as the 256 x 256 kernel)
+  int mt, nt, expert;
+  int64_t k_begin = 0;
+  int k_len;
+  if constexpr (MODE == kDw) {
+    const int per_expert = prm.m_tiles * prm.n_tiles;
+    const bool m_major = prm.m_tiles >= prm.n_tiles;
+    const int major = m_major ? prm.m_tiles : prm.n_tiles, minor = m_major ? prm.n_tiles : prm.m_tiles;
+    int pid = blockIdx.x, a, b;
+    if (major % kXcds == 0) {  // every XCD gets a slice of every expert's tile grid (experts differ in contraction length)
+      const int xcd = pid % kXcds, j = pid / kXcds;
+      const int slice = major / kXcds, per_slice = slice * minor;
+      expert = j / per_slice;
+      grouped_order(j - expert * per_slice, slice, minor, a, b);
+      a += xcd * slice;
+    } else {
+      expert = pid / per_expert;
+      grouped_order(pid - expert * per_expert, major, minor, a, b);
+    }
+    mt = m_major ? a : b;
+    nt = m_major ? b : a;
+    k_begin = prm.seg_starts[expert];
+    k_len = (int)((prm.counts[expert] + BK - 1) / BK * BK);  // the transposed operands are zero up to the tile boundary
+  } else {
+    const int live_m = prm.seg_starts[prm.num_experts] / prm.align;
+    const int total = live_m * prm.n_tiles;
+    int pid = blockIdx.x;
+    if (pid >= total) return;
+    const int per_xcd = total / kXcds;
+    if (pid < per_xcd * kXcds) pid = (pid % kXcds) * per_xcd + pid / kXcds;
+    grouped_order(pid, live_m, prm.n_tiles, mt, nt);
+    expert = prm.tile_expert[mt];
+    k_len = prm.K;
+  }
+  const int64_t m0 = (int64_t)mt * BM;
+  int64_t valid_end = 0;  // forward modes: first pad row of this expert's segment
+  if constexpr (MODE != kDw) valid_end = (int64_t)prm.seg_starts[expert] + prm.counts[expert];
+  // scatter epilogue: the output row of tile row `tid`, fetched now and parked in LDS once the main loop is over
+  int scatter_row = -1;
+  if constexpr (MODE == kScatter) {
+    if (tid < BM && m0 + tid < valid_end) scatter_row = prm.row_slot[m0 + tid];
+  }
+  static_assert(NT >= BM, "one thread per tile row");
+
+  f32x16 acc[MI][NI];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NI; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // ---- global -> LDS addressing: lane l of a wave-load fills slot l (16 bytes) of 64 consecutive slots = 16 rows
+  const char* a_base = static_cast<const char*>(prm.a);
+  const char* b_base = static_cast<const char*>(prm.w);
+  if constexpr (MODE != kDw) b_base += (int64_t)expert * prm.w_expert_stride * 2;
+  uint32_t a_off[A_LD], b_off[B_LD];
+#pragma unroll
+  for (int t = 0; t < A_LD; ++t) {
+    const int r = (wave * A_LD + t) * 16 + (lane >> 2);
+    const int c = (lane & 3) ^ lds_swizzle(r);
+    int64_t row;
+    if constexpr (MODE == kDw) {
+      row = min(m0 + r, (int64_t)prm.M - 1);
+    } else {
+      int64_t p = m0 + r;
+      if (p >= valid_end) p = valid_end - 1;  // pad rows re-read a valid row; their results are never stored
+      row = prm.a_gather_div > 0 ? (int64_t)(prm.row_slot[p] / prm.a_gather_div) : p;
+    }
+    a_off[t] = (uint32_t)((row * prm.lda + k_begin) * 2 + c * 16);
+  }
+#pragma unroll
+  for (int t = 0; t < B_LD; ++t) {
+    const int j = (wave * B_LD + t) * 16 + (lane >> 2);
+    const int c = (lane & 3) ^ lds_swizzle(j);
+    int64_t n;
+    if constexpr (MODE == kSwiglu) {  // a wave's 192 tile columns: 96 up columns, then the 96 gate columns of the same outputs
+      const int half = (j % WN) / (WN / 2);
+      const int within = (j / WN) * (WN / 2) + (j % (WN / 2));
+      n = (int64_t)half * prm.I + min((int64_t)nt * (BN / 2) + within, (int64_t)prm.I - 1);
+    } else {
+      n = min((int64_t)nt * BN + j, (int64_t)prm.N - 1);
+    }
+    b_off[t] = (uint32_t)((n * prm.ldw + k_begin) * 2 + c * 16);
+  }
+  const int nk = k_len / BK;
+
+  auto dma16 = [&](const char* src, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(src) : "m0");
+  };
+  const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds_c;
+  const uint32_t wave_a = __builtin_amdgcn_readfirstlane(lds_base + wave * A_LD * 1024);
+  const uint32_t wave_b = __builtin_amdgcn_readfirstlane(lds_base + BM * kRowBytes + wave * B_LD * 1024);
+  auto issue_one = [&](int step, int g) {
+    const int64_t kb = (int64_t)min(step, nk - 1) * kRowBytes;  // only the prologue of a short contraction clamps
+    const uint32_t st = (uint32_t)((step & (NSTAGE - 1)) * kStageBytes);
+    if (g < A_LD) dma16(a_base + kb + a_off[g], wave_a + st + g * 1024);
+    else dma16(b_base + kb + b_off[g - A_LD], wave_b + st + (g - A_LD) * 1024);
+  };
+  auto issue = [&](int step) {
+#pragma unroll
+    for (int g = 0; g < kLoadsPerStep; ++g) issue_one(step, g);
+  };
+
+  // ---- fragments: slice sl of a row is its 16-byte chunks 2 sl (lanes 0-31) and 2 sl + 1 (lanes 32-63)
+  typedef typename Mfma<T>::frag frag_t;
+  const int fsw = lds_swizzle(lane & 31), fh = lane >> 5;
+  int slice_off[KS];
+#pragma unroll
+  for (int sl = 0; sl < KS; ++sl) slice_off[sl] = ((2 * sl + fh) ^ fsw) * 16;
+  const int fa_row = (wm * WM + (lane & 31)) * kRowBytes;
+  const int fb_row = BM * kRowBytes + (wn * WN + (lane & 31)) * kRowBytes;
+  frag_t fa[MI], fb[NI];
+  auto read_a = [&](int stage, int sl, int i) {
+    fa[i] = *reinterpret_cast<const frag_t*>(lds_c + stage * kStageBytes + slice_off[sl] + fa_row + i * 32 * kRowBytes);
+  };
+  auto read_b = [&](int stage, int sl, int j) {
+    fb[j] = *reinterpret_cast<const frag_t*>(lds_c + stage * kStageBytes + slice_off[sl] + fb_row + j * 32 * kRowBytes);
+  };
+  // 384 accumulator registers per lane do not fit one register class (256 AGPRs, 256 VGPRs): column blocks 0 .. 3 are
+  // pinned to AGPRs and 4, 5 to VGPRs through the operand constraints (left to itself the register allocator keeps all of
+  // them in AGPRs and shuttles the overflow through scratch). Successive MFMAs on one block are 23 MFMAs apart, far beyond
+  // the back-to-back dependency window, and the fragments come from LDS reads, which the wait-count pass tracks through
+  // the asm operands.
+  auto mfma = [&](int i, int j) {
+    if (j < 4) {
+      if constexpr (std::is_same<T, bf16_t>::value)
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fa[i]), "v"(fb[j]));
+      else
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fa[i]), "v"(fb[j]));
+    } else {
+      if constexpr (std::is_same<T, bf16_t>::value)
+        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc[i][j]) : "v"(fa[i]), "v"(fb[j]));
+      else
+        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc[i][j]) : "v"(fa[i]), "v"(fb[j]));
+    }
+  };
+
+  if (nk > 0) {
+    issue(0);
+    issue(1);
+    issue(2);
+    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * kLoadsPerStep) : "memory");  // step 0 landed, all waves
+#pragma unroll
+    for (int i = 0; i < MI; ++i) read_a(0, 0, i);
+#pragma unroll
+    for (int j = 0; j < NI; ++j) read_b(0, 0, j);
+
+    // One 16-wide slice: 24 MFMAs, A row block by A row block, and the reloads for the slice after it.
+    // second == false: slice 0 of step kt; the next slice is slice 1 of the same stage.
+    // second == true:  slice 1 of step kt; the next slice is slice 0 of step kt + 1, whose stage must have landed for
+    //                  every wave -- wait + barrier after the first A row block, then the loads of step kt + 3 (phase 0)
+    //                  go out under the MFMAs of the middle A row blocks. The stage they overwrite, (kt + 3) % 4, was last
+    //                  read as slice 1 of step kt - 1, consumed by every wave before it reached this barrier.
+    // phase 0: steady state; 1: step nk - 3 (nothing left to fetch, two steps in flight); 2: last two steps (wait for all)
+    auto slice = [&](int kt, auto second, auto phase) {
+      constexpr bool kSecond = decltype(second)::value;
+      constexpr int kPhase = decltype(phase)::value;
+      const int ns = kSecond ? (kt + 1) & (NSTAGE - 1) : kt & (NSTAGE - 1);
+      const int nsl = kSecond ? 0 : 1;
+#pragma unroll
+      for (int j = 0; j < NI; ++j) mfma(0, j);
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (kSecond) {
+        if constexpr (kPhase == 2) asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kLoadsPerStep) : "memory");
+      }
+      read_a(ns, nsl, 0);
+#pragma unroll
+      for (int i = 1; i + 1 < MI; ++i) {
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+          mfma(i, j);
+          if constexpr (MI > 2 && kSecond && kPhase == 0) {
+            if ((i - 1) * NI + j < kLoadsPerStep) issue_one(kt + 3, (i - 1) * NI + j);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        read_a(ns, nsl, i);
+      }
+#pragma unroll
+      for (int j = 0; j < NI; ++j) {
+        mfma(MI - 1, j);
+        if constexpr (MI <= 2 && kSecond && kPhase == 0) {
+          if (j < kLoadsPerStep) issue_one(kt + 3, j);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        read_b(ns, nsl, j);
+      }
+      read_a(ns, nsl, MI - 1);
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    auto k_step = [&](int kt, auto phase) {
+      slice(kt, std::false_type{}, phase);
+      slice(kt, std::true_type{}, phase);
+    };
+    int kt = 0;
+    for (; kt + 3 < nk; ++kt) k_step(kt, std::integral_constant<int, 0>{});
+    if (kt + 3 == nk) k_step(kt++, std::integral_constant<int, 1>{});
+    for (; kt < nk; ++kt) k_step(kt, std::integral_constant<int, 2>{});
+  }
+
+  // ---- epilogue through LDS. Lane holds, per 32x32 block and q in 0..3, rows 8q + 4*(lane/32) + 0..3 of column lane%32:
+  // 8-byte writes into the transposed slab; ds_read_b64_tr_b16 brings row-major 16-byte pieces back out (a lane ends up
+  // with 8 consecutive columns of one row); transposed outputs leave with plain 16-byte reads.
+  typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4;
+  T* slab = reinterpret_cast<T*>(lds_raw);
+  int* scatter_rows = reinterpret_cast<int*>(lds_c + kMetaOffset);
+  // every wave is done with the stages; the no-ops cover the MFMA-result-to-VALU-read distance of the last MFMAs (18 wait
+  // states for a 16-pass MFMA), which the compiler cannot see through the asm
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier\n\ts_nop 15\n\ts_nop 7" ::: "memory");
+  if constexpr (MODE == kScatter) {
+    if (tid < BM) scatter_rows[tid] = scatter_row;  // first read after the first slab barrier below
+  }
+  const int col_in_block = lane & 31;
+  const int row_quad = (lane >> 5) * 4;
+  const T kZero = Elem<T>::down(0.f);
+
+  auto stage_blocks = [&](auto&& value /* (i, jj, q, s) -> T */) {
+    static_for<MI>([&](auto i) {
+      static_for<kSlabBlocks>([&](auto jj) {
+        static_for<4>([&](auto q) {
+          const int r = wm * WM + i * 32 + 8 * q + row_quad;
+          const int c = wn * (kSlabBlocks * 32) + jj * 32 + col_in_block;
+          store4(slab + c * kSlabLd + r, value(i, jj, q, std::integral_constant<int, 0>{}),
+                 value(i, jj, q, std::integral_constant<int, 1>{}), value(i, jj, q, std::integral_constant<int, 2>{}),
+                 value(i, jj, q, std::integral_constant<int, 3>{}));
+        });
+      });
+    });
+  };
+  // slab column -> column of the block tile, for pass `pass` (which half of each wave's column blocks is staged)
+  auto tile_col = [&](int sc, int pass) {
+    return (sc / (kSlabBlocks * 32)) * WN + pass * (kSlabBlocks * 32) + sc % (kSlabBlocks * 32);
+  };
+  auto drain_rows = [&](auto&& out_ptr /* (tile row, slab column) -> address of 8 output columns, or nullptr */) {
+    const int l16 = tid & 15, grp = tid >> 4;
+    const int tq = l16 & 3, tj = l16 >> 2;  // as a source lane: which slab column this lane points at
+    const int oq = l16 >> 2, oe = l16 & 3;  // as a destination lane: 8 columns oq of row oe of the 4 x 32 block
+    constexpr int kColBlocks = kSlabCols / 32;
+    constexpr int kBlocks = (BM / 4) * kColBlocks;
+#pragma unroll 4
+    for (int b = grp; b < kBlocks; b += NT / 16) {
+      const int rb = b / kColBlocks, cb = b % kColBlocks;
+      const T* src = slab + (cb * 32 + 8 * tq + tj) * kSlabLd + rb * 4;
+      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(src));
+      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(src + 4 * kSlabLd));
+      T* dst = out_ptr(rb * 4 + oe, cb * 32 + 8 * oq);
+      if (dst != nullptr) {
+        vec16 v;
+        v.w[0] = (uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
+        v.w[1] = (uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
+        v.w[2] = (uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
+        v.w[3] = (uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16);
+        store16(dst, v);
+      }
+    }
+  };
+  auto drain_cols = [&](auto&& out_ptr /* (slab column, tile row) -> address of 8 rows of that column, or nullptr */) {
+    constexpr int kChunks = kSlabCols * (BM / 8);
+#pragma unroll 4
+    for (int ch = tid; ch < kChunks; ch += NT) {
+      const int c = ch / (BM / 8), r = (ch % (BM / 8)) * 8;
+      T* dst = out_ptr(c, r);
+      if (dst != nullptr) store16(dst, load16(slab + c * kSlabLd + r));
+    }
+  };
+
+  if constexpr (MODE == kDw) {
+    T* dw = static_cast<T*>(prm.y) + (int64_t)expert * prm.M * prm.N;
+    static_for<2>([&](auto pass) {
+      stage_blocks([&](auto i, auto jj, auto q, auto s) {
+        return Elem<T>::down(acc[i][pass * kSlabBlocks + jj][4 * q + s]);
+      });
+      __syncthreads();
+      drain_rows([&](int r, int sc) -> T* {
+        const int64_t m = m0 + r, n = (int64_t)nt * BN + tile_col(sc, pass);
+        return (m < prm.M && n < prm.N) ? dw + m * prm.N + n : nullptr;
+      });
+      __syncthreads();
+    });
+  } else if constexpr (MODE == kGrouped || MODE == kScatter) {
+    T* y = static_cast<T*>(prm.y);
+    T* y_t = static_cast<T*>(prm.y_t);
+    static_for<2>([&](auto pass) {
+      // pad rows are staged as zeros: the transposed copy must hold zeros there
+      stage_blocks([&](auto i, auto jj, auto q, auto s) {
+        const int64_t p = m0 + wm * WM + i * 32 + 8 * q + row_quad + s;
+        return p < valid_end ? Elem<T>::down(acc[i][pass * kSlabBlocks + jj][4 * q + s]) : kZero;
+      });
+      __syncthreads();
+      drain_rows([&](int r, int sc) -> T* {
+        const int64_t p = m0 + r, n = (int64_t)nt * BN + tile_col(sc, pass);
+        if (p >= valid_end || n >= prm.N) return nullptr;
+        const int64_t row = (MODE == kScatter) ? (int64_t)scatter_rows[r] : p;
+        return y + row * prm.N + n;
+      });
+      if (MODE == kGrouped && y_t != nullptr) {
+        drain_cols([&](int sc, int r) -> T* {
+          const int64_t n = (int64_t)nt * BN + tile_col(sc, pass);
+          return n < prm.N ? y_t + n * prm.ld_t + m0 + r : nullptr;
+        });
+      }
+      __syncthreads();
+    });
+  } else {  // kSwiglu: column blocks 0 .. 2 of a wave are up, 3 .. 5 the gate of the same activation columns
+    T* pre = static_cast<T*>(prm.y);
+    T* act = static_cast<T*>(prm.aux);
+    T* act_t = static_cast<T*>(prm.y_t);
+    const int64_t two_i = 2 * (int64_t)prm.I;
+    auto act_col = [&](int sc) {
+      return (int64_t)nt * (BN / 2) + (sc / (kSlabBlocks * 32)) * (WN / 2) + sc % (kSlabBlocks * 32);
+    };
+    static_for<3>([&](auto pass) {  // 0: up half of the pre-activation, 1: gate half, 2: activation
+      stage_blocks([&](auto i, auto jj, auto q, auto s) {
+        const int64_t p = m0 + wm * WM + i * 32 + 8 * q + row_quad + s;
+        const T up = Elem<T>::down(acc[i][jj][4 * q + s]);
+        const T gate = Elem<T>::down(acc[i][jj + kSlabBlocks][4 * q + s]);
+        if (pass == 0) return up;
+        if (pass == 1) return gate;
+        const float gf = Elem<T>::up(gate);  // from the rounded pre-activation, like the unfused path
+        return p < valid_end ? Elem<T>::down(Elem<T>::up(up) * gf * sigmoid_fast(gf)) : kZero;
+      });
+      __syncthreads();
+      drain_rows([&](int r, int sc) -> T* {
+        const int64_t p = m0 + r, col = act_col(sc);
+        if (p >= valid_end || col >= prm.I) return nullptr;
+        if (pass == 0) return pre + p * two_i + col;
+        if (pass == 1) return pre + p * two_i + prm.I + col;
+        return act + p * prm.I + col;
+      });
+      if (pass == 2 && act_t != nullptr) {
+        drain_cols([&](int sc, int r) -> T* {
+          const int64_t col = act_col(sc);
+          return col < prm.I ? act_t + col * prm.ld_t + m0 + r : nullptr;
+        });
+      }
+      __syncthreads();
+    });
+  }
+}
+
+template <typename T, int MODE>
+int launch_mode(const GemmParams& prm, unsigned blocks, hipStream_t s, const char* name) {
+  auto kernel = grouped_gemm_wide_kernel<T, MODE>;
+  static bool attr_set = false;  // per instantiation; the attribute is idempotent, a race only repeats the call
+  if (!attr_set) {
+    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                       (int)kLdsBytes);
+    if (e != hipSuccess) {
+      set_error("%s: cannot reserve %zu bytes of LDS: %s", name, kLdsBytes, hipGetErrorString(e));
+      return CK_ERR_LAUNCH;
+    }
+    attr_set = true;
+  }
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(NT), kLdsBytes, s, prm);
+  CK_CHECK_LAUNCH(name);
+  return CK_OK;
+}
+
+}  // namespace
+
+int launch_wide(const GemmParams& prm, int mode, int dtype, unsigned blocks, hipStream_t stream, const char* name) {
+  CK_DISPATCH_HALF(dtype, name, {
+    switch (mode) {
+      case kGrouped: return launch_mode<scalar_t, kGrouped>(prm, blocks, stream, name);
+      case kScatter: return launch_mode<scalar_t, kScatter>(prm, blocks, stream, name);
+      case kSwiglu: return launch_mode<scalar_t, kSwiglu>(prm, blocks, stream, name);
+      case kDw: return launch_mode<scalar_t, kDw>(prm, blocks, stream, name);
+      default: break;
+    }
+  });
+  set_error("%s: the 256 x 384 tile has no epilogue %d", name, mode);
+  return CK_ERR_ARG;
+}
+
+}  // namespace ck

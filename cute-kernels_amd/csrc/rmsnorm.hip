@@ -26,6 +26,19 @@ struct Vec {
     }
     return v;
   }
+  // for rows that are read exactly once (non-temporal)
+  __device__ static inline Vec load_once(const T* p) {
+    Vec v;
+    if constexpr (P == 1) {
+      v.f[0] = Elem<T>::up(*p);
+    } else {
+      Pack16<T> k;
+      k.v = load16_nt(p);
+#pragma unroll
+      for (int i = 0; i < P; ++i) v.f[i] = Elem<T>::up(k.e[i]);
+    }
+    return v;
+  }
   __device__ static inline Vec ones() {
     Vec v;
 #pragma unroll
@@ -39,7 +52,7 @@ struct Vec {
       Pack16<T> k;
 #pragma unroll
       for (int i = 0; i < P; ++i) k.e[i] = Elem<T>::down(f[i]);
-      store16(p, k.v);
+      store16_nt(p, k.v);
     }
   }
 };
@@ -90,9 +103,10 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_fwd_kernel(const T* __restrict
     T* ar = fuse.residual ? fuse.added + row * H : nullptr;
     // the row to normalise: x, or the freshly written sum with the residual stream
     auto load_x = [&](int ch) {
-      Vec<T, P> v = Vec<T, P>::load(xr + (int64_t)ch * P);
+      // cached rows (NC > 0) are read once; streaming rows come back for the second pass
+      Vec<T, P> v = NC > 0 ? Vec<T, P>::load_once(xr + (int64_t)ch * P) : Vec<T, P>::load(xr + (int64_t)ch * P);
       if (rr != nullptr) {
-        const Vec<T, P> r = Vec<T, P>::load(rr + (int64_t)ch * P);
+        const Vec<T, P> r = Vec<T, P>::load_once(rr + (int64_t)ch * P);
 #pragma unroll
         for (int i = 0; i < P; ++i) {
           float t = v.f[i];
@@ -188,7 +202,7 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const T* __restrict
     // o = gradient w.r.t. the normalised row; with the fusion add the residual stream's gradient, emit both outputs
     auto finish = [&](Vec<T, P>& o, int ch) {
       if (fuse.d_added != nullptr) {
-        const Vec<T, P> a = Vec<T, P>::load(fuse.d_added + row * H + (int64_t)ch * P);
+        const Vec<T, P> a = Vec<T, P>::load_once(fuse.d_added + row * H + (int64_t)ch * P);
 #pragma unroll
         for (int i = 0; i < P; ++i) o.f[i] += a.f[i];
       }
@@ -206,8 +220,8 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const T* __restrict
       for (int c = 0; c < NC; ++c) {
         const int ch = c * TPR + lane;
         if (ch < chunks) {
-          xv[c] = Vec<T, P>::load(xr + (int64_t)ch * P);
-          gv[c] = Vec<T, P>::load(gr + (int64_t)ch * P);
+          xv[c] = Vec<T, P>::load_once(xr + (int64_t)ch * P);
+          gv[c] = Vec<T, P>::load_once(gr + (int64_t)ch * P);
           const Vec<T, P> wv = weight ? Vec<T, P>::load(weight + (int64_t)ch * P) : Vec<T, P>::ones();
 #pragma unroll
           for (int i = 0; i < P; ++i) {

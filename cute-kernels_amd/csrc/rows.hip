@@ -35,7 +35,7 @@ __global__ __launch_bounds__(kBlock) void gather_rows_kernel(const T* __restrict
       // the product is rounded to the tensor dtype, as the reference's gather does (kernels.py:268-273)
       v = scale16<T>(v, Elem<T>::up(coeff[slot]));
     }
-    store16(out + c * P, v);
+    store16_nt(out + c * P, v);
   }
 }
 
@@ -55,7 +55,7 @@ __global__ __launch_bounds__(kBlock) void combine_rows_kernel(const T* __restric
     for (int i = 0; i < P; ++i) acc[i] = 0.f;
     for (int j = 0; j < k; ++j) {
       Pack16<T> p;
-      p.v = load16(expanded + ((t * k + j) * chunks_per_row + ch) * P);
+      p.v = load16_nt(expanded + ((t * k + j) * chunks_per_row + ch) * P);  // read once
       const float g = gates ? Elem<T>::up(gates[t * k + j]) : 1.0f;
 #pragma unroll
       for (int i = 0; i < P; ++i) acc[i] += g * Elem<T>::up(p.e[i]);
@@ -63,7 +63,7 @@ __global__ __launch_bounds__(kBlock) void combine_rows_kernel(const T* __restric
     Pack16<T> o;
 #pragma unroll
     for (int i = 0; i < P; ++i) o.e[i] = Elem<T>::down(acc[i]);
-    store16(out + c * P, o.v);
+    store16_nt(out + c * P, o.v);
   }
 }
 
@@ -80,7 +80,7 @@ __global__ __launch_bounds__(kBlock) void gate_grad_kernel(const T* __restrict__
   float acc = 0.f;
   for (int ch = lane; ch < chunks_per_row; ch += kWave) {
     Pack16<T> a, b;
-    a.v = load16(expanded + (pair * chunks_per_row + ch) * P);
+    a.v = load16_nt(expanded + (pair * chunks_per_row + ch) * P);  // read once
     b.v = load16(grad_out + (t * chunks_per_row + ch) * P);
 #pragma unroll
     for (int i = 0; i < P; ++i) acc += Elem<T>::up(a.e[i]) * Elem<T>::up(b.e[i]);
@@ -183,19 +183,19 @@ __global__ __launch_bounds__(kBlock) void swiglu_bwd_grouped_kernel(
     dg.v = zero16();
     if (p < valid_end && c < I) {
       Pack16<T> u, g, dy;
-      u.v = load16(pre + p * two_i + c);
-      g.v = load16(pre + p * two_i + I + c);
-      dy.v = load16(d_act + p * I + c);
+      u.v = load16_nt(pre + p * two_i + c);  // all three are read once
+      g.v = load16_nt(pre + p * two_i + I + c);
+      dy.v = load16_nt(d_act + p * I + c);
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const float gf = Elem<T>::up(g.e[i]), uf = Elem<T>::up(u.e[i]), dyf = Elem<T>::up(dy.e[i]);
-        const float sg = sigmoid_f32(gf);
+        const float sg = sigmoid_for<T>(gf);
         const float gsg = gf * sg;
         dg.e[i] = Elem<T>::down(dyf * uf * (sg + gsg * (1.0f - sg)));
         du.e[i] = Elem<T>::down(dyf * gsg);
       }
-      store16(d_pre + p * two_i + c, du.v);
-      store16(d_pre + p * two_i + I + c, dg.v);
+      store16_nt(d_pre + p * two_i + c, du.v);
+      store16_nt(d_pre + p * two_i + I + c, dg.v);
     }
     if (d_pre_t != nullptr) {
       fill_tile_chunk(tile_up, r, cc, du.v);
@@ -221,7 +221,7 @@ __global__ __launch_bounds__(kBlock) void transpose_batched_kernel(const T* __re
     const int chunk = q * kBlock + threadIdx.x;
     const int r = chunk >> 3, cc = chunk & 7;
     vec16 v = zero16();
-    if (r0 + r < rows && c0 + cc * 8 < cols) v = load16(src + boff + (int64_t)(r0 + r) * cols + c0 + cc * 8);
+    if (r0 + r < rows && c0 + cc * 8 < cols) v = load16_nt(src + boff + (int64_t)(r0 + r) * cols + c0 + cc * 8);
     fill_tile_chunk(tile, r, cc, v);
   }
   __syncthreads();

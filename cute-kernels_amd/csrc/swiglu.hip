@@ -17,7 +17,7 @@ struct Chunk {
       c.e[0] = *p;
     } else {
       Pack16<T> k;
-      k.v = load16(p);
+      k.v = load16_nt(p);  // streaming: every element is read once
 #pragma unroll
       for (int i = 0; i < N; ++i) c.e[i] = k.e[i];
     }
@@ -30,7 +30,7 @@ struct Chunk {
       Pack16<T> k;
 #pragma unroll
       for (int i = 0; i < N; ++i) k.e[i] = e[i];
-      store16(p, k.v);
+      store16_nt(p, k.v);
     }
   }
 };
@@ -39,21 +39,26 @@ template <typename T, int P>
 __global__ __launch_bounds__(kBlock) void swiglu_fwd_kernel(const T* __restrict__ gate, int64_t gate_stride,
                                                              const T* __restrict__ up, int64_t up_stride,
                                                              T* __restrict__ out, int64_t out_stride, int64_t rows,
-                                                             int chunks_per_row) {
-  const int64_t total = rows * chunks_per_row;
-  const int64_t stride = (int64_t)gridDim.x * kBlock;
-  for (int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x; c < total; c += stride) {
-    const int64_t r = c / chunks_per_row;
-    const int64_t col = (c - r * chunks_per_row) * P;
-    const Chunk<T, P> g = Chunk<T, P>::load(gate + r * gate_stride + col);
-    const Chunk<T, P> u = Chunk<T, P>::load(up + r * up_stride + col);
-    Chunk<T, P> o;
+                                                             int64_t chunks_per_row, int tpr_log2) {
+  // 2^tpr_log2 threads share a row (chunk index = lane within the row, strided), the block's remaining threads take
+  // further rows: no division per chunk, and short rows still fill the block. A flat tensor is one long row.
+  const int tpr = 1 << tpr_log2;
+  const int lane_in_row = threadIdx.x & (tpr - 1);
+  const int64_t rows_per_block = kBlock >> tpr_log2;
+  for (int64_t r = (int64_t)blockIdx.x * rows_per_block + (threadIdx.x >> tpr_log2); r < rows;
+       r += (int64_t)gridDim.x * rows_per_block) {
+    for (int64_t ch = (int64_t)blockIdx.y * tpr + lane_in_row; ch < chunks_per_row; ch += (int64_t)gridDim.y * tpr) {
+      const int64_t col = ch * P;
+      const Chunk<T, P> g = Chunk<T, P>::load(gate + r * gate_stride + col);
+      const Chunk<T, P> u = Chunk<T, P>::load(up + r * up_stride + col);
+      Chunk<T, P> o;
 #pragma unroll
-    for (int i = 0; i < P; ++i) {
-      const float gf = Elem<T>::up(g.e[i]);
-      o.e[i] = Elem<T>::down(Elem<T>::up(u.e[i]) * gf * sigmoid_f32(gf));
+      for (int i = 0; i < P; ++i) {
+        const float gf = Elem<T>::up(g.e[i]);
+        o.e[i] = Elem<T>::down(Elem<T>::up(u.e[i]) * gf * sigmoid_for<T>(gf));
+      }
+      o.store(out + r * out_stride + col);
     }
-    o.store(out + r * out_stride + col);
   }
 }
 
@@ -63,26 +68,29 @@ __global__ __launch_bounds__(kBlock) void swiglu_bwd_kernel(const T* __restrict_
                                                              const T* __restrict__ d_out, int64_t d_out_stride,
                                                              T* __restrict__ d_gate, int64_t d_gate_stride,
                                                              T* __restrict__ d_up, int64_t d_up_stride, int64_t rows,
-                                                             int chunks_per_row) {
-  const int64_t total = rows * chunks_per_row;
-  const int64_t stride = (int64_t)gridDim.x * kBlock;
-  for (int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x; c < total; c += stride) {
-    const int64_t r = c / chunks_per_row;
-    const int64_t col = (c - r * chunks_per_row) * P;
-    const Chunk<T, P> g = Chunk<T, P>::load(gate + r * gate_stride + col);
-    const Chunk<T, P> u = Chunk<T, P>::load(up + r * up_stride + col);
-    const Chunk<T, P> dy = Chunk<T, P>::load(d_out + r * d_out_stride + col);
-    Chunk<T, P> dg, du;
+                                                             int64_t chunks_per_row, int tpr_log2) {
+  const int tpr = 1 << tpr_log2;
+  const int lane_in_row = threadIdx.x & (tpr - 1);
+  const int64_t rows_per_block = kBlock >> tpr_log2;
+  for (int64_t r = (int64_t)blockIdx.x * rows_per_block + (threadIdx.x >> tpr_log2); r < rows;
+       r += (int64_t)gridDim.x * rows_per_block) {
+    for (int64_t ch = (int64_t)blockIdx.y * tpr + lane_in_row; ch < chunks_per_row; ch += (int64_t)gridDim.y * tpr) {
+      const int64_t col = ch * P;
+      const Chunk<T, P> g = Chunk<T, P>::load(gate + r * gate_stride + col);
+      const Chunk<T, P> u = Chunk<T, P>::load(up + r * up_stride + col);
+      const Chunk<T, P> dy = Chunk<T, P>::load(d_out + r * d_out_stride + col);
+      Chunk<T, P> dg, du;
 #pragma unroll
-    for (int i = 0; i < P; ++i) {
-      const float gf = Elem<T>::up(g.e[i]), uf = Elem<T>::up(u.e[i]), dyf = Elem<T>::up(dy.e[i]);
-      const float sg = sigmoid_f32(gf);
-      const float gsg = gf * sg;
-      dg.e[i] = Elem<T>::down(dyf * uf * (sg + gsg * (1.0f - sg)));
-      du.e[i] = Elem<T>::down(dyf * gsg);
+      for (int i = 0; i < P; ++i) {
+        const float gf = Elem<T>::up(g.e[i]), uf = Elem<T>::up(u.e[i]), dyf = Elem<T>::up(dy.e[i]);
+        const float sg = sigmoid_for<T>(gf);
+        const float gsg = gf * sg;
+        dg.e[i] = Elem<T>::down(dyf * uf * (sg + gsg * (1.0f - sg)));
+        du.e[i] = Elem<T>::down(dyf * gsg);
+      }
+      dg.store(d_gate + r * d_gate_stride + col);
+      du.store(d_up + r * d_up_stride + col);
     }
-    dg.store(d_gate + r * d_gate_stride + col);
-    du.store(d_up + r * d_up_stride + col);
   }
 }
 
@@ -91,11 +99,30 @@ bool view_vector_ok(const void* p, int64_t stride, int64_t rows) {
   return aligned16(p) && (rows == 1 || stride % Elem<T>::per16 == 0);
 }
 
-inline unsigned grid_for(int64_t chunks) {
-  int64_t b = ceil_div(chunks, (int64_t)kBlock * 2);
-  if (b < 1) b = 1;
-  if (b > (1 << 20)) b = (1 << 20);
-  return (unsigned)b;
+// Launch shape for rows x chunks_per_row chunks: threads per row = smallest power of two covering the row (at most the
+// block), grid.x over row groups, grid.y over the chunks of long rows (a flat tensor is one row).
+struct Shape {
+  dim3 grid;
+  int tpr_log2;
+};
+inline Shape shape_for(int64_t rows, int64_t chunks_per_row) {
+  Shape s;
+  s.tpr_log2 = 0;
+  while ((1 << s.tpr_log2) < kBlock && (1 << s.tpr_log2) < chunks_per_row) ++s.tpr_log2;
+  const int64_t rows_per_block = kBlock >> s.tpr_log2;
+  int64_t gx = ceil_div(rows, rows_per_block);
+  if (gx > 65535) gx = 65535;
+  // long rows: split them over grid.y, two chunks per thread (many small blocks stream fastest here), at most 2^20 blocks
+  int64_t gy = 1;
+  if (s.tpr_log2 == 8) {
+    gy = ceil_div(chunks_per_row, (int64_t)kBlock * 2);
+    const int64_t most = ceil_div((int64_t)1 << 20, gx);
+    if (gy > most) gy = most;
+    if (gy < 1) gy = 1;
+    if (gy > 65535) gy = 65535;
+  }
+  s.grid = dim3((unsigned)gx, (unsigned)gy);
+  return s;
 }
 
 }  // namespace
@@ -119,13 +146,15 @@ extern "C" int ck_swiglu_fwd(const void* gate, int64_t gate_stride, const void* 
     int64_t done = 0;  // columns covered by the 128-bit kernel
     if (vec && cols >= P) {
       done = cols / P * P;
-      hipLaunchKernelGGL((swiglu_fwd_kernel<scalar_t, P>), dim3(grid_for(rows * (done / P))), dim3(kBlock), 0, s, g,
-                         gate_stride, u, up_stride, o, out_stride, rows, (int)(done / P));
+      const Shape sh = shape_for(rows, done / P);
+      hipLaunchKernelGGL((swiglu_fwd_kernel<scalar_t, P>), sh.grid, dim3(kBlock), 0, s, g, gate_stride, u, up_stride, o,
+                         out_stride, rows, done / P, sh.tpr_log2);
     }
     if (done < cols) {  // misaligned views, or the ragged end of a flat tensor
       const int64_t rest = cols - done;
-      hipLaunchKernelGGL((swiglu_fwd_kernel<scalar_t, 1>), dim3(grid_for(rows * rest)), dim3(kBlock), 0, s, g + done,
-                         gate_stride, u + done, up_stride, o + done, out_stride, rows, (int)rest);
+      const Shape sh = shape_for(rows, rest);
+      hipLaunchKernelGGL((swiglu_fwd_kernel<scalar_t, 1>), sh.grid, dim3(kBlock), 0, s, g + done, gate_stride, u + done,
+                         up_stride, o + done, out_stride, rows, rest, sh.tpr_log2);
     }
   });
   CK_CHECK_LAUNCH("ck_swiglu_fwd");
@@ -153,15 +182,16 @@ extern "C" int ck_swiglu_bwd(const void* gate, int64_t gate_stride, const void* 
     int64_t done = 0;
     if (vec && cols >= P) {
       done = cols / P * P;
-      hipLaunchKernelGGL((swiglu_bwd_kernel<scalar_t, P>), dim3(grid_for(rows * (done / P))), dim3(kBlock), 0, s, g,
-                         gate_stride, u, up_stride, dy, d_out_stride, dg, d_gate_stride, du, d_up_stride, rows,
-                         (int)(done / P));
+      const Shape sh = shape_for(rows, done / P);
+      hipLaunchKernelGGL((swiglu_bwd_kernel<scalar_t, P>), sh.grid, dim3(kBlock), 0, s, g, gate_stride, u, up_stride, dy,
+                         d_out_stride, dg, d_gate_stride, du, d_up_stride, rows, done / P, sh.tpr_log2);
     }
     if (done < cols) {
       const int64_t rest = cols - done;
-      hipLaunchKernelGGL((swiglu_bwd_kernel<scalar_t, 1>), dim3(grid_for(rows * rest)), dim3(kBlock), 0, s, g + done,
-                         gate_stride, u + done, up_stride, dy + done, d_out_stride, dg + done, d_gate_stride,
-                         du + done, d_up_stride, rows, (int)rest);
+      const Shape sh = shape_for(rows, rest);
+      hipLaunchKernelGGL((swiglu_bwd_kernel<scalar_t, 1>), sh.grid, dim3(kBlock), 0, s, g + done, gate_stride, u + done,
+                         up_stride, dy + done, d_out_stride, dg + done, d_gate_stride, du + done, d_up_stride, rows, rest,
+                         sh.tpr_log2);
     }
   });
   CK_CHECK_LAUNCH("ck_swiglu_bwd");
