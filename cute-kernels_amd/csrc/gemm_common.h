@@ -37,6 +37,7 @@ struct GemmParams {
   const void* aux_in;
   const float* a_scale;  // fp8 only: per-row dequantisation scale of a (indexed like the rows of a)
   const float* w_scale;  // fp8 only: per-output-channel scale of w, [E, N]
+  void* trace;           // measurement builds only: per-workgroup phase timestamps (8 x uint64 each), else NULL
 };
 
 // The 256 x 384 tile variant of the 16-bit kernel (grouped_gemm_wide.hip): modes kGrouped, kScatter, kSwiglu, kDw.

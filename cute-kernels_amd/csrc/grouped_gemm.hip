@@ -39,18 +39,18 @@ const bool g_eight_waves = [] {
 
 // CK_GEMM_TILE=256 / 384 in the environment forces the 256 x 256 / 256 x 384 block tile wherever both are possible
 // (A/B measurements); otherwise the choice follows the column utilisation, see use_wide_tile
-const int g_forced_tile = [] {
+inline int forced_tile() {  // read per call, so that tests can switch it inside one process
   const char* env = getenv("CK_GEMM_TILE");
   return env == nullptr ? 0 : atoi(env);
-}();
+}
 
 // 256 x 384 tiles carry 20 % more FLOPs per byte loaded from L2 but pay more for the ragged column edge and for their
 // (longer) epilogue. Measured at the Mixtral shape: +10 % with a long contraction (scatter epilogue, K = 14,336 / 28,672),
 // +4 % for the weight gradients, nothing at K = 4,096 -- so they serve those two cases, when the padded column count does
 // not eat the gain. `cols` output columns, `narrow` / `wide` columns per tile, `contraction`: (average) K.
 inline bool use_wide_tile(int64_t cols, int narrow, int wide, int64_t contraction) {
-  if (g_forced_tile == 256) return false;
-  if (g_forced_tile == 384) return true;
+  if (forced_tile() == 256) return false;
+  if (forced_tile() == 384) return true;
   if (contraction < 2048) return false;  // short contractions are dominated by the per-tile epilogue: more, smaller tiles
   const double util_narrow = (double)cols / (double)(ceil_div(cols, narrow) * narrow);
   const double util_wide = (double)cols / (double)(ceil_div(cols, wide) * wide);
@@ -134,6 +134,15 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
       if (m0 + r < valid_end) scatter_row = prm.row_slot[m0 + r];
   }
 
+#if (CK_ABLATE & 256)
+  auto stamp = [&](int i) {  // measurement builds: wall-clock (100 MHz) of phase boundaries, one record per workgroup
+    __builtin_amdgcn_s_waitcnt(0);
+    if (prm.trace != nullptr && tid == 0) static_cast<uint64_t*>(prm.trace)[(size_t)blockIdx.x * 8 + i] = wall_clock64();
+  };
+#else
+  auto stamp = [&](int) {};
+#endif
+  stamp(0);
   f32x16 acc[MI][NI];
 #pragma unroll
   for (int i = 0; i < MI; ++i)
@@ -399,6 +408,7 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
     };
     // MFMAs [mfma_begin(g), mfma_begin(g + 1)) follow fragment read g
     auto mfma_begin = [](int g) { return g * kMfma / kReads; };
+    stamp(1);
     if (nk > 0) {
       issue(0);
       issue(1);
@@ -442,6 +452,7 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
     }
   }
 
+  stamp(2);
   // ---- epilogue. Lane holds, per 32x32 block and q in 0..3, rows 8q + 4*(lane/32) + 0..3 of column lane%32.
   // static_for keeps every accumulator index a compile-time constant (the accumulators live in AGPRs).
   const int col_in_block = lane & 31;
@@ -523,6 +534,8 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
     };
     auto sync_slab = [&]() { __syncthreads(); };
     const T kZero = Elem<T>::down(0.f);
+    // most tiles have no pad rows: then nothing is tested per element (the test is a 64-bit compare and a branch each)
+    const bool tile_full = MODE == kDw || m0 + BM <= valid_end;
 
     if constexpr (MODE == kDw) {
       T* dw = static_cast<T*>(prm.y) + (int64_t)expert * prm.M * prm.N;
@@ -540,10 +553,14 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
       T* y_t = static_cast<T*>(prm.y_t);
       static_for<2>([&](auto pass) {
         // pad rows are staged as zeros: the transposed copy must hold zeros there
-        stage_blocks([&](auto i, auto jj, auto q, auto sidx) {
-          const int64_t p = m0 + wm * WM + i * 32 + 8 * q + row_quad + sidx;
-          return p < valid_end ? Elem<T>::down(acc[i][pass * 2 + jj][4 * q + sidx]) : kZero;
-        });
+        if (tile_full) {
+          stage_blocks([&](auto i, auto jj, auto q, auto sidx) { return Elem<T>::down(acc[i][pass * 2 + jj][4 * q + sidx]); });
+        } else {
+          stage_blocks([&](auto i, auto jj, auto q, auto sidx) {
+            const int64_t p = m0 + wm * WM + i * 32 + 8 * q + row_quad + sidx;
+            return p < valid_end ? Elem<T>::down(acc[i][pass * 2 + jj][4 * q + sidx]) : kZero;
+          });
+        }
         sync_slab();
         drain_rows([&](int r, int sc) -> T* {
           const int64_t p = m0 + r, n = (int64_t)nt * BN + tile_col(sc, pass);
@@ -567,15 +584,22 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
       // activation column of slab column sc (64 per wave column)
       auto act_col = [&](int sc) { return (int64_t)nt * (BN / 2) + (sc >> 6) * (WN / 2) + (sc & 63); };
       static_for<3>([&](auto pass) {  // 0: up half of the pre-activation, 1: gate half, 2: activation
-        stage_blocks([&](auto i, auto jj, auto q, auto sidx) {
-          const int64_t p = m0 + wm * WM + i * 32 + 8 * q + row_quad + sidx;
+        auto value = [&](auto i, auto jj, auto q, auto sidx, bool valid) {
           const T up = Elem<T>::down(acc[i][jj][4 * q + sidx]);
           const T gate = Elem<T>::down(acc[i][jj + 2][4 * q + sidx]);
           if (pass == 0) return up;
           if (pass == 1) return gate;
-          const float gf = Elem<T>::up(gate);
-          return p < valid_end ? Elem<T>::down(Elem<T>::up(up) * gf * sigmoid_fast(gf)) : kZero;
-        });
+          const float gf = Elem<T>::up(gate);  // from the rounded pre-activation, like the unfused path
+          const T a = Elem<T>::down(Elem<T>::up(up) * gf * sigmoid_fast(gf));
+          return valid ? a : kZero;
+        };
+        if (tile_full) {
+          stage_blocks([&](auto i, auto jj, auto q, auto sidx) { return value(i, jj, q, sidx, true); });
+        } else {
+          stage_blocks([&](auto i, auto jj, auto q, auto sidx) {
+            return value(i, jj, q, sidx, m0 + wm * WM + i * 32 + 8 * q + row_quad + sidx < valid_end);
+          });
+        }
         sync_slab();
         drain_rows([&](int r, int sc) -> T* {
           const int64_t p = m0 + r, col = act_col(sc);
@@ -593,6 +617,7 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
         sync_slab();
       });
     }
+    stamp(3);
     return;
   }
   if constexpr (MODE == kDw) {
@@ -784,6 +809,9 @@ extern "C" int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* 
   prm.ld_t = ld_t;
   prm.aux = aux;
   prm.aux_in = aux_in;
+#if (CK_ABLATE & 256)
+  if (const char* t = getenv("CK_TRACE_PTR")) prm.trace = reinterpret_cast<void*>(strtoull(t, nullptr, 16));
+#endif
   int out_cols = N;  // columns that tile along the grid
   if (epilogue == CK_EPI_SWIGLU) {
     CK_REQUIRE(N % 16 == 0 && aux != nullptr, "%s: the SwiGLU epilogue needs N = 2*I with I %% 8 == 0 and aux", name);
@@ -797,10 +825,10 @@ extern "C" int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* 
   hipStream_t s = static_cast<hipStream_t>(stream);
   // kSwiglu tiles cover BN/2 activation columns each
   auto n_tiles_for = [&](int bn) { return (int)ceil_div(out_cols, epilogue == CK_EPI_SWIGLU ? bn / 2 : bn); };
-  const bool wide_mode = g_forced_tile == 384 ? epilogue != CK_EPI_SWIGLU_BWD : epilogue == CK_EPI_SCATTER;
+  const bool wide_mode = forced_tile() == 384 ? epilogue != CK_EPI_SWIGLU_BWD : epilogue == CK_EPI_SCATTER;
   if (seg->align == kWideBM && K % 32 == 0 && wide_mode && !g_force_pipe0 &&
       use_wide_tile(out_cols, epilogue == CK_EPI_SWIGLU ? 128 : 256, epilogue == CK_EPI_SWIGLU ? kWideBN / 2 : kWideBN,
-                    g_forced_tile == 384 ? 1 << 20 : (K >= 8192 ? K : 0))) {
+                    forced_tile() == 384 ? 1 << 20 : (K >= 8192 ? K : 0))) {
     prm.n_tiles = n_tiles_for(kWideBN);
     const int64_t wide_blocks = m_tiles * prm.n_tiles;
     CK_REQUIRE(wide_blocks < (int64_t)0x7fffffff, "%s: grid too large", name);
@@ -848,6 +876,9 @@ extern "C" int ck_grouped_gemm_dw(const void* a_t, const void* b_t, int64_t ld_t
   prm.tile_expert = seg->tile_expert;
   prm.row_slot = seg->row_slot;
   prm.y = dw;
+#if (CK_ABLATE & 256)
+  if (const char* t = getenv("CK_TRACE_PTR")) prm.trace = reinterpret_cast<void*>(strtoull(t, nullptr, 16));
+#endif
   hipStream_t s = static_cast<hipStream_t>(stream);
   // tile size follows the problem, not the segment alignment: small weight matrices get 128x128 tiles
   const bool big = (M >= 1024 && N >= 1024);

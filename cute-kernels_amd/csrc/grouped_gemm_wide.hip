@@ -1,8 +1,10 @@
 // 256 x 384 tile variant of the scattered grouped GEMM (bf16 / f16 inputs, fp32 accumulation).
 //
 // Why a wider tile: the 256 x 256 kernel is bound by L2 -> LDS load throughput, and a tile's FLOPs per loaded byte are
-// BM*BN / (BM + BN): 128 at 256 x 256, 153.6 here. The accumulators (384 fp32 registers per lane) only fit with one wave
-// per SIMD, so the workgroup is 4 waves in a 2 x 2 grid with 128 x 192 wave tiles = 4 x 6 v_mfma_f32_32x32x16 blocks.
+// BM*BN / (BM + BN): 128 at 256 x 256, 153.6 here. Workgroup = 8 waves (two per SIMD) in a 4 x 2 grid with 64 x 192 wave
+// tiles = 2 x 6 v_mfma_f32_32x32x16 blocks: 192 accumulator registers per lane, which leaves 64 for everything else --
+// hence single-buffered fragments. (With 4 waves and 128 x 192 wave tiles the 384 accumulators have to be split over
+// AGPRs and VGPRs by hand; that variant measured no faster than the 256 x 256 kernel.)
 //
 // Pipeline: K step 32 (64-byte LDS rows, XOR-swizzled), operands go global -> LDS directly (global_load_lds_dwordx4),
 // four stages of 40 KiB = the whole 160 KiB of LDS, loads issued 2.5 steps ahead and never past the last step. Fragments
@@ -16,10 +18,7 @@ namespace ck {
 namespace {
 
 constexpr int BM = kWideBM, BN = kWideBN;
-#ifndef CK_WIDE_WGM
-#define CK_WIDE_WGM 4
-#endif
-constexpr int WGM = CK_WIDE_WGM;           // waves along M (always 2 along N)
+constexpr int WGM = 4;                     // waves along M (always 2 along N)
 constexpr int NW = 2 * WGM, NT = 64 * NW;
 constexpr int WM = BM / WGM, WN = BN / 2;  // wave tile
 constexpr int MI = WM / 32, NI = WN / 32;
@@ -162,24 +161,7 @@ __global__ __launch_bounds__(NT) void grouped_gemm_wide_kernel(const GemmParams 
   auto read_b = [&](int stage, int sl, int j) {
     fb[j] = *reinterpret_cast<const frag_t*>(lds_c + stage * kStageBytes + slice_off[sl] + fb_row + j * 32 * kRowBytes);
   };
-  // 384 accumulator registers per lane do not fit one register class (256 AGPRs, 256 VGPRs): column blocks 0 .. 3 are
-  // pinned to AGPRs and 4, 5 to VGPRs through the operand constraints (left to itself the register allocator keeps all of
-  // them in AGPRs and shuttles the overflow through scratch). Successive MFMAs on one block are 23 MFMAs apart, far beyond
-  // the back-to-back dependency window, and the fragments come from LDS reads, which the wait-count pass tracks through
-  // the asm operands.
-  auto mfma = [&](int i, int j) {
-    if (j < 4) {
-      if constexpr (std::is_same<T, bf16_t>::value)
-        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fa[i]), "v"(fb[j]));
-      else
-        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+a"(acc[i][j]) : "v"(fa[i]), "v"(fb[j]));
-    } else {
-      if constexpr (std::is_same<T, bf16_t>::value)
-        asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(acc[i][j]) : "v"(fa[i]), "v"(fb[j]));
-      else
-        asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(acc[i][j]) : "v"(fa[i]), "v"(fb[j]));
-    }
-  };
+  auto mfma = [&](int i, int j) { acc[i][j] = Mfma<T>::run(fa[i], fb[j], acc[i][j]); };
 
   if (nk > 0) {
     issue(0);
@@ -251,15 +233,15 @@ __global__ __launch_bounds__(NT) void grouped_gemm_wide_kernel(const GemmParams 
   typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4;
   T* slab = reinterpret_cast<T*>(lds_raw);
   int* scatter_rows = reinterpret_cast<int*>(lds_c + kMetaOffset);
-  // every wave is done with the stages; the no-ops cover the MFMA-result-to-VALU-read distance of the last MFMAs (18 wait
-  // states for a 16-pass MFMA), which the compiler cannot see through the asm
-  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier\n\ts_nop 15\n\ts_nop 7" ::: "memory");
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave is done with the stages
   if constexpr (MODE == kScatter) {
     if (tid < BM) scatter_rows[tid] = scatter_row;  // first read after the first slab barrier below
   }
   const int col_in_block = lane & 31;
   const int row_quad = (lane >> 5) * 4;
   const T kZero = Elem<T>::down(0.f);
+  // most tiles have no pad rows: then nothing is tested per element (the test is a 64-bit compare and a branch each)
+  const bool tile_full = MODE == kDw || m0 + BM <= valid_end;
 
   auto stage_blocks = [&](auto&& value /* (i, jj, q, s) -> T */) {
     static_for<MI>([&](auto i) {
@@ -329,10 +311,14 @@ __global__ __launch_bounds__(NT) void grouped_gemm_wide_kernel(const GemmParams 
     T* y_t = static_cast<T*>(prm.y_t);
     static_for<2>([&](auto pass) {
       // pad rows are staged as zeros: the transposed copy must hold zeros there
-      stage_blocks([&](auto i, auto jj, auto q, auto s) {
-        const int64_t p = m0 + wm * WM + i * 32 + 8 * q + row_quad + s;
-        return p < valid_end ? Elem<T>::down(acc[i][pass * kSlabBlocks + jj][4 * q + s]) : kZero;
-      });
+      if (tile_full) {
+        stage_blocks([&](auto i, auto jj, auto q, auto s) { return Elem<T>::down(acc[i][pass * kSlabBlocks + jj][4 * q + s]); });
+      } else {
+        stage_blocks([&](auto i, auto jj, auto q, auto s) {
+          const int64_t p = m0 + wm * WM + i * 32 + 8 * q + row_quad + s;
+          return p < valid_end ? Elem<T>::down(acc[i][pass * kSlabBlocks + jj][4 * q + s]) : kZero;
+        });
+      }
       __syncthreads();
       drain_rows([&](int r, int sc) -> T* {
         const int64_t p = m0 + r, n = (int64_t)nt * BN + tile_col(sc, pass);
@@ -357,15 +343,22 @@ __global__ __launch_bounds__(NT) void grouped_gemm_wide_kernel(const GemmParams 
       return (int64_t)nt * (BN / 2) + (sc / (kSlabBlocks * 32)) * (WN / 2) + sc % (kSlabBlocks * 32);
     };
     static_for<3>([&](auto pass) {  // 0: up half of the pre-activation, 1: gate half, 2: activation
-      stage_blocks([&](auto i, auto jj, auto q, auto s) {
-        const int64_t p = m0 + wm * WM + i * 32 + 8 * q + row_quad + s;
+      auto value = [&](auto i, auto jj, auto q, auto s, bool valid) {
         const T up = Elem<T>::down(acc[i][jj][4 * q + s]);
         const T gate = Elem<T>::down(acc[i][jj + kSlabBlocks][4 * q + s]);
         if (pass == 0) return up;
         if (pass == 1) return gate;
         const float gf = Elem<T>::up(gate);  // from the rounded pre-activation, like the unfused path
-        return p < valid_end ? Elem<T>::down(Elem<T>::up(up) * gf * sigmoid_fast(gf)) : kZero;
-      });
+        const T a = Elem<T>::down(Elem<T>::up(up) * gf * sigmoid_fast(gf));
+        return valid ? a : kZero;
+      };
+      if (tile_full) {
+        stage_blocks([&](auto i, auto jj, auto q, auto s) { return value(i, jj, q, s, true); });
+      } else {
+        stage_blocks([&](auto i, auto jj, auto q, auto s) {
+          return value(i, jj, q, s, m0 + wm * WM + i * 32 + 8 * q + row_quad + s < valid_end);
+        });
+      }
       __syncthreads();
       drain_rows([&](int r, int sc) -> T* {
         const int64_t p = m0 + r, col = act_col(sc);
