@@ -30,10 +30,10 @@ PEAK_HBM_GBS = 8000.0  # MI355X HBM3E
 # this same command, FETCH_SIZE scaled x2.0 and WRITE_SIZE x1.0 against transpose_batched_kernel (known size);
 # summary and commands: profiles/grouped_gemm_c3_moe_fwd_bwd.md. Not measurable from inside this process.
 TRAFFIC_BYTES_PER_LAUNCH = {
-    "grouped_gemm<scatter>": 13.9e9 + 0.27e9,
-    "grouped_gemm<dw>": 10.0e9 + 1.41e9,
-    "grouped_gemm<swiglu>": 19.5e9 + 4.92e9,
-    "grouped_gemm<grouped>": 9.5e9 + 0.94e9,
+    "grouped_gemm<scatter>": 2 * 5.727e6 * 1024 + 2.834e5 * 1024,  # 256 x 384 tiles
+    "grouped_gemm<dw>": 2 * 6.043e6 * 1024 + 1.516e6 * 1024,  # 256 x 384 tiles
+    "grouped_gemm<swiglu>": 2 * 8.842e6 * 1024 + 3.706e6 * 1024,
+    "grouped_gemm<grouped>": 2 * 4.111e6 * 1024 + 9.175e5 * 1024,
 }
 
 # workload: configs[2] of the baseline, the configuration its headline metric (MoE fwd+bwd TFLOP/s) is quoted on
