@@ -359,46 +359,80 @@ int launch_fp8(const GemmParams& prm, unsigned blocks, hipStream_t s, const char
 constexpr int kQuantBlock = 256;
 constexpr float kE4M3Max = 448.0f;
 
-// scale[r] = amax(x[r, :]) / 448 (1 for an all-zero row); q[r, c] = e4m3(x[r, c] * (448 / amax)), round to nearest even
-template <typename T>
+// scale[r] = amax(x[r, :]) / 448 (1 for an all-zero row); q[r, c] = e4m3(x[r, c] * (448 / amax)), round to nearest even.
+// A row is owned by TPR = 64 lanes (one wave, no block synchronisation) or 256 (the block); a lane keeps its NC chunks of
+// 16 elements in registers between the reduction and the conversion, so x is read once (NC == 0: long rows, re-read).
+template <typename T, int TPR, int NC>
 __global__ __launch_bounds__(kQuantBlock) void quant_rows_e4m3_kernel(const T* __restrict__ x, int64_t rows, int cols,
                                                                        uint8_t* __restrict__ q, float* __restrict__ scales) {
   __shared__ float red[kQuantBlock / kWave];
+  constexpr int ROWS = kQuantBlock / TPR;
   const int chunks = cols / 16;  // 16 elements: 32 bytes in, 16 bytes out
-  for (int64_t row = blockIdx.x; row < rows; row += gridDim.x) {
-    const T* xr = x + row * cols;
-    float amax = 0.f;
-    for (int ch = threadIdx.x; ch < chunks; ch += kQuantBlock) {
-      Pack16<T> a, b;
-      a.v = load16(xr + ch * 16);
-      b.v = load16(xr + ch * 16 + 8);
+  const int lane = threadIdx.x % TPR;
+  auto chunk_amax = [&](const Pack16<T>& a, const Pack16<T>& b, float m) {
 #pragma unroll
-      for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fmaxf(fabsf(Elem<T>::up(a.e[i])), fabsf(Elem<T>::up(b.e[i]))));
+    for (int i = 0; i < 8; ++i) m = fmaxf(m, fmaxf(fabsf(Elem<T>::up(a.e[i])), fabsf(Elem<T>::up(b.e[i]))));
+    return m;
+  };
+  auto convert = [&](const Pack16<T>& a, const Pack16<T>& b, float inv) {
+    vec16 o;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const T* src = i < 2 ? a.e : b.e;
+      const int k = (i & 1) * 4;
+      int w = 0;
+      w = __builtin_amdgcn_cvt_pk_fp8_f32(Elem<T>::up(src[k]) * inv, Elem<T>::up(src[k + 1]) * inv, w, false);
+      w = __builtin_amdgcn_cvt_pk_fp8_f32(Elem<T>::up(src[k + 2]) * inv, Elem<T>::up(src[k + 3]) * inv, w, true);
+      o.w[i] = (uint32_t)w;
+    }
+    return o;
+  };
+  // TPR == 256: every thread of the block runs the same trip count (the reduction synchronises the block)
+  for (int64_t row = (int64_t)blockIdx.x * ROWS + threadIdx.x / TPR; row < rows; row += (int64_t)gridDim.x * ROWS) {
+    const T* xr = x + row * cols;
+    uint8_t* qr = q + row * cols;
+    float amax = 0.f;
+    Pack16<T> a[NC > 0 ? NC : 1], b[NC > 0 ? NC : 1];
+    if constexpr (NC > 0) {
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const int ch = c * TPR + lane;
+        if (ch < chunks) {
+          a[c].v = load16_nt(xr + ch * 16);
+          b[c].v = load16_nt(xr + ch * 16 + 8);
+          amax = chunk_amax(a[c], b[c], amax);
+        }
+      }
+    } else {
+      for (int ch = lane; ch < chunks; ch += TPR) {
+        a[0].v = load16(xr + ch * 16);
+        b[0].v = load16(xr + ch * 16 + 8);
+        amax = chunk_amax(a[0], b[0], amax);
+      }
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, kWave));
-    __syncthreads();
-    if ((threadIdx.x & (kWave - 1)) == 0) red[threadIdx.x / kWave] = amax;
-    __syncthreads();
+    if constexpr (TPR == kQuantBlock) {
+      __syncthreads();
+      if ((threadIdx.x & (kWave - 1)) == 0) red[threadIdx.x / kWave] = amax;
+      __syncthreads();
 #pragma unroll
-    for (int w = 0; w < kQuantBlock / kWave; ++w) amax = fmaxf(amax, red[w]);
+      for (int w = 0; w < kQuantBlock / kWave; ++w) amax = fmaxf(amax, red[w]);
+    }
     const float inv = amax > 0.f ? kE4M3Max / amax : 1.0f;
-    if (threadIdx.x == 0) scales[row] = amax > 0.f ? amax / kE4M3Max : 1.0f;
-    for (int ch = threadIdx.x; ch < chunks; ch += kQuantBlock) {
-      Pack16<T> a, b;
-      a.v = load16(xr + ch * 16);  // second read is served by L1 / L2
-      b.v = load16(xr + ch * 16 + 8);
-      vec16 o;
+    if (lane == 0) scales[row] = amax > 0.f ? amax / kE4M3Max : 1.0f;
+    if constexpr (NC > 0) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const T* src = i < 2 ? a.e : b.e;
-        const int k = (i & 1) * 4;
-        int w = 0;
-        w = __builtin_amdgcn_cvt_pk_fp8_f32(Elem<T>::up(src[k]) * inv, Elem<T>::up(src[k + 1]) * inv, w, false);
-        w = __builtin_amdgcn_cvt_pk_fp8_f32(Elem<T>::up(src[k + 2]) * inv, Elem<T>::up(src[k + 3]) * inv, w, true);
-        o.w[i] = (uint32_t)w;
+      for (int c = 0; c < NC; ++c) {
+        const int ch = c * TPR + lane;
+        if (ch < chunks) store16_nt(qr + ch * 16, convert(a[c], b[c], inv));
       }
-      store16(q + row * cols + ch * 16, o);
+    } else {
+      for (int ch = lane; ch < chunks; ch += TPR) {
+        a[0].v = load16(xr + ch * 16);  // second read is served by L1 / L2
+        b[0].v = load16(xr + ch * 16 + 8);
+        store16_nt(qr + ch * 16, convert(a[0], b[0], inv));
+      }
     }
   }
 }
@@ -414,11 +448,23 @@ extern "C" int ck_quant_rows_e4m3(const void* x, int64_t rows, int32_t cols, voi
   if (rows == 0) return CK_OK;
   CK_REQUIRE(x && q && scales && aligned16(x) && aligned16(q), "ck_quant_rows_e4m3: NULL or misaligned pointer");
   hipStream_t s = static_cast<hipStream_t>(stream);
-  const unsigned blocks = (unsigned)(rows < 65535 * 8 ? rows : 65535 * 8);
+  const int chunks = cols / 16;
+#define CK_QUANT(TPR, NC)                                                                                          \
+  do {                                                                                                             \
+    const int64_t want = ceil_div(rows, (int64_t)(kQuantBlock / (TPR)));                                           \
+    const unsigned blocks = (unsigned)(want < 65535 * 4 ? want : 65535 * 4);                                       \
+    hipLaunchKernelGGL((quant_rows_e4m3_kernel<scalar_t, TPR, NC>), dim3(blocks), dim3(kQuantBlock), 0, s,         \
+                       static_cast<const scalar_t*>(x), rows, (int)cols, static_cast<uint8_t*>(q), scales);        \
+  } while (0)
   CK_DISPATCH_HALF(dtype, "ck_quant_rows_e4m3", {
-    hipLaunchKernelGGL((quant_rows_e4m3_kernel<scalar_t>), dim3(blocks), dim3(kQuantBlock), 0, s,
-                       static_cast<const scalar_t*>(x), rows, (int)cols, static_cast<uint8_t*>(q), scales);
+    if (chunks <= kWave) CK_QUANT(kWave, 1);
+    else if (chunks <= 2 * kWave) CK_QUANT(kWave, 2);
+    else if (chunks <= kQuantBlock) CK_QUANT(kQuantBlock, 1);
+    else if (chunks <= 2 * kQuantBlock) CK_QUANT(kQuantBlock, 2);
+    else if (chunks <= 4 * kQuantBlock) CK_QUANT(kQuantBlock, 4);
+    else CK_QUANT(kQuantBlock, 0);
   });
+#undef CK_QUANT
   CK_CHECK_LAUNCH("ck_quant_rows_e4m3");
   return CK_OK;
 }

@@ -20,13 +20,15 @@ from .scattermoe import (
     sort_by_expert,
     swiglu_experts,
 )
+from .softmax import softmax_cute
 from .swiglu import swiglu_cute, swiglu_packed_cute
 from .utils import ceil_divide, divide_if_divisible, get_num_elements_and_hidden_size, set_seed
 
 # torch.compile support: the public functions switch to the registered ops while a trace is being taken
 from . import compile_ops as _compile_ops
-from . import continuous_count as _m_count, fused_residual_add_rmsnorm as _m_frn, rmsnorm as _m_rms, scattermoe as _m_moe, swiglu as _m_swiglu
+from . import continuous_count as _m_count, fused_residual_add_rmsnorm as _m_frn, rmsnorm as _m_rms, scattermoe as _m_moe
+from . import softmax as _m_softmax, swiglu as _m_swiglu
 
-for _m in (_m_count, _m_frn, _m_rms, _m_moe, _m_swiglu):
+for _m in (_m_count, _m_frn, _m_rms, _m_moe, _m_softmax, _m_swiglu):
     _m._ops = _compile_ops
 del _m

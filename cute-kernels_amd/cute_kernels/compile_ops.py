@@ -22,6 +22,7 @@ from . import continuous_count as _count
 from . import fused_residual_add_rmsnorm as _frn
 from . import rmsnorm as _rms
 from . import scattermoe as _moe
+from . import softmax as _softmax
 from . import swiglu as _swiglu
 
 NS = "ck_mi355"
@@ -241,6 +242,44 @@ def _frn_bwd(ctx, output_grad, added_grad, _rstd_grad):
 
 
 fused_residual_add_rmsnorm.register_autograd(_frn_bwd, setup_context=_frn_setup)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# softmax
+# ---------------------------------------------------------------------------------------------------------------
+@custom_op(f"{NS}::softmax", mutates_args=())
+def softmax(x: Tensor, multiplier: float) -> Tensor:
+    return _softmax._Softmax_Cute.forward(_Ctx(), x, multiplier)
+
+
+@softmax.register_fake
+def _(x, multiplier):
+    return torch.empty_like(x, memory_format=torch.contiguous_format)
+
+
+@custom_op(f"{NS}::softmax_backward", mutates_args=())
+def softmax_backward(output: Tensor, output_grad: Tensor, multiplier: float) -> Tensor:
+    ctx = _Ctx()
+    ctx.saved_tensors = (output,)
+    ctx.multiplier = multiplier
+    return _softmax._Softmax_Cute.backward(ctx, output_grad)[0]
+
+
+@softmax_backward.register_fake
+def _(output, output_grad, multiplier):
+    return torch.empty_like(output)
+
+
+def _softmax_setup(ctx, inputs, output):
+    ctx.save_for_backward(output)
+    ctx.multiplier = inputs[1]
+
+
+def _softmax_bwd(ctx, output_grad):
+    return softmax_backward(ctx.saved_tensors[0], output_grad, ctx.multiplier), None
+
+
+softmax.register_autograd(_softmax_bwd, setup_context=_softmax_setup)
 
 
 # ---------------------------------------------------------------------------------------------------------------

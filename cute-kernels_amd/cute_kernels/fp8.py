@@ -120,7 +120,7 @@ class MoE_E4M3(nn.Module):
         original_shape = hidden_states.shape
         hidden_states = hidden_states.view(-1, self.hidden_size)
         router_logits = self.gate(hidden_states)
-        router_weights, selected_experts = route_topk_softmax(router_logits, self.top_k)
+        router_weights, selected_experts = route_topk_softmax(router_logits, self.top_k, long_indices=False)
         seg = sort_by_expert(selected_experts, self.num_experts, 256)
         out = swiglu_experts_e4m3(
             hidden_states, self.c_fc_weight_e4m3, self.c_fc_scale, self.c_proj_weight_e4m3, self.c_proj_scale,

@@ -26,7 +26,7 @@ class _RouteTopKSoftmax(torch.autograd.Function):
     """logits [T, E] -> gates [T, k] (softmax over the k largest logits, in logits.dtype), selected [T, k] int64."""
 
     @staticmethod
-    def forward(ctx, logits: torch.Tensor, k: int):
+    def forward(ctx, logits: torch.Tensor, k: int, long_indices: bool = True):
         _C.require_gpu(logits)
         logits = logits.contiguous()
         T, E = logits.shape
@@ -42,9 +42,9 @@ class _RouteTopKSoftmax(torch.autograd.Function):
         ctx.save_for_backward(gates, selected)
         ctx.E = E
         ctx.dtype = logits.dtype
-        selected_long = selected.long()
-        ctx.mark_non_differentiable(selected_long)
-        return gates.to(logits.dtype), selected_long
+        selected_out = selected.long() if long_indices else selected
+        ctx.mark_non_differentiable(selected_out)
+        return gates.to(logits.dtype), selected_out
 
     @staticmethod
     def backward(ctx, d_gates: torch.Tensor, _d_selected):
@@ -60,16 +60,17 @@ class _RouteTopKSoftmax(torch.autograd.Function):
                     _C.dtype_code(ctx.dtype), _C.stream(),
                 )
             )
-        return d_logits, None
+        return d_logits, None, None
 
 
-def route_topk_softmax(logits: torch.Tensor, k: int) -> tuple[torch.Tensor, torch.Tensor]:
+def route_topk_softmax(logits: torch.Tensor, k: int, long_indices: bool = True) -> tuple[torch.Tensor, torch.Tensor]:
     """Top-k over the logits and softmax over the k selected logits in fp32, cast back to logits.dtype
-    (torch_implementation.py:122-135). Equal logits: the lowest expert index wins."""
+    (torch_implementation.py:122-135). Equal logits: the lowest expert index wins. The indices come back as int64 like
+    torch.topk's; long_indices=False keeps the kernel's int32 (what the sort consumes fastest)."""
     if torch.compiler.is_compiling():
         gates, selected = _ops.route_topk_softmax(logits, k)
-        return gates.to(logits.dtype), selected.long()
-    return _RouteTopKSoftmax.apply(logits, k)
+        return gates.to(logits.dtype), (selected.long() if long_indices else selected)
+    return _RouteTopKSoftmax.apply(logits, k, long_indices)
 
 
 @torch.no_grad()

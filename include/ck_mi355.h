@@ -238,6 +238,17 @@ int ck_fused_residual_add_rmsnorm_bwd(const void* added, const void* weight, con
                                       void* d_residual, float* d_weight_partial, float* d_weight, int32_t dtype,
                                       void* stream);
 
+/* ---------------------------------------------------------------------------------------------------------------
+ * Softmax over the last dimension (what a load-balancing loss applies to the router logits the MoE layer returns)
+ * Replaces: softmax_forward_triton / softmax_backward_triton -- cute_kernels/kernels/softmax/triton_implementation/
+ *           (launched from kernels/softmax/__init__.py:12-36); semantics of softmax_torch (torch_implementation.py:9-18):
+ *           fp32 math, x pre-multiplied by `multiplier` (pass 1 for none).
+ * x, out, y, d_y, d_x [B, H] contiguous. backward: d_x = multiplier * y * (d_y - sum_h(d_y * y)).
+ * ------------------------------------------------------------------------------------------------------------- */
+int ck_softmax_fwd(const void* x, float multiplier, int64_t B, int32_t H, void* out, int32_t dtype, void* stream);
+int ck_softmax_bwd(const void* y, const void* d_y, float multiplier, int64_t B, int32_t H, void* d_x, int32_t dtype,
+                   void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -52,6 +52,15 @@ def fused_residual_add_rmsnorm_torch(
     return rmsnorm_torch(x, weight, eps), x
 
 
+def softmax_torch(x: torch.Tensor, logits_multiplier: float | None = 1) -> torch.Tensor:
+    """cute_kernels/kernels/softmax/torch_implementation.py:9-18: fp32 softmax of x * logits_multiplier, cast back."""
+    dtype = x.dtype
+    x = x.float()
+    if logits_multiplier is not None:
+        x = x * logits_multiplier
+    return F.softmax(x, dim=-1).to(dtype)
+
+
 def topk_lowest_index_first(logits: torch.Tensor, k: int) -> tuple[torch.Tensor, torch.Tensor]:
     """Top-k with a fixed tie rule (equal logits: lowest expert index first). torch.topk's own tie order is
     unspecified (torch_implementation.py:195-201 just calls it); values are identical either way."""

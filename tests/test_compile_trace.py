@@ -25,6 +25,7 @@ def test_elementwise_and_norm_ops_trace():
     _traces(lambda a, b: ck.rmsnorm_cute(a, b, None), x, w)
     _traces(lambda a: ck.rmsnorm_cute(a, None, 1e-5, memory_efficient=True), x)
     _traces(lambda a, r, b: ck.fused_residual_add_rmsnorm_cute(a, r, b, 1e-5, 0.9), x, y, w)
+    _traces(lambda a: ck.softmax_cute(a, 0.7), x)
 
 
 @pytest.mark.parametrize("act,is_glu", [(ck.swiglu_packed_cute, True), (torch.nn.GLU(), True), (torch.nn.GELU("tanh"), False)])

@@ -31,6 +31,7 @@ def test_swiglu_and_norms_compiled(device, dtype):
         "swiglu_packed": (lambda a, b, c: ck.swiglu_packed_cute(a), 1),
         "rmsnorm": (lambda a, b, c: ck.rmsnorm_cute(a, c, 1e-5), 3),
         "rmsnorm_me": (lambda a, b, c: ck.rmsnorm_cute(a, None, None, memory_efficient=True), 1),
+        "softmax": (lambda a, b, c: ck.softmax_cute(a, 0.7), 1),
         "frn": (lambda a, b, c: sum(t.float() for t in ck.fused_residual_add_rmsnorm_cute(a, b, c, 1e-5, 0.9)), 3),
         "frn_me": (lambda a, b, c: ck.fused_residual_add_rmsnorm_cute(a, b, None, 1e-5, None, True)[0], 2),
     }

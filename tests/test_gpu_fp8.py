@@ -16,7 +16,7 @@ pytestmark = pytest.mark.gpu
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("rows,cols", [(1, 16), (37, 64), (300, 4096), (5, 1536)])
+@pytest.mark.parametrize("rows,cols", [(1, 16), (37, 64), (300, 4096), (5, 1536), (7, 8192), (3, 16384), (2, 32784), (1030, 2048)])
 def test_quantize_rows_is_bit_exact(device, dtype, rows, cols):
     g = torch.Generator().manual_seed(rows + cols)
     x = (torch.randn(rows, cols, generator=g) * 3).to(dtype)

@@ -218,3 +218,39 @@ def test_fused_residual_add_rmsnorm_without_residual_gradient(device):
     z_ref.square().sum().backward()
     for ours, ref in ((xa, xc), (ra, rc), (wa, wc)):
         torch.testing.assert_close(ours.grad.cpu(), ref.grad, rtol=1e-4, atol=1e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("logits_multiplier", [None, 0.7])
+def test_softmax_reference_grid(device, dtype, logits_multiplier):
+    # reference grid and bounds: softmax_test.py:19-70 (std 0.02 inputs, sum().backward(), atol 4e-5 / 1.1e-3 on the grads)
+    g = torch.Generator().manual_seed(42)
+    for size in _rms_sizes() + [(3, 70000)]:
+        x = (0.02 * torch.randn(size, generator=g)).to(dtype)
+        a, c = x.clone().to(device).requires_grad_(), x.clone().requires_grad_()
+        z = cute_kernels.softmax_cute(a, logits_multiplier)
+        z_ref = mo.softmax_torch(c, logits_multiplier)
+        z.sum().backward()
+        z_ref.sum().backward()
+        assert z.dtype == dtype and z.shape == x.shape
+        if dtype == torch.float32:
+            torch.testing.assert_close(z.cpu(), z_ref, rtol=1e-5, atol=1e-7)
+            torch.testing.assert_close(a.grad.cpu(), c.grad, rtol=0, atol=4e-5)
+        else:
+            torch.testing.assert_close(z.cpu(), z_ref, rtol=1.6e-2, atol=1e-5)
+            torch.testing.assert_close(a.grad.cpu(), c.grad, rtol=0, atol=1.1e-3)
+
+
+def test_softmax_router_logits_shape_and_sharp_rows(device):
+    # what a load-balancing loss does with the router logits the MoE layer returns: softmax over E, mean over tokens
+    g = torch.Generator().manual_seed(1)
+    logits = (4 * torch.randn(16384, 64, generator=g)).to(torch.bfloat16)
+    p = cute_kernels.softmax_cute(logits.to(device))
+    torch.testing.assert_close(p.float().cpu(), mo.softmax_torch(logits).float(), rtol=1.6e-2, atol=1e-6)
+    # large-magnitude rows (max subtraction) and a weighted backward
+    x = torch.randn(33, 4096, generator=g) * 30
+    w = torch.randn(33, 4096, generator=g)
+    a, c = x.clone().to(device).requires_grad_(), x.clone().requires_grad_()
+    (cute_kernels.softmax_cute(a, 0.5) * w.to(device)).sum().backward()
+    (mo.softmax_torch(c, 0.5) * w).sum().backward()
+    torch.testing.assert_close(a.grad.cpu(), c.grad, rtol=1e-4, atol=1e-6)

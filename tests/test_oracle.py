@@ -244,3 +244,20 @@ def test_fused_residual_add_rmsnorm_closed_form():
     xb, rb = x.to(torch.bfloat16), r.to(torch.bfloat16)
     _, added_b = mo.fused_residual_add_rmsnorm_torch(xb, rb, None, 1e-5, 0.9)
     assert torch.equal(added_b, ((xb.float() * 0.9).to(torch.bfloat16).float() + rb.float()).to(torch.bfloat16))
+
+
+def test_softmax_closed_form_and_jacobian():
+    g = torch.Generator().manual_seed(9)
+    x = torch.randn(5, 17, generator=g, dtype=torch.float64, requires_grad=True)
+    for mult in (None, 0.7):
+        m = 1.0 if mult is None else mult
+        y = mo.softmax_torch(x, mult)
+        e = torch.exp(m * x.detach() - (m * x.detach()).amax(-1, keepdim=True))  # written out, not through F.softmax
+        torch.testing.assert_close(y.detach().double(), e / e.sum(-1, keepdim=True), rtol=1e-6, atol=1e-7)  # fp32 inside
+        assert torch.allclose(y.sum(-1).double(), torch.ones(5, dtype=torch.float64), atol=1e-6)
+        # backward closed form: d_x = m * y * (d_y - sum(d_y * y)); a dropped multiplier or sign would show
+        dy = torch.randn(5, 17, generator=g, dtype=torch.float64)
+        (gx,) = torch.autograd.grad(y, x, dy.to(y.dtype))
+        yd = y.detach().double()
+        torch.testing.assert_close(gx, m * yd * (dy - (dy * yd).sum(-1, keepdim=True)), rtol=1e-5, atol=1e-6)
+    assert mo.softmax_torch(x.detach().to(torch.bfloat16), 0.7).dtype == torch.bfloat16
