@@ -40,10 +40,11 @@ struct GemmParams {
   void* trace;           // measurement builds only: per-workgroup phase timestamps (8 x uint64 each), else NULL
 };
 
-// The 256 x 384 tile variant of the 16-bit kernel (grouped_gemm_wide.hip): modes kGrouped, kScatter, kSwiglu, kDw.
-// The caller fills `prm` for these tile dimensions (n_tiles, m_tiles) and sizes the grid accordingly.
-constexpr int kWideBM = 256, kWideBN = 384;
-int launch_wide(const GemmParams& prm, int mode, int dtype, unsigned blocks, hipStream_t stream, const char* name);
+// The 16-bit kernel with 128-byte LDS rows (grouped_gemm_line.hip): 256 x bn tiles, bn = 256 or 384, contraction length a
+// multiple of 64, modes kGrouped, kScatter, kSwiglu, kDw. The caller fills `prm` for these tile dimensions (n_tiles,
+// m_tiles) and sizes the grid accordingly.
+constexpr int kLineBM = 256, kLineK = 64;
+int launch_line(const GemmParams& prm, int mode, int bn, int dtype, unsigned blocks, hipStream_t stream, const char* name);
 
 namespace {
 

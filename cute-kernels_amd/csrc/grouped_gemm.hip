@@ -37,24 +37,27 @@ const bool g_eight_waves = [] {
   return !(env != nullptr && env[0] == '4');
 }();
 
-// CK_GEMM_TILE=256 / 384 in the environment forces the 256 x 256 / 256 x 384 block tile wherever both are possible
-// (A/B measurements); otherwise the choice follows the column utilisation, see use_wide_tile
-inline int forced_tile() {  // read per call, so that tests can switch it inside one process
+// CK_GEMM_LINE=0 in the environment keeps every launch on the kernels of this file (A/B measurements); CK_GEMM_TILE=256 /
+// 384 forces the width of the 128-byte-row kernel's tile. Both are read per call, so tests can switch them in-process.
+inline bool line_kernel_enabled() {
+  const char* env = getenv("CK_GEMM_LINE");
+  return !(env != nullptr && env[0] == '0');
+}
+inline int forced_tile() {
   const char* env = getenv("CK_GEMM_TILE");
   return env == nullptr ? 0 : atoi(env);
 }
 
 // 256 x 384 tiles carry 20 % more FLOPs per byte loaded from L2 but pay more for the ragged column edge and for their
-// (longer) epilogue. Measured at the Mixtral shape: +10 % with a long contraction (scatter epilogue, K = 14,336 / 28,672),
-// +4 % for the weight gradients, nothing at K = 4,096 -- so they serve those two cases, when the padded column count does
-// not eat the gain. `cols` output columns, `narrow` / `wide` columns per tile, `contraction`: (average) K.
-inline bool use_wide_tile(int64_t cols, int narrow, int wide, int64_t contraction) {
-  if (forced_tile() == 256) return false;
-  if (forced_tile() == 384) return true;
-  if (contraction < 2048) return false;  // short contractions are dominated by the per-tile epilogue: more, smaller tiles
+// (longer) epilogue: they serve long contractions, when the padded column count does not eat the gain.
+// `cols` output columns, `narrow` / `wide` columns per tile, `contraction`: (average) K.
+inline int line_tile_width(int64_t cols, int narrow, int wide, int64_t contraction) {
+  if (forced_tile() == 256) return 256;
+  if (forced_tile() == 384) return 384;
+  if (contraction < 2048) return 256;  // short contractions are dominated by the per-tile epilogue: more, smaller tiles
   const double util_narrow = (double)cols / (double)(ceil_div(cols, narrow) * narrow);
   const double util_wide = (double)cols / (double)(ceil_div(cols, wide) * wide);
-  return util_wide * 1.05 > util_narrow;
+  return util_wide * 1.05 > util_narrow ? 384 : 256;
 }
 
 // PIPE 0: K step 64, global -> registers -> padded LDS, two stages (any K % 8 == 0).
@@ -825,14 +828,14 @@ extern "C" int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* 
   hipStream_t s = static_cast<hipStream_t>(stream);
   // kSwiglu tiles cover BN/2 activation columns each
   auto n_tiles_for = [&](int bn) { return (int)ceil_div(out_cols, epilogue == CK_EPI_SWIGLU ? bn / 2 : bn); };
-  const bool wide_mode = forced_tile() == 384 ? epilogue != CK_EPI_SWIGLU_BWD : epilogue == CK_EPI_SCATTER;
-  if (seg->align == kWideBM && K % 32 == 0 && wide_mode && !g_force_pipe0 &&
-      use_wide_tile(out_cols, epilogue == CK_EPI_SWIGLU ? 128 : 256, epilogue == CK_EPI_SWIGLU ? kWideBN / 2 : kWideBN,
-                    forced_tile() == 384 ? 1 << 20 : (K >= 8192 ? K : 0))) {
-    prm.n_tiles = n_tiles_for(kWideBN);
-    const int64_t wide_blocks = m_tiles * prm.n_tiles;
-    CK_REQUIRE(wide_blocks < (int64_t)0x7fffffff, "%s: grid too large", name);
-    return launch_wide(prm, epilogue, dtype, (unsigned)wide_blocks, s, name);
+  if (seg->align == kLineBM && K % kLineK == 0 && epilogue != CK_EPI_SWIGLU_BWD && !g_force_pipe0 && line_kernel_enabled()) {
+    const bool swiglu = epilogue == CK_EPI_SWIGLU;
+    const int bn = epilogue == CK_EPI_SCATTER ? line_tile_width(out_cols, 256, 384, K >= 8192 ? K : 0)
+                                              : (forced_tile() == 384 ? 384 : 256);
+    prm.n_tiles = (int)ceil_div(out_cols, swiglu ? bn / 2 : bn);
+    const int64_t line_blocks = m_tiles * prm.n_tiles;
+    CK_REQUIRE(line_blocks < (int64_t)0x7fffffff, "%s: grid too large", name);
+    return launch_line(prm, epilogue, bn, dtype, (unsigned)line_blocks, s, name);
   }
   const int bn = seg->align;  // square tiles
   prm.n_tiles = n_tiles_for(bn);
@@ -882,12 +885,13 @@ extern "C" int ck_grouped_gemm_dw(const void* a_t, const void* b_t, int64_t ld_t
   hipStream_t s = static_cast<hipStream_t>(stream);
   // tile size follows the problem, not the segment alignment: small weight matrices get 128x128 tiles
   const bool big = (M >= 1024 && N >= 1024);
-  if (big && !g_force_pipe0 && use_wide_tile(N, 256, kWideBN, seg->max_rows / seg->num_experts)) {
-    prm.m_tiles = (int)ceil_div(M, kWideBM);
-    prm.n_tiles = (int)ceil_div(N, kWideBN);
-    const int64_t wide_blocks = (int64_t)prm.m_tiles * prm.n_tiles * seg->num_experts;
-    CK_REQUIRE(wide_blocks < (int64_t)0x7fffffff, "%s: grid too large", name);
-    return launch_wide(prm, kDw, dtype, (unsigned)wide_blocks, s, name);
+  if (big && !g_force_pipe0 && line_kernel_enabled()) {
+    const int bn = line_tile_width(N, 256, 384, seg->max_rows / seg->num_experts);
+    prm.m_tiles = (int)ceil_div(M, kLineBM);
+    prm.n_tiles = (int)ceil_div(N, bn);
+    const int64_t line_blocks = (int64_t)prm.m_tiles * prm.n_tiles * seg->num_experts;
+    CK_REQUIRE(line_blocks < (int64_t)0x7fffffff, "%s: grid too large", name);
+    return launch_line(prm, kDw, bn, dtype, (unsigned)line_blocks, s, name);
   }
   const int bt = big ? 256 : 128;
   prm.m_tiles = (int)ceil_div(M, bt);

@@ -58,7 +58,7 @@ def _make_case(device, dtype, T, k, E, align, empty=(3,), seed=0):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("align", [128, 256])
-@pytest.mark.parametrize("K,N", [(200, 136), (64, 128), (576, 264), (160, 840)])
+@pytest.mark.parametrize("K,N", [(200, 136), (64, 128), (576, 264), (160, 840), (192, 840), (320, 392)])
 def test_grouped_gemm_gather_in_grouped_out(device, dtype, align, K, N, gemm_tile):
     T, k, E = 300, 2, 5
     g, seg = _make_case(device, dtype, T, k, E, align)
@@ -75,7 +75,7 @@ def test_grouped_gemm_gather_in_grouped_out(device, dtype, align, K, N, gemm_til
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("align", [128, 256])
-@pytest.mark.parametrize("K,N", [(136, 200), (160, 840)])
+@pytest.mark.parametrize("K,N", [(136, 200), (160, 840), (128, 840), (320, 264)])
 def test_grouped_gemm_grouped_in_scatter_out(device, dtype, align, K, N, gemm_tile):
     T, k, E = 300, 2, 5
     g, seg = _make_case(device, dtype, T, k, E, align, seed=1)
@@ -95,7 +95,7 @@ def test_grouped_gemm_grouped_in_scatter_out(device, dtype, align, K, N, gemm_ti
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("align", [128, 256])
-@pytest.mark.parametrize("K,I", [(200, 72), (128, 256), (64, 136), (96, 440)])
+@pytest.mark.parametrize("K,I", [(200, 72), (128, 256), (64, 136), (96, 440), (192, 440)])
 def test_grouped_gemm_swiglu_epilogues(device, dtype, align, K, I, gemm_tile):
     T, k, E = 300, 2, 5
     g, seg = _make_case(device, dtype, T, k, E, align, seed=2)
