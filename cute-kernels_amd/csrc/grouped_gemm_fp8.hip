@@ -2,10 +2,11 @@
 // Forward (inference) only: Y = (A_e * diag(a_scale)) (W[e] * diag(w_scale[e]))^T, the two scale vectors applied to the
 // fp32 accumulators in the epilogue.
 //
-// Same machinery as the 16-bit kernel (tile-aligned expert segments, 256x256 tile, 8 waves, global -> LDS direct loads,
-// four XOR-swizzled 64-byte-row stages, hand-ordered load / fragment-read / MFMA stream, LDS-staged epilogue), with one
-// byte per element: a K step is 64 elements = one v_mfma_f32_32x32x64_f8f6f4 per 32 x 32 block (twice the rate of the
-// 16-bit MFMA), fragments are 32 bytes per lane, and every byte fetched from L2 carries twice the FLOPs.
+// Same machinery as the 16-bit kernel with 128-byte LDS rows (tile-aligned expert segments, 256x256 tile, 8 waves,
+// global -> LDS direct loads of whole cache lines, two XOR-swizzled stages, hand-ordered load / fragment-read / MFMA
+// stream, LDS-staged epilogue), with one byte per element: a K step is 128 elements = two v_mfma_f32_32x32x64_f8f6f4 per
+// 32 x 32 block (twice the rate of the 16-bit MFMA), fragments are 32 bytes per lane, and every byte fetched from L2
+// carries twice the FLOPs.
 #include <stdlib.h>
 
 #include "gemm_common.h"
@@ -21,10 +22,13 @@ constexpr int BM = 256, BN = 256;
 constexpr int WGM = 4, NW = WGM * 2, NT = 64 * NW;  // 8 waves: 4 along M, 2 along N
 constexpr int WM = BM / WGM, WN = BN / 2;           // 64 x 128 wave tile
 constexpr int MI = WM / 32, NI = WN / 32;
-constexpr int BK = 64, NSTAGE = 4;
-constexpr int kRowBytes = 64;
+constexpr int BK = 128, KS = BK / 64, NSTAGE = 2;
+constexpr int kRowBytes = BK;  // one cache line per tile row and K step
 constexpr int kStageBytes = (BM + BN) * kRowBytes;
-constexpr int A_LD = BM / (16 * NW), B_LD = BN / (16 * NW);
+constexpr int A_LD = BM * kRowBytes / (1024 * NW), B_LD = BN * kRowBytes / (1024 * NW);
+// 16-byte chunk c of row r sits in slot c ^ swz128(r): 16 lanes reading one chunk index of 16 consecutive rows then touch
+// all 64 banks once (even rows cover banks 0-31 with 8 distinct slots, odd rows 32-63)
+__device__ inline int swz128(int row) { return (row >> 1) & 7; }
 constexpr int kLoadsPerStep = A_LD + B_LD;
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x8 __attribute__((ext_vector_type(8)));
@@ -70,14 +74,14 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
-  // ---- global -> LDS addressing: lane l of a wave-load fills slot l (16 bytes) of 64 consecutive slots = 16 rows
+  // ---- global -> LDS addressing: lane l of a wave-load fills slot l (16 bytes) of 64 consecutive slots = 8 rows of 128 B
   const char* a_base = static_cast<const char*>(prm.a);
   const char* b_base = static_cast<const char*>(prm.w) + (int64_t)expert * prm.w_expert_stride;
   uint32_t a_off[A_LD], b_off[B_LD];
 #pragma unroll
   for (int t = 0; t < A_LD; ++t) {
-    const int r = (wave * A_LD + t) * 16 + (lane >> 2);
-    const int c = (lane & 3) ^ lds_swizzle(r);
+    const int r = (wave * A_LD + t) * 8 + (lane >> 3);
+    const int c = (lane & 7) ^ swz128(r);
     int64_t p = m0 + r;
     if (p >= valid_end) p = valid_end - 1;  // pad rows re-read a valid row; their results are never stored
     const int64_t row = prm.a_gather_div > 0 ? (int64_t)(prm.row_slot[p] / prm.a_gather_div) : p;
@@ -85,8 +89,8 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
   }
 #pragma unroll
   for (int t = 0; t < B_LD; ++t) {
-    const int j = (wave * B_LD + t) * 16 + (lane >> 2);
-    const int c = (lane & 3) ^ lds_swizzle(j);
+    const int j = (wave * B_LD + t) * 8 + (lane >> 3);
+    const int c = (lane & 7) ^ swz128(j);
     int64_t n;
     if constexpr (MODE == kSwiglu) {
       const int half = (j % WN) / (WN / 2);
@@ -129,10 +133,10 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
   const uint32_t wave_a = __builtin_amdgcn_readfirstlane(lds_base + wave * A_LD * 1024);
   const uint32_t wave_b = __builtin_amdgcn_readfirstlane(lds_base + BM * kRowBytes + wave * B_LD * 1024);
   auto issue_one = [&](int step, int g) {
-    const int64_t kb = (int64_t)min(step, nk - 1) * kRowBytes;  // past the end: re-fetch the last step (never read)
+    const int64_t kb = (int64_t)step * kRowBytes;
     const uint32_t st = (uint32_t)((step & (NSTAGE - 1)) * kStageBytes);
     if constexpr ((CK_ABLATE & 2) != 0) {
-      if (step >= NSTAGE - 1) return;
+      if (step >= NSTAGE) return;
     }
     if (g < A_LD) dma16(a_base + kb + a_off[g], wave_a + st + g * 1024);
     else dma16(b_base + kb + b_off[g - A_LD], wave_b + st + (g - A_LD) * 1024);
@@ -142,20 +146,26 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
     for (int g = 0; g < kLoadsPerStep; ++g) issue_one(step, g);
   };
 
-  // ---- fragments for v_mfma_f32_32x32x64_f8f6f4: lane l holds 32 bytes of row l % 32 -- 16-byte chunks 2h and 2h + 1 of
-  // the 64-byte row, h = l / 32. Both operands use the same byte -> k assignment, which is all a dot product needs.
-  const int fsw = lds_swizzle(lane & 31), fh = lane >> 5;
-  const int chunk_lo = ((2 * fh) ^ fsw) * 16, chunk_hi = ((2 * fh + 1) ^ fsw) * 16;
+  // ---- fragments for v_mfma_f32_32x32x64_f8f6f4: slice sl (64 of the row's 128 bytes) of row l % 32 -- lane l holds its
+  // 16-byte chunks 4 sl + 2 h and 4 sl + 2 h + 1, h = l / 32. Both operands use the same byte -> k assignment, which is
+  // all a dot product needs.
+  const int fsw = swz128(lane & 31), fh = lane >> 5;
+  int chunk_lo[KS], chunk_hi[KS];
+#pragma unroll
+  for (int sl = 0; sl < KS; ++sl) {
+    chunk_lo[sl] = ((4 * sl + 2 * fh) ^ fsw) * 16;
+    chunk_hi[sl] = ((4 * sl + 2 * fh + 1) ^ fsw) * 16;
+  }
   const int fa_row = (wm * WM + (lane & 31)) * kRowBytes;
   const int fb_row = BM * kRowBytes + (wn * WN + (lane & 31)) * kRowBytes;
   i32x8 fa[MI], fb[NI];
-  auto read_frag = [&](int stage, int g) {  // g < MI: A block g; else B block g - MI
+  auto read_frag = [&](int stage, int sl, int g) {  // g < MI: A block g; else B block g - MI
     if constexpr ((CK_ABLATE & 4) != 0) {
-      if (stage != 0) return;
+      if (stage != 0 || sl != 0) return;
     }
     const char* row = lds_c + stage * kStageBytes + (g < MI ? fa_row + g * 32 * kRowBytes : fb_row + (g - MI) * 32 * kRowBytes);
-    const i32x4 lo = *reinterpret_cast<const i32x4*>(row + chunk_lo);
-    const i32x4 hi = *reinterpret_cast<const i32x4*>(row + chunk_hi);
+    const i32x4 lo = *reinterpret_cast<const i32x4*>(row + chunk_lo[sl]);
+    const i32x4 hi = *reinterpret_cast<const i32x4*>(row + chunk_hi[sl]);
     const i32x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     if (g < MI) fa[g] = v;
     else fb[g - MI] = v;
@@ -168,58 +178,54 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
     // scale operands 0: the compiler emits the unscaled v_mfma_f32_32x32x64_f8f6f4 (both operands e4m3: cbsz = blgp = 0)
     acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], 0, 0, 0, 0, 0, 0);
   };
-  static_assert(MI == 2 && NI == 4 && kLoadsPerStep == 4, "the hand schedule below is written for a 64 x 128 wave tile");
+  static_assert(MI == 2 && NI == 4 && kLoadsPerStep == 8 && KS == 2, "the hand schedule below is written for this shape");
 
-  stamp(1);
   if (nk > 0) {
     issue(0);
-    issue(1);
-    issue(2);
-    asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(2 * kLoadsPerStep) : "memory");  // step 0 landed, all waves
+    if (nk > 1) {
+      issue(1);
+      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kLoadsPerStep) : "memory");  // step 0 landed, all waves
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    }
 #pragma unroll
-    for (int g = 0; g < MI + NI; ++g) read_frag(0, g);
-    // One 64-byte K step per iteration = one MFMA per 32 x 32 block. Fragments are single-buffered and rotate: as soon
-    // as the last MFMA that needs a fragment has issued, the same registers are reloaded from the next step's stage.
-    // phase 0: steady state (prefetch step kt + 3, steps kt + 1 and kt + 2 in flight); phase 1: step nk - 3 (nothing left
-    // to prefetch, same wait); phase 2: the last two steps (at most one step in flight: wait for everything)
-    auto k_step = [&](int kt, auto phase) {
-      constexpr bool kTail = decltype(phase)::value > 0;
-      constexpr bool kWaitAll = decltype(phase)::value > 1;
-      const int next = (kt + 1) & (NSTAGE - 1);
-      mfma(0, 0);
-      mfma(0, 1);
-      mfma(0, 2);
-      mfma(0, 3);
-      __builtin_amdgcn_sched_barrier(0);
-      // step kt + 1 has landed for every wave (only step kt + 2 may be in flight); every fragment read of stage
-      // (kt + 3) % 4 was consumed before the barrier of step kt - 1, so its overwrite below is ordered too
-      if constexpr (kWaitAll) asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-      else asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kLoadsPerStep) : "memory");
-      read_frag(next, 0);
-      if constexpr (!kTail) issue_one(kt + 3, 0);
-      mfma(1, 0);
-      __builtin_amdgcn_sched_barrier(0);
-      read_frag(next, MI + 0);
-      if constexpr (!kTail) issue_one(kt + 3, 1);
-      mfma(1, 1);
-      __builtin_amdgcn_sched_barrier(0);
-      read_frag(next, MI + 1);
-      if constexpr (!kTail) issue_one(kt + 3, 2);
-      mfma(1, 2);
-      __builtin_amdgcn_sched_barrier(0);
-      read_frag(next, MI + 2);
-      if constexpr (!kTail) issue_one(kt + 3, 3);
-      mfma(1, 3);
-      __builtin_amdgcn_sched_barrier(0);
-      read_frag(next, MI + 3);
-      read_frag(next, 1);
+    for (int g = 0; g < MI + NI; ++g) read_frag(0, 0, g);
+    // One 64-byte slice = one MFMA per 32 x 32 block. Fragments are single-buffered and rotate: as soon as the last MFMA
+    // that needs a fragment has issued, the same registers are reloaded for the next slice.
+    // Slice 0: the next slice is in the same stage. Slice 1 (last): the next slice is slice 0 of step kt + 1 in the other
+    // stage -- phase 0 / 1: wait for that stage (the only loads in flight) and for this wave's own fragment reads, then
+    // meet the other waves; the whole current stage has been read by everyone, so in phase 0 the loads of step kt + 2
+    // overwrite it under this slice's MFMAs. Phase 1 is step nk - 2 (nothing left to fetch), phase 2 the last step.
+    auto slice = [&](int kt, auto sl, auto phase) {
+      constexpr bool kLast = decltype(sl)::value == KS - 1;
+      constexpr int kPhase = decltype(phase)::value;
+      const int ns = kLast ? (kt + 1) & (NSTAGE - 1) : kt & (NSTAGE - 1);
+      constexpr int nsl = kLast ? 0 : decltype(sl)::value + 1;
+      constexpr bool kReload = !(kLast && kPhase == 2);
+      constexpr bool kIssue = kLast && kPhase == 0;
+      if constexpr (kLast && kPhase < 2) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+#pragma unroll
+      for (int j = 0; j < NI; ++j) {
+        mfma(0, j);
+        if constexpr (kIssue) issue_one(kt + 2, j);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      if constexpr (kReload) read_frag(ns, nsl, 0);
+#pragma unroll
+      for (int j = 0; j < NI; ++j) {
+        mfma(1, j);
+        if constexpr (kIssue) issue_one(kt + 2, NI + j);
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (kReload) read_frag(ns, nsl, MI + j);
+      }
+      if constexpr (kReload) read_frag(ns, nsl, 1);
       __builtin_amdgcn_sched_barrier(0);
     };
-    // a prefetch past the end would only re-fetch the last step and waste L2 bandwidth
+    auto k_step = [&](int kt, auto phase) { static_for<KS>([&](auto sl) { slice(kt, sl, phase); }); };
     int kt = 0;
-    for (; kt + 3 < nk; ++kt) k_step(kt, std::integral_constant<int, 0>{});
-    if (kt + 3 == nk) k_step(kt++, std::integral_constant<int, 1>{});
-    for (; kt < nk; ++kt) k_step(kt, std::integral_constant<int, 2>{});
+    for (; kt + 2 < nk; ++kt) k_step(kt, std::integral_constant<int, 0>{});
+    if (kt + 2 == nk) k_step(kt++, std::integral_constant<int, 1>{});
+    k_step(kt, std::integral_constant<int, 2>{});
   }
 
   // ---- epilogue through LDS (see the 16-bit kernel): slab S[col][row] of 128 tile columns, 8-byte writes from the
@@ -476,7 +482,7 @@ extern "C" int ck_grouped_gemm_fp8(const void* a8, const float* a_scale, int32_t
   if (int rc = check_segments(seg, name)) return rc;
   CK_REQUIRE(seg->align == 256, "%s: fp8 tiles are 256 rows high; sort with align = 256", name);
   CK_REQUIRE(N >= 8 && N % 8 == 0, "%s: N=%d must be a positive multiple of 8", name, N);
-  CK_REQUIRE(K >= 64 && K % 64 == 0, "%s: K=%d must be a positive multiple of 64", name, K);
+  CK_REQUIRE(K >= 128 && K % 128 == 0, "%s: K=%d must be a positive multiple of 128", name, K);
   CK_REQUIRE(a_gather_div >= 0, "%s: a_gather_div=%d is negative", name, a_gather_div);
   CK_REQUIRE(epilogue == CK_EPI_GROUPED || epilogue == CK_EPI_SCATTER || epilogue == CK_EPI_SWIGLU,
              "%s: epilogue %d is not available in fp8 (grouped, scatter, swiglu)", name, epilogue);

@@ -100,8 +100,8 @@ class MoE_E4M3(nn.Module):
         super().__init__()
         assert moe.is_glu, "the fp8 expert path implements the packed SwiGLU layer"
         assert moe.c_fc.bias is None and moe.c_proj.bias is None, "expert biases are not supported"
-        assert moe.hidden_size % 64 == 0 and moe.intermediate_size % 64 == 0, (
-            "the fp8 GEMMs need hidden_size and intermediate_size to be multiples of 64"
+        assert moe.hidden_size % 128 == 0 and moe.intermediate_size % 128 == 0, (
+            "the fp8 GEMMs need hidden_size and intermediate_size to be multiples of 128"
         )
         self.num_experts = moe.num_experts
         self.top_k = moe.top_k

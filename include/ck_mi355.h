@@ -182,7 +182,7 @@ int ck_grouped_gemm_dw(const void* a_t, const void* b_t, int64_t ld_t, int32_t M
 int ck_quant_rows_e4m3(const void* x, int64_t rows, int32_t cols, void* q, float* scales, int32_t dtype, void* stream);
 /* Y = (A_e * diag(a_scale)) * (W[e] * diag(w_scale[e]))^T over tile-aligned expert segments (align must be 256).
  * a8: e4m3 rows [*, K], gathered like ck_grouped_gemm (a_gather_div); a_scale is indexed by the row of a8 that is read.
- * w8 [E, N, K] e4m3, w_scale [E, N]. K % 64 == 0. Epilogues: CK_EPI_GROUPED (y [max_rows, N]), CK_EPI_SCATTER
+ * w8 [E, N, K] e4m3, w_scale [E, N]. K % 128 == 0. Epilogues: CK_EPI_GROUPED (y [max_rows, N]), CK_EPI_SCATTER
  * (y [R, N]), CK_EPI_SWIGLU (N = 2I packed [up | gate]; only the activation is written, to aux [max_rows, I]).
  * Outputs have `out_dtype` (bf16 / f16). */
 int ck_grouped_gemm_fp8(const void* a8, const float* a_scale, int32_t a_gather_div, const void* w8,

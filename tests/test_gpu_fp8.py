@@ -42,7 +42,7 @@ def _segments(device, T, k, E, seed, empty=()):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("K,N", [(64, 128), (256, 264), (1024, 512)])
+@pytest.mark.parametrize("K,N", [(128, 128), (256, 264), (384, 72), (1024, 512)])
 def test_grouped_gemm_fp8_grouped_and_scatter(device, dtype, K, N):
     T, k, E = 300, 2, 5
     g, ids, seg = _segments(device, T, k, E, seed=K + N, empty=(3,))
@@ -80,7 +80,7 @@ def test_grouped_gemm_fp8_grouped_and_scatter(device, dtype, K, N):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-@pytest.mark.parametrize("T,E,k,H,I", [(257, 8, 2, 128, 256), (33, 4, 4, 64, 192), (700, 16, 8, 256, 320)])
+@pytest.mark.parametrize("T,E,k,H,I", [(257, 8, 2, 128, 256), (33, 4, 4, 128, 384), (700, 16, 8, 256, 640)])
 def test_moe_e4m3_layer_forward(device, dtype, T, E, k, H, I):
     torch.manual_seed(E + k)
     moe = cute_kernels.MoE(E, k, H, I, cute_kernels.swiglu_packed_cute, True, False, 0.02).to(dtype)
@@ -106,9 +106,9 @@ def test_moe_e4m3_layer_forward(device, dtype, T, E, k, H, I):
 
 def test_fp8_rejects_unsupported(device):
     g, ids, seg128 = None, None, cute_kernels.sort_by_expert(torch.zeros(64, dtype=torch.int32, device=device), 2, 128)
-    x8 = torch.zeros(64, 64, dtype=torch.float8_e4m3fn, device=device)
+    x8 = torch.zeros(64, 128, dtype=torch.float8_e4m3fn, device=device)
     s = torch.ones(64, device=device)
-    w8 = torch.zeros(2, 64, 64, dtype=torch.float8_e4m3fn, device=device)
+    w8 = torch.zeros(2, 64, 128, dtype=torch.float8_e4m3fn, device=device)
     ws = torch.ones(2, 64, device=device)
     y = torch.zeros(seg128.max_rows, 64, dtype=torch.bfloat16, device=device)
     with pytest.raises(RuntimeError, match="256"):
