@@ -5,9 +5,11 @@
 // "NT": both operands are contraction-contiguous (the backward passes get that from transposed copies written by the
 // producing epilogues), so global loads are 128-bit along K and LDS fragments feed v_mfma_f32_32x32x16 directly.
 //
-// Workgroup = 256 threads = 4 waves in a 2x2 grid; wave tile (BM/2)x(BN/2) built from 32x32 MFMA blocks; K step 64
-// staged through double-buffered LDS (rows padded to 72 elements so 16 lanes x 16 bytes cover all banks); the global
-// loads of step k+1 are in flight while step k is multiplied.
+// This file holds the general kernel (256 x 256 or 128 x 128 tiles, any K % 8 == 0, every epilogue) and the two C entry
+// points. Launches with 256-row alignment and a contraction length that is a multiple of 64 go to the kernel with
+// 128-byte LDS rows in grouped_gemm_line.hip instead. Here: workgroup = 8 waves in a 4 x 2 grid (or 4 in 2 x 2), wave
+// tiles built from 32x32 MFMA blocks, and two pipelines -- K step 32 straight from global memory into four swizzled LDS
+// stages (K % 32 == 0), or K step 64 through registers into two padded LDS stages (any K % 8 == 0).
 #include <stdlib.h>
 
 #include "gemm_common.h"

@@ -235,6 +235,74 @@ inline unsigned grid_for(int64_t work_items, int per_thread) {
   return (unsigned)b;
 }
 
+
+// ---- expert biases (the reference's Experts_Torch applies one bias row per expert: torch_implementation.py:20-22,42) ----
+// y[r, :] += bias[e(r), :]. Grouped rows: e(r) is the expert of the row's tile, pad rows are skipped. Token-order rows
+// (row_expert != nullptr): e(r) = row_expert[r], negative = skip.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void add_expert_bias_kernel(T* __restrict__ y, int64_t rows, int N,
+                                                                  const T* __restrict__ bias,
+                                                                  const int32_t* __restrict__ row_expert,
+                                                                  const int32_t* __restrict__ seg_starts,
+                                                                  const uint32_t* __restrict__ counts,
+                                                                  const int32_t* __restrict__ tile_expert, int align) {
+  const int chunks = N / 8;
+  for (int64_t r = blockIdx.y; r < rows; r += gridDim.y) {
+    int e;
+    if (row_expert != nullptr) {
+      e = row_expert[r];
+    } else {
+      e = tile_expert[r / align];
+      if (e >= 0 && r >= (int64_t)seg_starts[e] + counts[e]) e = -1;
+    }
+    if (e < 0) continue;
+    for (int ch = blockIdx.x * kBlock + threadIdx.x; ch < chunks; ch += gridDim.x * kBlock) {
+      Pack16<T> v, b;
+      v.v = load16(y + r * N + ch * 8);
+      b.v = load16(bias + (int64_t)e * N + ch * 8);
+#pragma unroll
+      for (int i = 0; i < 8; ++i) v.e[i] = Elem<T>::down(Elem<T>::up(v.e[i]) + Elem<T>::up(b.e[i]));
+      store16(y + r * N + ch * 8, v.v);
+    }
+  }
+}
+
+// d_bias[e, :] = sum over the rows of expert e of d_y (padded grouped rows), fp32 accumulation in a fixed order.
+// grid (ceil(N / 64), E); a block owns 64 columns, its 4 waves split the rows, 8 loads in flight per wave.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void expert_bias_grad_kernel(const T* __restrict__ d_y, int N,
+                                                                   const int32_t* __restrict__ seg_starts,
+                                                                   const uint32_t* __restrict__ counts,
+                                                                   T* __restrict__ d_bias) {
+  __shared__ float part[kBlock / kWave][kWave];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int e = blockIdx.y, col = blockIdx.x * kWave + lane;
+  const int64_t first = seg_starts[e], last = first + counts[e];
+  float s = 0.f;
+  if (col < N) {
+    constexpr int U = 8, W = kBlock / kWave;
+    float acc[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) acc[u] = 0.f;
+    int64_t r = first + wave;
+    for (; r + (U - 1) * W < last; r += U * W) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) acc[u] += Elem<T>::up(d_y[(r + u * W) * N + col]);
+    }
+    for (; r < last; r += W) acc[0] += Elem<T>::up(d_y[r * N + col]);
+#pragma unroll
+    for (int u = 0; u < U; ++u) s += acc[u];
+  }
+  part[wave][lane] = s;
+  __syncthreads();
+  if (wave == 0 && col < N) {
+    float t = 0.f;
+#pragma unroll
+    for (int g = 0; g < kBlock / kWave; ++g) t += part[g][lane];
+    d_bias[(int64_t)e * N + col] = Elem<T>::down(t);
+  }
+}
+
 }  // namespace
 }  // namespace ck
 
@@ -359,5 +427,44 @@ extern "C" int ck_transpose_batched(const void* src, int64_t batch, int32_t rows
                        static_cast<const scalar_t*>(src), (int)rows, (int)cols, static_cast<scalar_t*>(dst));
   });
   CK_CHECK_LAUNCH("ck_transpose_batched");
+  return CK_OK;
+}
+
+extern "C" int ck_add_expert_bias(void* y, int64_t rows, int32_t N, const void* bias, const int32_t* row_expert,
+                                  const ck_segments* seg, int32_t dtype, void* stream) {
+  const char* name = "ck_add_expert_bias";
+  CK_REQUIRE(rows >= 0 && N >= 8 && N % 8 == 0, "%s: N=%d must be a positive multiple of 8", name, N);
+  if (rows == 0) return CK_OK;
+  CK_REQUIRE(y && bias && aligned16(y) && aligned16(bias), "%s: NULL or misaligned pointer", name);
+  CK_REQUIRE(row_expert != nullptr || seg != nullptr, "%s: give row_expert (token-order rows) or seg (grouped rows)", name);
+  CK_REQUIRE(row_expert != nullptr || (seg->seg_starts && seg->counts && seg->tile_expert && seg->align >= 1 &&
+                                        rows <= seg->max_rows),
+             "%s: seg is incomplete or has fewer rows than y", name);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)ceil_div(N / 8, kBlock), (unsigned)(rows < 65535 ? rows : 65535));
+  CK_DISPATCH_HALF(dtype, name, {
+    hipLaunchKernelGGL((add_expert_bias_kernel<scalar_t>), grid, dim3(kBlock), 0, s, static_cast<scalar_t*>(y), rows, (int)N,
+                       static_cast<const scalar_t*>(bias), row_expert, row_expert ? nullptr : seg->seg_starts,
+                       row_expert ? nullptr : seg->counts, row_expert ? nullptr : seg->tile_expert,
+                       row_expert ? 1 : seg->align);
+  });
+  CK_CHECK_LAUNCH(name);
+  return CK_OK;
+}
+
+extern "C" int ck_expert_bias_grad(const void* d_y, int32_t N, const ck_segments* seg, void* d_bias, int32_t dtype,
+                                   void* stream) {
+  const char* name = "ck_expert_bias_grad";
+  CK_REQUIRE(N >= 1, "%s: N=%d must be positive", name, N);
+  CK_REQUIRE(seg && seg->seg_starts && seg->counts && seg->num_experts >= 1 && seg->num_experts <= 65535,
+             "%s: seg is incomplete (or more than 65535 experts)", name);
+  CK_REQUIRE(d_bias != nullptr && (seg->max_rows == 0 || d_y != nullptr), "%s: NULL argument", name);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const dim3 grid((unsigned)ceil_div(N, kWave), (unsigned)seg->num_experts);
+  CK_DISPATCH_HALF(dtype, name, {
+    hipLaunchKernelGGL((expert_bias_grad_kernel<scalar_t>), grid, dim3(kBlock), 0, s, static_cast<const scalar_t*>(d_y),
+                       (int)N, seg->seg_starts, seg->counts, static_cast<scalar_t*>(d_bias));
+  });
+  CK_CHECK_LAUNCH(name);
   return CK_OK;
 }

@@ -74,6 +74,8 @@ _SIGNATURES = {
     "ck_rmsnorm_fwd": (c_int32, [c_void_p, c_void_p, c_float, c_int64, c_int32, c_void_p, c_void_p, c_int32, c_void_p]),
     "ck_rmsnorm_bwd_partial_rows": (c_int64, [c_int64]),
     "ck_rmsnorm_bwd": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_float, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_int32, c_void_p]),
+    "ck_add_expert_bias": (c_int32, [c_void_p, c_int64, c_int32, c_void_p, c_void_p, POINTER(ck_segments), c_int32, c_void_p]),
+    "ck_expert_bias_grad": (c_int32, [c_void_p, c_int32, POINTER(ck_segments), c_void_p, c_int32, c_void_p]),
     "ck_softmax_fwd": (c_int32, [c_void_p, c_float, c_int64, c_int32, c_void_p, c_int32, c_void_p]),
     "ck_softmax_bwd": (c_int32, [c_void_p, c_void_p, c_float, c_int64, c_int32, c_void_p, c_int32, c_void_p]),
     "ck_fused_residual_add_rmsnorm_fwd": (c_int32, [c_void_p, c_void_p, c_void_p, c_float, c_float, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_int32, c_void_p]),

@@ -441,46 +441,50 @@ swiglu_experts.register_autograd(_swiglu_experts_bwd, setup_context=_swiglu_expe
 
 @custom_op(f"{NS}::experts_up", mutates_args=())
 def experts_up(
-    x: Tensor, w: Tensor, seg_starts: Tensor, counts: Tensor, tile_expert: Tensor, row_slot: Tensor, max_rows: int,
-    num_experts: int, align: int, k: int,
+    x: Tensor, w: Tensor, bias: Optional[Tensor], seg_starts: Tensor, counts: Tensor, tile_expert: Tensor, row_slot: Tensor,
+    max_rows: int, num_experts: int, align: int, k: int,
 ) -> Tensor:
     seg = _segments(seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, align)
-    return _moe._ExpertsUp.forward(_Ctx(), x, w, seg, k)
+    return _moe._ExpertsUp.forward(_Ctx(), x, w, seg, k, bias)
 
 
 @experts_up.register_fake
-def _(x, w, seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, align, k):
+def _(x, w, bias, seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, align, k):
     return x.new_empty(max_rows, w.shape[1])
 
 
 @custom_op(f"{NS}::experts_up_backward", mutates_args=())
 def experts_up_backward(
     d_y: Tensor, x: Tensor, w: Tensor, seg_starts: Tensor, counts: Tensor, tile_expert: Tensor, row_slot: Tensor,
-    max_rows: int, num_experts: int, align: int, k: int, need_x: bool, need_w: bool,
-) -> tuple[Tensor, Tensor]:
-    ctx = _Ctx((need_x, need_w, False, False))
+    max_rows: int, num_experts: int, align: int, k: int, need_x: bool, need_w: bool, need_bias: bool,
+) -> tuple[Tensor, Tensor, Tensor]:
+    ctx = _Ctx((need_x, need_w, False, False, need_bias))
     ctx.seg, ctx.k = _segments(seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, align), k
     ctx.saved_tensors = (x.contiguous(), w.contiguous())
-    d_x, d_w, _, _ = _moe._ExpertsUp.backward(ctx, d_y)
-    return _or_empty(d_x, x), _or_empty(d_w, x)
+    d_x, d_w, _, _, d_bias = _moe._ExpertsUp.backward(ctx, d_y)
+    return _or_empty(d_x, x), _or_empty(d_w, x), _or_empty(d_bias, x)
 
 
 @experts_up_backward.register_fake
-def _(d_y, x, w, seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, align, k, need_x, need_w):
+def _(d_y, x, w, seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, align, k, need_x, need_w, need_bias):
     e = x.new_empty(0)
-    return (torch.empty_like(x) if need_x else e), (torch.empty_like(w) if need_w else e)
+    return (
+        torch.empty_like(x) if need_x else e,
+        torch.empty_like(w) if need_w else e,
+        x.new_empty(num_experts, w.shape[1]) if need_bias else e,
+    )
 
 
 def _experts_up_setup(ctx, inputs, output):
-    x, w, seg_starts, counts, tile_expert, row_slot, *rest = inputs
+    x, w, _bias, seg_starts, counts, tile_expert, row_slot, *rest = inputs
     ctx.save_for_backward(x, w, seg_starts, counts, tile_expert, row_slot)
     ctx.rest = tuple(rest)
 
 
 def _experts_up_bwd(ctx, d_y):
-    need_x, need_w = ctx.needs_input_grad[0], ctx.needs_input_grad[1]
-    d_x, d_w = experts_up_backward(d_y.contiguous(), *ctx.saved_tensors, *ctx.rest, need_x, need_w)
-    return (d_x if need_x else None), (d_w if need_w else None), *(None,) * 8
+    need_x, need_w, need_bias = ctx.needs_input_grad[:3]
+    d_x, d_w, d_bias = experts_up_backward(d_y.contiguous(), *ctx.saved_tensors, *ctx.rest, need_x, need_w, need_bias)
+    return (d_x if need_x else None), (d_w if need_w else None), (d_bias if need_bias else None), *(None,) * 8
 
 
 experts_up.register_autograd(_experts_up_bwd, setup_context=_experts_up_setup)
@@ -488,18 +492,18 @@ experts_up.register_autograd(_experts_up_bwd, setup_context=_experts_up_setup)
 
 @custom_op(f"{NS}::experts_down", mutates_args=())
 def experts_down(
-    h: Tensor, w: Tensor, gates: Tensor, seg_starts: Tensor, counts: Tensor, tile_expert: Tensor, row_slot: Tensor,
-    max_rows: int, num_experts: int, align: int,
+    h: Tensor, w: Tensor, gates: Tensor, bias: Optional[Tensor], slot_expert: Optional[Tensor], seg_starts: Tensor,
+    counts: Tensor, tile_expert: Tensor, row_slot: Tensor, max_rows: int, num_experts: int, align: int,
 ) -> tuple[Tensor, Tensor]:
     """(out [T, N], expanded [T * k, N])"""
     ctx = _Ctx()
     seg = _segments(seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, align)
-    out = _moe._ExpertsDown.forward(ctx, h, w, gates, seg)
+    out = _moe._ExpertsDown.forward(ctx, h, w, gates, seg, bias, slot_expert)
     return out, ctx.saved_tensors[3]
 
 
 @experts_down.register_fake
-def _(h, w, gates, seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, align):
+def _(h, w, gates, bias, slot_expert, seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, align):
     T, k = gates.shape
     return h.new_empty(T, w.shape[1]), h.new_empty(T * k, w.shape[1])
 
@@ -508,38 +512,42 @@ def _(h, w, gates, seg_starts, counts, tile_expert, row_slot, max_rows, num_expe
 def experts_down_backward(
     grad_out: Tensor, h: Tensor, w: Tensor, gates: Tensor, expanded: Tensor, seg_starts: Tensor, counts: Tensor,
     tile_expert: Tensor, row_slot: Tensor, max_rows: int, num_experts: int, align: int, need_h: bool, need_w: bool,
-    need_gates: bool,
-) -> tuple[Tensor, Tensor, Tensor]:
-    ctx = _Ctx((need_h, need_w, need_gates, False))
+    need_gates: bool, need_bias: bool,
+) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+    ctx = _Ctx((need_h, need_w, need_gates, False, need_bias))
     ctx.seg = _segments(seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, align)
     ctx.saved_tensors = (h.contiguous(), w.contiguous(), gates.contiguous(), expanded)
-    d_h, d_w, d_gates, _ = _moe._ExpertsDown.backward(ctx, grad_out)
-    return _or_empty(d_h, h), _or_empty(d_w, h), _or_empty(d_gates, h)
+    d_h, d_w, d_gates, _, d_bias, _ = _moe._ExpertsDown.backward(ctx, grad_out)
+    return _or_empty(d_h, h), _or_empty(d_w, h), _or_empty(d_gates, h), _or_empty(d_bias, h)
 
 
 @experts_down_backward.register_fake
 def _(grad_out, h, w, gates, expanded, seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, align, need_h,
-      need_w, need_gates):
+      need_w, need_gates, need_bias):
     e = h.new_empty(0)
     return (
         torch.empty_like(h) if need_h else e,
         torch.empty_like(w) if need_w else e,
         torch.empty_like(gates) if need_gates else e,
+        h.new_empty(num_experts, w.shape[1]) if need_bias else e,
     )
 
 
 def _experts_down_setup(ctx, inputs, output):
-    h, w, gates, seg_starts, counts, tile_expert, row_slot, *rest = inputs
+    h, w, gates, _bias, _slot_expert, seg_starts, counts, tile_expert, row_slot, *rest = inputs
     ctx.save_for_backward(h, w, gates, output[1], seg_starts, counts, tile_expert, row_slot)
     ctx.rest = tuple(rest)
 
 
 def _experts_down_bwd(ctx, grad_out, _expanded_grad):
-    need_h, need_w, need_gates = ctx.needs_input_grad[:3]
-    d_h, d_w, d_gates = experts_down_backward(
-        grad_out.contiguous(), *ctx.saved_tensors, *ctx.rest, need_h, need_w, need_gates
+    need_h, need_w, need_gates, need_bias = ctx.needs_input_grad[:4]
+    d_h, d_w, d_gates, d_bias = experts_down_backward(
+        grad_out.contiguous(), *ctx.saved_tensors, *ctx.rest, need_h, need_w, need_gates, need_bias
     )
-    return (d_h if need_h else None), (d_w if need_w else None), (d_gates if need_gates else None), *(None,) * 7
+    return (
+        (d_h if need_h else None), (d_w if need_w else None), (d_gates if need_gates else None),
+        (d_bias if need_bias else None), *(None,) * 8,
+    )
 
 
 experts_down.register_autograd(_experts_down_bwd, setup_context=_experts_down_setup)

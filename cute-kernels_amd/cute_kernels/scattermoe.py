@@ -299,6 +299,38 @@ def gather_rows(src: torch.Tensor, idx: torch.Tensor, coeff: torch.Tensor | None
     return out
 
 
+def _add_expert_bias(y: torch.Tensor, bias: torch.Tensor, seg: ExpertSegments, row_expert: torch.Tensor | None) -> None:
+    """y[r] += bias[expert of row r] in place: padded grouped rows (row_expert None) or token-order rows."""
+    cs = seg.c_struct()
+    with torch.cuda.device(y.device):
+        _C.check(
+            _C.lib().ck_add_expert_bias(
+                _C.ptr(y), y.size(0), y.size(1), _C.ptr(bias), _C.ptr(row_expert), None if row_expert is not None else ctypes.byref(cs),
+                _C.dtype_code(y.dtype), _C.stream(),
+            )
+        )
+
+
+def _expert_bias_grad(d_y: torch.Tensor, seg: ExpertSegments) -> torch.Tensor:
+    """[E, N] column sums of the padded grouped rows of every expert."""
+    d_bias = torch.empty(seg.num_experts, d_y.size(1), dtype=d_y.dtype, device=d_y.device)
+    cs = seg.c_struct()
+    with torch.cuda.device(d_y.device):
+        _C.check(
+            _C.lib().ck_expert_bias_grad(
+                _C.ptr(d_y), d_y.size(1), ctypes.byref(cs), _C.ptr(d_bias), _C.dtype_code(d_y.dtype), _C.stream()
+            )
+        )
+    return d_bias
+
+
+def _slot_experts(seg: ExpertSegments) -> torch.Tensor:
+    """Expert of every flat (token, slot) index, int32 [R] (the inverse of the sort)."""
+    slot_expert = torch.empty_like(seg.sorted_expert_idxs)
+    slot_expert[seg.sorted_scattered_idxs.long()] = seg.sorted_expert_idxs
+    return slot_expert
+
+
 def _check_expert_dtypes(x: torch.Tensor, *weights: torch.Tensor) -> None:
     if x.dtype not in (torch.bfloat16, torch.float16):
         raise NotImplementedError(
@@ -316,13 +348,15 @@ class _ExpertsUp(torch.autograd.Function):
     """x [T, H] (token order) -> y [max_rows, N] (padded grouped): the reference's c_fc with grouped_out=True."""
 
     @staticmethod
-    def forward(ctx, x, w, seg: ExpertSegments, k: int):
+    def forward(ctx, x, w, seg: ExpertSegments, k: int, bias=None):
         x = x.contiguous()
         w = w.contiguous()
         E, N, K = w.shape
         # pad rows are never written by the kernel; zeros keep any activation applied on top finite
         y = torch.zeros(seg.max_rows, N, dtype=x.dtype, device=x.device)
         _gemm(x, k, w, seg, _C.CK_EPI_GROUPED, y)
+        if bias is not None:
+            _add_expert_bias(y, bias.contiguous(), seg, None)
         ctx.save_for_backward(x, w)
         ctx.seg, ctx.k = seg, k
         return y
@@ -333,7 +367,9 @@ class _ExpertsUp(torch.autograd.Function):
         seg, k = ctx.seg, ctx.k
         T, K = x.shape
         d_y = d_y.contiguous()
-        d_x = d_w = None
+        d_x = d_w = d_bias = None
+        if len(ctx.needs_input_grad) > 4 and ctx.needs_input_grad[4]:
+            d_bias = _expert_bias_grad(d_y, seg)
         if ctx.needs_input_grad[1]:
             _, d_y_t = _group_rows(d_y, None, 0, seg, False, True)
             _, x_t = _group_rows(x, None, k, seg, False, True)
@@ -344,14 +380,14 @@ class _ExpertsUp(torch.autograd.Function):
             d_expanded = torch.empty(T * k, K, dtype=x.dtype, device=x.device)
             _gemm(d_y, 0, w_t, seg, _C.CK_EPI_SCATTER, d_expanded)
             d_x = d_expanded if k == 1 else _combine(d_expanded, None, T, k, K)[0]
-        return d_x, d_w, None, None
+        return d_x, d_w, None, None, d_bias
 
 
 class _ExpertsDown(torch.autograd.Function):
     """h [max_rows, I] (padded grouped), gates [T, k] -> out [T, H]: the reference's c_proj with grouped_in=True."""
 
     @staticmethod
-    def forward(ctx, h, w, gates, seg: ExpertSegments):
+    def forward(ctx, h, w, gates, seg: ExpertSegments, bias=None, slot_expert=None):
         h = h.contiguous()
         w = w.contiguous()
         gates = gates.contiguous()
@@ -359,6 +395,8 @@ class _ExpertsDown(torch.autograd.Function):
         E, N, K = w.shape
         expanded = torch.empty(T * k, N, dtype=h.dtype, device=h.device)
         _gemm(h, 0, w, seg, _C.CK_EPI_SCATTER, expanded)
+        if bias is not None:  # before the gate multiply, as torch_implementation.py:160-163
+            _add_expert_bias(expanded, bias.contiguous(), seg, slot_expert if slot_expert is not None else _slot_experts(seg))
         out, _ = _combine(expanded, gates, T, k, N)
         ctx.save_for_backward(h, w, gates, expanded)
         ctx.seg = seg
@@ -371,11 +409,13 @@ class _ExpertsDown(torch.autograd.Function):
         T, k = gates.shape
         E, N, K = w.shape
         grad_out = grad_out.contiguous()
-        d_h = d_w = d_gates = None
+        d_h = d_w = d_gates = d_bias = None
         if ctx.needs_input_grad[2]:
             _, d_gates = _combine(expanded, None, T, k, N, grad_out=grad_out, want_out=False, want_d_gates=True)
         need_w = ctx.needs_input_grad[1]
         d_y, d_y_t = _group_rows(grad_out, gates, k, seg, True, need_w)
+        if len(ctx.needs_input_grad) > 4 and ctx.needs_input_grad[4]:
+            d_bias = _expert_bias_grad(d_y, seg)  # d_y: the gate-scaled grad_out rows in padded grouped order
         if need_w:
             _, h_t = _group_rows(h, None, 0, seg, False, True)
             d_w = torch.empty_like(w)
@@ -384,28 +424,36 @@ class _ExpertsDown(torch.autograd.Function):
             w_t = _transpose_weights(w)  # [E, K, N]
             d_h = torch.zeros(seg.max_rows, K, dtype=h.dtype, device=h.device)
             _gemm(d_y, 0, w_t, seg, _C.CK_EPI_GROUPED, d_h)
-        return d_h, d_w, d_gates, None
+        return d_h, d_w, d_gates, None, d_bias, None
 
 
-def experts_up(x: torch.Tensor, weight: torch.Tensor, seg: ExpertSegments, k: int) -> torch.Tensor:
+def experts_up(
+    x: torch.Tensor, weight: torch.Tensor, seg: ExpertSegments, k: int, bias: torch.Tensor | None = None
+) -> torch.Tensor:
+    """x [T, H] -> c_fc output in padded grouped order [max_rows, N] (+ bias[e] on expert e's rows)."""
     _check_expert_dtypes(x, weight)
     if torch.compiler.is_compiling():
         return _ops.experts_up(
-            x, weight, seg.seg_starts, seg.counts, seg.tile_expert, seg.row_slot, seg.max_rows, seg.num_experts, seg.align, k
+            x, weight, bias, seg.seg_starts, seg.counts, seg.tile_expert, seg.row_slot, seg.max_rows, seg.num_experts,
+            seg.align, k,
         )
-    _C.require_gpu(x, weight)
-    return _ExpertsUp.apply(x, weight, seg, k)
+    _C.require_gpu(x, weight, bias)
+    return _ExpertsUp.apply(x, weight, seg, k, bias)
 
 
-def experts_down(h: torch.Tensor, weight: torch.Tensor, gates: torch.Tensor, seg: ExpertSegments) -> torch.Tensor:
+def experts_down(
+    h: torch.Tensor, weight: torch.Tensor, gates: torch.Tensor, seg: ExpertSegments, bias: torch.Tensor | None = None
+) -> torch.Tensor:
+    """h [max_rows, I] (padded grouped) -> sum_k gates * (c_proj output + bias[e]) in token order [T, N]."""
     _check_expert_dtypes(h, weight)
     if torch.compiler.is_compiling():
+        slot_expert = _slot_experts(seg) if bias is not None else None
         return _ops.experts_down(
-            h, weight, gates.to(h.dtype), seg.seg_starts, seg.counts, seg.tile_expert, seg.row_slot, seg.max_rows,
-            seg.num_experts, seg.align,
+            h, weight, gates.to(h.dtype), bias, slot_expert, seg.seg_starts, seg.counts, seg.tile_expert, seg.row_slot,
+            seg.max_rows, seg.num_experts, seg.align,
         )[0]
-    _C.require_gpu(h, weight, gates)
-    return _ExpertsDown.apply(h, weight, gates.to(h.dtype), seg)
+    _C.require_gpu(h, weight, gates, bias)
+    return _ExpertsDown.apply(h, weight, gates.to(h.dtype), seg, bias)
 
 
 # ---------------------------------------------------------------------------------------------------------------

@@ -221,6 +221,19 @@ int ck_rmsnorm_bwd(const void* x, const void* weight, const void* d_out, const f
                    int32_t H, void* d_x, float* d_weight_partial, float* d_weight, int32_t dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------------------------------
+ * Expert biases
+ * Replaces: the bias operand of F.linear in Experts_Torch.forward -- cute_kernels/kernels/scattermoe/
+ *           torch_implementation.py:20-22,42 (one bias row [out] per expert; the reference's Triton path drops it,
+ *           triton_implementation/__init__.py:26-36).
+ * ck_add_expert_bias: y[r, :] += bias[e(r), :], y [rows, N], bias [E, N]. Padded grouped rows: pass seg, e(r) is the
+ *   expert of the row's tile and pad rows are left alone. Token-order rows: pass row_expert [rows] (negative = skip).
+ * ck_expert_bias_grad: d_bias[e, :] = sum of d_y over expert e's rows of the padded grouped layout (fp32 sums).
+ * ------------------------------------------------------------------------------------------------------------- */
+int ck_add_expert_bias(void* y, int64_t rows, int32_t N, const void* bias, const int32_t* row_expert,
+                       const ck_segments* seg, int32_t dtype, void* stream);
+int ck_expert_bias_grad(const void* d_y, int32_t N, const ck_segments* seg, void* d_bias, int32_t dtype, void* stream);
+
+/* ---------------------------------------------------------------------------------------------------------------
  * Residual add fused with RMSNorm (the step in front of an MoE block in a transformer layer)
  * Replaces: fused_residual_add_rmsnorm_forward_triton / _backward_triton -- cute_kernels/kernels/
  *           fused_residual_add_rmsnorm/triton_implementation/forward.py:14-104, backward.py:14-149; semantics of

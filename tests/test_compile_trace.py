@@ -34,6 +34,11 @@ def test_moe_layer_traces(act, is_glu):
     _traces(lambda a: moe(a)[0], torch.randn(16, 64, dtype=torch.bfloat16, requires_grad=True))
 
 
+def test_moe_layer_with_biases_traces():
+    moe = ck.MoE(4, 2, 64, 32, torch.nn.GLU(), True, True, 0.02).to(torch.bfloat16)
+    _traces(lambda a: moe(a)[0], torch.randn(16, 64, dtype=torch.bfloat16, requires_grad=True))
+
+
 def test_traced_max_rows_formula_matches_the_library():
     lib = _C.lib()
     for R in (0, 1, 255, 256, 32768, 524288, 1000003):

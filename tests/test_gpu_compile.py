@@ -10,6 +10,14 @@ import cute_kernels as ck
 pytestmark = pytest.mark.gpu
 
 
+@pytest.fixture(autouse=True)
+def _fresh_dynamo():
+    """Every case compiles a new module instance of the same code objects: start from an empty cache so that dynamo's
+    per-function recompile limit is not what a later case trips over."""
+    torch._dynamo.reset()
+    yield
+
+
 def _compile(fn):
     return torch.compile(fn, fullgraph=True, backend="aot_eager")
 
@@ -49,10 +57,15 @@ def test_swiglu_and_norms_compiled(device, dtype):
                 assert torch.equal(a.grad, b.grad), name
 
 
+@pytest.mark.parametrize("add_bias", [False, True])
 @pytest.mark.parametrize("act,is_glu", [(ck.swiglu_packed_cute, True), (torch.nn.GLU(), True), (torch.nn.GELU("tanh"), False)])
-def test_moe_layer_compiled(device, act, is_glu):
+def test_moe_layer_compiled(device, act, is_glu, add_bias):
     torch.manual_seed(1)
-    moe = ck.MoE(8, 2, 128, 256, act, is_glu, False, 0.02).to(torch.bfloat16).to(device)
+    moe = ck.MoE(8, 2, 128, 256, act, is_glu, add_bias, 0.02).to(torch.bfloat16).to(device)
+    if add_bias:
+        with torch.no_grad():
+            moe.c_fc.bias.normal_(0, 0.1)
+            moe.c_proj.bias.normal_(0, 0.1)
     x = torch.randn(512, 128, dtype=torch.bfloat16, device=device)
     xe, xc = x.clone().requires_grad_(), x.clone().requires_grad_()
     y, logits = moe(xe)

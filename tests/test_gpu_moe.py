@@ -208,13 +208,17 @@ def _acts(name):
     return nn.GELU(approximate="tanh"), nn.GELU(approximate="tanh"), False
 
 
-def _run_layer_case(device, dtype, T, E, k, H, I, act_name, x_shape=None, seed=42):
+def _run_layer_case(device, dtype, T, E, k, H, I, act_name, x_shape=None, seed=42, add_bias=False):
     torch.manual_seed(seed)
     act_gpu, act_cpu, is_glu = _acts(act_name)
-    moe = cute_kernels.MoE(E, k, H, I, act_gpu, is_glu, False, 0.02).to(dtype)
-    oracle = _OracleWithSelection(E, k, H, I, act_cpu, is_glu, False, 0.02).to(dtype)
+    moe = cute_kernels.MoE(E, k, H, I, act_gpu, is_glu, add_bias, 0.02).to(dtype)
+    if add_bias:  # the constructor zeroes biases (torch_implementation.py:56-60); give them values
+        with torch.no_grad():
+            moe.c_fc.bias.normal_(0, 0.1)
+            moe.c_proj.bias.normal_(0, 0.1)
+    oracle = _OracleWithSelection(E, k, H, I, act_cpu, is_glu, add_bias, 0.02).to(dtype)
     oracle.load_state_dict(moe.state_dict())  # same state_dict keys as the reference (scattermoe_test.py:83-94)
-    truth = _OracleWithSelection(E, k, H, I, act_cpu, is_glu, False, 0.02).float()
+    truth = _OracleWithSelection(E, k, H, I, act_cpu, is_glu, add_bias, 0.02).float()
     truth.load_state_dict({n: v.float() for n, v in moe.state_dict().items()})
     moe = moe.to(device)
 
@@ -252,6 +256,12 @@ def _run_layer_case(device, dtype, T, E, k, H, I, act_name, x_shape=None, seed=4
             getattr(moe, name).weight.grad, getattr(oracle, name).weight.grad, getattr(truth, name).weight.grad,
             f"{name}.weight.grad", atol=3e-2,
         )
+    if add_bias:
+        for name in ["c_fc", "c_proj"]:
+            _close_via_truth(
+                getattr(moe, name).bias.grad, getattr(oracle, name).bias.grad, getattr(truth, name).bias.grad,
+                f"{name}.bias.grad", atol=3e-2,
+            )
     # d_gates is rounded to the activation dtype by the reference's accelerated path (ops.py:214), by its torch path and
     # by ours; the softmax backward then subtracts nearly equal numbers, so that one rounding -- not the kernels -- is
     # the error floor of gate.weight.grad: about eps * max|d_gates| * max|x| per element.
@@ -284,10 +294,16 @@ def test_moe_layer_3d_input_top1_and_large_tiles(device):
     _run_layer_case(device, torch.bfloat16, 9000, 4, 2, 128, 136, "swiglu")
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("act", ["swiglu", "glu", "gelu"])
+@pytest.mark.parametrize("T,E,k,H,I", [(257, 8, 2, 128, 256), (33, 4, 4, 64, 72), (700, 64, 8, 128, 136)])
+def test_moe_layer_with_expert_biases(device, dtype, act, T, E, k, H, I):
+    # add_bias=True: the reference's torch path applies one bias row per expert (torch_implementation.py:20-22,42); its
+    # Triton path drops them, so the reference's own test only runs add_bias=False (scattermoe_test.py:62-77)
+    _run_layer_case(device, dtype, T, E, k, H, I, act, add_bias=True)
+
+
 def test_moe_layer_rejects_unsupported(device):
-    moe = cute_kernels.MoE(4, 2, 64, 72, cute_kernels.swiglu_packed_cute, True, True, 0.02).to(torch.bfloat16).to(device)
-    with pytest.raises(NotImplementedError, match="bias"):
-        moe(torch.randn(5, 64, dtype=torch.bfloat16, device=device))
     moe = cute_kernels.MoE(4, 2, 64, 72, cute_kernels.swiglu_packed_cute, True, False, 0.02).to(device)
     with pytest.raises(NotImplementedError, match="bf16 / fp16"):
         moe(torch.randn(5, 64, device=device))
