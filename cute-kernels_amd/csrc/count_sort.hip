@@ -229,11 +229,16 @@ struct SortPlan {
   int64_t seg_len; // multiple of kWave
 };
 
+inline int64_t sort_ids_per_segment() {  // measurement knob (more, shorter segments lengthen the last block's scan: 1024 is best)
+  const char* env = getenv("CK_SORT_SEG");
+  return env ? atol(env) : 1024;
+}
+
 SortPlan make_sort_plan(int64_t R, int E) {
   int64_t cap = kSortTableWords / (E > 0 ? E : 1);
   cap = (cap / kWavesPerBlock) * kWavesPerBlock;
   if (cap < kWavesPerBlock) cap = kWavesPerBlock;
-  int64_t want = ceil_div(R > 0 ? R : 1, 1024);
+  int64_t want = ceil_div(R > 0 ? R : 1, sort_ids_per_segment());
   want = round_up(want, kWavesPerBlock);
   SortPlan p;
   p.segments = (int)(want < cap ? want : cap);

@@ -106,7 +106,7 @@ __device__ inline void store_tile_transposed(const T (*tile)[kTileStride], T* __
       Pack16<T> p;
 #pragma unroll
       for (int i = 0; i < 8; ++i) p.e[i] = tile[rc + i][c];
-      store16(dst + (c0 + c) * ld + r0 + rc, p.v);
+      store16_nt(dst + (c0 + c) * ld + r0 + rc, p.v);  // multi-GB outputs: written once, read by a later kernel
     }
   }
 }
@@ -148,7 +148,7 @@ __global__ __launch_bounds__(kBlock) void group_rows_padded_kernel(
         v = load16(src + p * H + h);
       }
     }
-    if (grouped != nullptr && h < H) store16(grouped + p * H + h, v);
+    if (grouped != nullptr && h < H) store16_nt(grouped + p * H + h, v);
     if (grouped_t != nullptr) fill_tile_chunk(tile, r, cc, v);
   }
   if (grouped_t == nullptr) return;
