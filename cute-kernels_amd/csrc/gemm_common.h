@@ -44,7 +44,10 @@ struct GemmParams {
 // multiple of 64, modes kGrouped, kScatter, kSwiglu, kDw. The caller fills `prm` for these tile dimensions (n_tiles,
 // m_tiles) and sizes the grid accordingly.
 constexpr int kLineBM = 256, kLineK = 64;
-int launch_line(const GemmParams& prm, int mode, int bn, int dtype, unsigned blocks, hipStream_t stream, const char* name);
+// bt: the weight operand is [E, contraction, columns] (contraction-strided) instead of [E, columns, contraction];
+// grouped and scatter epilogues only, prm.ldw = its row length.
+int launch_line(const GemmParams& prm, int mode, int bn, bool bt, int dtype, unsigned blocks, hipStream_t stream,
+                const char* name);
 
 namespace {
 

@@ -837,7 +837,7 @@ extern "C" int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* 
     prm.n_tiles = (int)ceil_div(out_cols, swiglu ? bn / 2 : bn);
     const int64_t line_blocks = m_tiles * prm.n_tiles;
     CK_REQUIRE(line_blocks < (int64_t)0x7fffffff, "%s: grid too large", name);
-    return launch_line(prm, epilogue, bn, dtype, (unsigned)line_blocks, s, name);
+    return launch_line(prm, epilogue, bn, false, dtype, (unsigned)line_blocks, s, name);
   }
   const int bn = seg->align;  // square tiles
   prm.n_tiles = n_tiles_for(bn);
@@ -855,6 +855,40 @@ extern "C" int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* 
   });
 #undef CK_GEMM_MODE
   return CK_OK;
+}
+
+extern "C" int ck_grouped_gemm_nn(const void* a, const void* w, int32_t N, int32_t K, const ck_segments* seg,
+                                  int32_t epilogue, void* y, int32_t dtype, void* stream) {
+  const char* name = "ck_grouped_gemm_nn";
+  if (int rc = check_segments(seg, name)) return rc;
+  CK_REQUIRE(seg->align == kLineBM, "%s: needs 256-row tiles (sort with align = 256)", name);
+  CK_REQUIRE(N >= 8 && N % 8 == 0, "%s: N=%d must be a positive multiple of 8", name, N);
+  CK_REQUIRE(K >= kLineK && K % kLineK == 0, "%s: K=%d must be a positive multiple of %d", name, K, kLineK);
+  CK_REQUIRE(epilogue == CK_EPI_GROUPED || epilogue == CK_EPI_SCATTER, "%s: epilogue %d is not grouped or scatter", name,
+             epilogue);
+  if (seg->max_rows == 0) return CK_OK;
+  CK_REQUIRE(a && w && y && aligned16(a) && aligned16(w), "%s: NULL or misaligned pointer", name);
+  CK_REQUIRE((int64_t)N * K * 2 < ((int64_t)1 << 32) && seg->max_rows * (int64_t)K * 2 < ((int64_t)1 << 32),
+             "%s: one expert's weight matrix and the grouped input must each stay below 4 GiB", name);
+  GemmParams prm = {};
+  prm.a = a;
+  prm.w = w;
+  prm.lda = K;
+  prm.ldw = N;  // rows of w are contraction indices, N columns each
+  prm.w_expert_stride = (int64_t)N * K;
+  prm.N = N;
+  prm.K = K;
+  prm.align = seg->align;
+  prm.num_experts = seg->num_experts;
+  prm.seg_starts = seg->seg_starts;
+  prm.counts = seg->counts;
+  prm.tile_expert = seg->tile_expert;
+  prm.row_slot = seg->row_slot;
+  prm.y = y;
+  prm.n_tiles = (int)ceil_div(N, 256);
+  const int64_t blocks = (seg->max_rows / seg->align) * prm.n_tiles;
+  CK_REQUIRE(blocks < (int64_t)0x7fffffff, "%s: grid too large", name);
+  return launch_line(prm, epilogue, 256, true, dtype, (unsigned)blocks, static_cast<hipStream_t>(stream), name);
 }
 
 extern "C" int ck_grouped_gemm_dw(const void* a_t, const void* b_t, int64_t ld_t, int32_t M, int32_t N,
@@ -893,7 +927,7 @@ extern "C" int ck_grouped_gemm_dw(const void* a_t, const void* b_t, int64_t ld_t
     prm.n_tiles = (int)ceil_div(N, bn);
     const int64_t line_blocks = (int64_t)prm.m_tiles * prm.n_tiles * seg->num_experts;
     CK_REQUIRE(line_blocks < (int64_t)0x7fffffff, "%s: grid too large", name);
-    return launch_line(prm, kDw, bn, dtype, (unsigned)line_blocks, s, name);
+    return launch_line(prm, kDw, bn, false, dtype, (unsigned)line_blocks, s, name);
   }
   const int bt = big ? 256 : 128;
   prm.m_tiles = (int)ceil_div(M, bt);

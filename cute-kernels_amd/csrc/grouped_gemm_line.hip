@@ -52,7 +52,10 @@ struct Tile {
   static_assert(kLoadsPerStep <= 2 * NI, "every load of a step has an MFMA of the last slice to hide behind");
 };
 
-template <typename T, int MODE, int BN>
+// BT ("B as stored by its owner"): the weight operand is [contraction, columns] row-major, i.e. contraction-strided --
+// the input-gradient GEMMs read W[e] [out, in] this way instead of a transposed copy. Its stage holds 64 contraction rows
+// of BN columns, and fragments come out of LDS through ds_read_b64_tr_b16 (see read_b).
+template <typename T, int MODE, int BN, bool BT>
 __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams prm) {
   typedef Tile<BN> TL;
   constexpr int WN = TL::WN, NI = TL::NI, B_LD = TL::B_LD, kLoadsPerStep = TL::kLoadsPerStep, kStageBytes = TL::kStageBytes;
@@ -134,20 +137,35 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
     }
     a_off[t] = (uint32_t)((row * prm.lda + k_begin) * 2 + c * 16);
   }
+  // BT: 32-byte window q of contraction row n sits at window position swap02(q) ^ (n & 3) of the row (swap02 exchanges
+  // bits 0 and 2 of the window index): the 4 rows x 32 bytes one 16-lane group of a transposing read touches fill one
+  // 128-byte block, and the neighbouring group (next 16 columns) falls into the other half of the banks.
+  constexpr int kBtRowBytes = BN * 2, kBtWindows = kBtRowBytes / 32;
+  auto swap02 = [](int w) { return (w & ~5) | ((w & 1) << 2) | ((w >> 2) & 1); };
 #pragma unroll
   for (int t = 0; t < B_LD; ++t) {
-    const int j = (wave * B_LD + t) * 8 + (lane >> 3);
-    const int c = (lane & 7) ^ swz128(j);
-    int64_t n;
-    if constexpr (MODE == kSwiglu) {  // a wave's WN tile columns: WN/2 up columns, then the gate columns of the same outputs
-      const int half = (j % WN) / (WN / 2);
-      const int within = (j / WN) * (WN / 2) + (j % (WN / 2));
-      n = (int64_t)half * prm.I + min((int64_t)nt * (BN / 2) + within, (int64_t)prm.I - 1);
+    if constexpr (BT) {
+      const int pos = (wave * B_LD + t) * 1024 + lane * 16;  // byte position of this lane's slot in the B stage
+      const int n = pos / kBtRowBytes, slot16 = (pos % kBtRowBytes) / 16;
+      const int q = swap02((slot16 >> 1) ^ (n & 3));           // the window that belongs at this position
+      int64_t col = (int64_t)nt * BN + (2 * q + (slot16 & 1)) * 8;
+      if (col >= prm.N) col = (int64_t)nt * BN;                // ragged edge: re-read a valid chunk, never stored
+      b_off[t] = (uint32_t)(((int64_t)n * prm.ldw + col) * 2);
     } else {
-      n = min((int64_t)nt * BN + j, (int64_t)prm.N - 1);
+      const int j = (wave * B_LD + t) * 8 + (lane >> 3);
+      const int c = (lane & 7) ^ swz128(j);
+      int64_t n;
+      if constexpr (MODE == kSwiglu) {  // a wave's WN tile columns: WN/2 up columns, then the gate columns of the same outputs
+        const int half = (j % WN) / (WN / 2);
+        const int within = (j / WN) * (WN / 2) + (j % (WN / 2));
+        n = (int64_t)half * prm.I + min((int64_t)nt * (BN / 2) + within, (int64_t)prm.I - 1);
+      } else {
+        n = min((int64_t)nt * BN + j, (int64_t)prm.N - 1);
+      }
+      b_off[t] = (uint32_t)((n * prm.ldw + k_begin) * 2 + c * 16);
     }
-    b_off[t] = (uint32_t)((n * prm.ldw + k_begin) * 2 + c * 16);
   }
+  static_assert(!BT || kBtWindows % 8 == 0 || kBtWindows == 24, "window swizzle works on groups of 8 windows");
   const int nk = k_len / BK;
 
   auto dma16 = [&](const char* src, uint32_t lds_addr) {
@@ -158,9 +176,10 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
   const uint32_t wave_b = __builtin_amdgcn_readfirstlane(lds_base + BM * kRowBytes + wave * B_LD * 1024);
   auto issue_one = [&](int step, int g) {
     const int64_t kb = (int64_t)step * kRowBytes;
+    const int64_t kb_b = BT ? (int64_t)step * BK * prm.ldw * 2 : kb;  // BT: 64 contraction rows further down
     const uint32_t st = (uint32_t)((step & (NSTAGE - 1)) * kStageBytes);
     if (g < A_LD) dma16(a_base + kb + a_off[g], wave_a + st + g * 1024);
-    else dma16(b_base + kb + b_off[g - A_LD], wave_b + st + (g - A_LD) * 1024);
+    else dma16(b_base + kb_b + b_off[g - A_LD], wave_b + st + (g - A_LD) * 1024);
   };
   auto issue = [&](int step) {
 #pragma unroll
@@ -179,8 +198,32 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
   auto read_a = [&](int stage, int sl, int i) {
     fa[i] = *reinterpret_cast<const frag_t*>(lds_c + stage * kStageBytes + slice_off[sl] + fa_row + i * 32 * kRowBytes);
   };
+  // BT: lane l = 16 g + i of a transposing read points at 4 consecutive columns (4 (i % 4) ..) of contraction row i / 4
+  // of a 4-row x 16-column patch and receives the 4 rows of column i; two reads (rows +0..3, +4..7) make the 8 contraction
+  // values of column 16 (g % 2) + i for k-half g / 2 -- the MFMA's B layout.
+  typedef __attribute__((__vector_size__(4 * sizeof(short)))) short tr16x4;
+  int bt_off[NI];
+  if constexpr (BT) {
+    const int g = lane >> 4, i = lane & 15, n_low = i >> 2;
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int q = (wn * WN + j * 32) / 16 + (g & 1);
+      bt_off[j] = BM * kRowBytes + (8 * (g >> 1) + n_low) * kBtRowBytes + (swap02(q) ^ n_low) * 32 + 8 * (i & 3);
+    }
+  }
   auto read_b = [&](int stage, int sl, int j) {
-    fb[j] = *reinterpret_cast<const frag_t*>(lds_c + stage * kStageBytes + slice_off[sl] + fb_row + j * 32 * kRowBytes);
+    if constexpr (BT) {
+      const char* p = lds_c + stage * kStageBytes + bt_off[j] + 16 * sl * kBtRowBytes;
+      union {
+        tr16x4 h[2];
+        frag_t f;
+      } u;
+      u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr16x4 __attribute__((address_space(3)))*)(p));
+      u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr16x4 __attribute__((address_space(3)))*)(p + 4 * kBtRowBytes));
+      fb[j] = u.f;
+    } else {
+      fb[j] = *reinterpret_cast<const frag_t*>(lds_c + stage * kStageBytes + slice_off[sl] + fb_row + j * 32 * kRowBytes);
+    }
   };
   auto mfma = [&](int i, int j) {
     if constexpr ((CK_ABLATE & 64) != 0) {
@@ -406,9 +449,9 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
   }
 }
 
-template <typename T, int MODE, int BN>
+template <typename T, int MODE, int BN, bool BT>
 int launch_mode(const GemmParams& prm, unsigned blocks, hipStream_t s, const char* name) {
-  auto kernel = grouped_gemm_line_kernel<T, MODE, BN>;
+  auto kernel = grouped_gemm_line_kernel<T, MODE, BN, BT>;
   constexpr size_t kLds = Tile<BN>::kLdsBytes;
   static bool attr_set = false;  // per instantiation; the attribute is idempotent, a race only repeats the call
   if (!attr_set) {
@@ -426,12 +469,21 @@ int launch_mode(const GemmParams& prm, unsigned blocks, hipStream_t s, const cha
 }
 
 template <typename T, int BN>
-int launch_bn(const GemmParams& prm, int mode, unsigned blocks, hipStream_t stream, const char* name) {
+int launch_bn(const GemmParams& prm, int mode, bool bt, unsigned blocks, hipStream_t stream, const char* name) {
+  if (bt) {  // the input-gradient GEMMs: grouped or scatter epilogue, 256-wide tiles (the 384-wide tile has no registers
+             // left for the transposing reads' addresses)
+    if constexpr (BN == 256) {
+      if (mode == kGrouped) return launch_mode<T, kGrouped, BN, true>(prm, blocks, stream, name);
+      if (mode == kScatter) return launch_mode<T, kScatter, BN, true>(prm, blocks, stream, name);
+    }
+    set_error("%s: the contraction-strided weight operand goes with 256-wide tiles and the grouped / scatter epilogues", name);
+    return CK_ERR_ARG;
+  }
   switch (mode) {
-    case kGrouped: return launch_mode<T, kGrouped, BN>(prm, blocks, stream, name);
-    case kScatter: return launch_mode<T, kScatter, BN>(prm, blocks, stream, name);
-    case kSwiglu: return launch_mode<T, kSwiglu, BN>(prm, blocks, stream, name);
-    case kDw: return launch_mode<T, kDw, BN>(prm, blocks, stream, name);
+    case kGrouped: return launch_mode<T, kGrouped, BN, false>(prm, blocks, stream, name);
+    case kScatter: return launch_mode<T, kScatter, BN, false>(prm, blocks, stream, name);
+    case kSwiglu: return launch_mode<T, kSwiglu, BN, false>(prm, blocks, stream, name);
+    case kDw: return launch_mode<T, kDw, BN, false>(prm, blocks, stream, name);
     default: break;
   }
   set_error("%s: the 128-byte-row kernel has no epilogue %d", name, mode);
@@ -440,10 +492,11 @@ int launch_bn(const GemmParams& prm, int mode, unsigned blocks, hipStream_t stre
 
 }  // namespace
 
-int launch_line(const GemmParams& prm, int mode, int bn, int dtype, unsigned blocks, hipStream_t stream, const char* name) {
+int launch_line(const GemmParams& prm, int mode, int bn, bool bt, int dtype, unsigned blocks, hipStream_t stream,
+                const char* name) {
   CK_DISPATCH_HALF(dtype, name, {
-    if (bn == 384) return launch_bn<scalar_t, 384>(prm, mode, blocks, stream, name);
-    return launch_bn<scalar_t, 256>(prm, mode, blocks, stream, name);
+    if (bn == 384) return launch_bn<scalar_t, 384>(prm, mode, bt, blocks, stream, name);
+    return launch_bn<scalar_t, 256>(prm, mode, bt, blocks, stream, name);
   });
   return CK_ERR_ARG;
 }

@@ -228,6 +228,37 @@ def _gemm(a, gather_div, w, seg: ExpertSegments, epilogue, y, y_t=None, aux=None
         launch_timer.time(_EPILOGUE_NAMES[epilogue], (N, K), launch)
 
 
+def _gemm_dx(d_y, w, seg: ExpertSegments, epilogue, out):
+    """out = d_y @ w[e] per expert, w [E, out_features, in_features] as the forward stores it: the input-gradient GEMM.
+    Reads w contraction-strided where the kernel for that exists (256-row tiles, out_features % 64 == 0); otherwise
+    through a transposed copy."""
+    E, n_out, n_in = w.shape
+    if seg.align == 256 and n_out % 64 == 0 and _nn_enabled():
+        cs = seg.c_struct()
+
+        def launch():
+            with torch.cuda.device(w.device):
+                _C.check(
+                    _C.lib().ck_grouped_gemm_nn(
+                        _C.ptr(d_y), _C.ptr(w), n_in, n_out, ctypes.byref(cs), epilogue, _C.ptr(out), _C.dtype_code(w.dtype),
+                        _C.stream(),
+                    )
+                )
+
+        if launch_timer is None:
+            launch()
+        else:
+            launch_timer.time(_EPILOGUE_NAMES[epilogue], (n_in, n_out), launch)
+        return
+    _gemm(d_y, 0, _transpose_weights(w), seg, epilogue, out)
+
+
+def _nn_enabled() -> bool:
+    import os
+
+    return os.environ.get("CK_GEMM_NN", "1") != "0"  # measurement knob: 0 = always go through the transposed copy
+
+
 def _gemm_dw(a_t, b_t, seg: ExpertSegments, dw):
     E, M, N = dw.shape
     cs = seg.c_struct()
@@ -376,9 +407,8 @@ class _ExpertsUp(torch.autograd.Function):
             d_w = torch.empty_like(w)
             _gemm_dw(d_y_t, x_t, seg, d_w)
         if ctx.needs_input_grad[0]:
-            w_t = _transpose_weights(w)  # [E, K, N]
             d_expanded = torch.empty(T * k, K, dtype=x.dtype, device=x.device)
-            _gemm(d_y, 0, w_t, seg, _C.CK_EPI_SCATTER, d_expanded)
+            _gemm_dx(d_y, w, seg, _C.CK_EPI_SCATTER, d_expanded)
             d_x = d_expanded if k == 1 else _combine(d_expanded, None, T, k, K)[0]
         return d_x, d_w, None, None, d_bias
 
@@ -421,9 +451,8 @@ class _ExpertsDown(torch.autograd.Function):
             d_w = torch.empty_like(w)
             _gemm_dw(d_y_t, h_t, seg, d_w)
         if ctx.needs_input_grad[0]:
-            w_t = _transpose_weights(w)  # [E, K, N]
             d_h = torch.zeros(seg.max_rows, K, dtype=h.dtype, device=h.device)
-            _gemm(d_y, 0, w_t, seg, _C.CK_EPI_GROUPED, d_h)
+            _gemm_dx(d_y, w, seg, _C.CK_EPI_GROUPED, d_h)
         return d_h, d_w, d_gates, None, d_bias, None
 
 
@@ -517,10 +546,9 @@ class _SwigluExperts(torch.autograd.Function):
             # d_act = d_y @ w_proj with the leanest epilogue, then one streaming pass for the SwiGLU backward and the
             # transpose d_w_fc needs. (The GEMM can also do this in its epilogue, CK_EPI_SWIGLU_BWD, but with one
             # workgroup per CU the epilogue is time the MFMA units idle, while the streaming pass runs at HBM speed.)
-            w_proj_t = _transpose_weights(w_proj)  # [E, I, H]
             d_act = torch.empty(seg.max_rows, I, dtype=dt, device=dev)
-            _gemm(d_y, 0, w_proj_t, seg, _C.CK_EPI_GROUPED, d_act)
-            del w_proj_t, d_y
+            _gemm_dx(d_y, w_proj, seg, _C.CK_EPI_GROUPED, d_act)
+            del d_y
             d_pre = torch.empty(seg.max_rows, two_i, dtype=dt, device=dev)
             d_pre_t = torch.empty(two_i, seg.ld_t, dtype=dt, device=dev) if need_fc else None
             with torch.cuda.device(dev):
@@ -537,9 +565,8 @@ class _SwigluExperts(torch.autograd.Function):
                 _gemm_dw(d_pre_t, x_t, seg, d_w_fc)
                 del d_pre_t, x_t
             if need_x:
-                w_fc_t = _transpose_weights(w_fc)  # [E, H, 2I]
                 d_expanded = torch.empty(T * k, H, dtype=dt, device=dev)
-                _gemm(d_pre, 0, w_fc_t, seg, _C.CK_EPI_SCATTER, d_expanded)
+                _gemm_dx(d_pre, w_fc, seg, _C.CK_EPI_SCATTER, d_expanded)
                 d_x = d_expanded if k == 1 else _combine(d_expanded, None, T, k, H)[0]
         return d_x, d_w_fc, d_w_proj, d_gates, None
 

@@ -166,6 +166,16 @@ typedef struct ck_segments {
 int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* w, int32_t N, int32_t K,
                     const ck_segments* seg, int32_t epilogue, void* y, void* y_t, int64_t ld_t, void* aux,
                     const void* aux_in, int32_t dtype, void* stream);
+/* Input-gradient form of the grouped GEMM: y[p, :] = a[p, :] @ w[e(p)] with w [E, K, N] row-major, i.e. the weight
+ * exactly as the forward pass stores it ([E, out, in] = [E, K, N] here: K = the forward's out, N = its in), read
+ * contraction-strided instead of through a transposed copy.
+ * Replaces: the dX calls of scatter2scatter on the permuted weight view -- cute_kernels/kernels/scattermoe/
+ *           triton_implementation/ops.py:258-292 (expert_weights.permute(0, 2, 1) there; the Triton kernel takes strides).
+ * a [max_rows, K] padded grouped rows; epilogue CK_EPI_GROUPED (y [max_rows, N]) or CK_EPI_SCATTER (y [R, N]).
+ * Needs seg->align == 256, K % 64 == 0, N % 8 == 0. */
+int ck_grouped_gemm_nn(const void* a, const void* w, int32_t N, int32_t K, const ck_segments* seg, int32_t epilogue,
+                       void* y, int32_t dtype, void* stream);
+
 /* dW[e] = A_t[:, seg_e] * B_t[:, seg_e]^T : A_t [M, ld_t], B_t [N, ld_t] are transposed padded-grouped operands with
  * zeros in pad rows; dw [E, M, N]. Experts with no rows get exact zeros (ops.py:252, kernels.py:181). */
 int ck_grouped_gemm_dw(const void* a_t, const void* b_t, int64_t ld_t, int32_t M, int32_t N, const ck_segments* seg,

@@ -94,6 +94,34 @@ def test_grouped_gemm_grouped_in_scatter_out(device, dtype, align, K, N, gemm_ti
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("epilogue", ["grouped", "scatter"])
+@pytest.mark.parametrize("n_out,n_in", [(64, 128), (192, 264), (576, 840), (128, 8)])
+def test_grouped_gemm_input_gradient_form(device, dtype, epilogue, n_out, n_in):
+    """out = d_y @ w[e] with w [E, n_out, n_in] as the forward stores it (read contraction-strided) equals the same
+    product through an explicitly transposed copy, bit for bit (same tiles, same accumulation order), and the fp64 value
+    within the 16-bit tolerance."""
+    T, k, E = 300, 2, 5
+    g, seg = _make_case(device, dtype, T, k, E, 256, seed=7)
+    d_y = torch.randn(seg.max_rows, n_out, generator=g).to(dtype)
+    w = (0.1 * torch.randn(E, n_out, n_in, generator=g)).to(dtype)
+    epi = _C.CK_EPI_GROUPED if epilogue == "grouped" else _C.CK_EPI_SCATTER
+    rows = seg.max_rows if epilogue == "grouped" else T * k
+    out = torch.zeros(rows, n_in, dtype=dtype, device=device)
+    ref = torch.zeros(rows, n_in, dtype=dtype, device=device)
+    scattermoe._gemm_dx(d_y.to(device), w.to(device), seg, epi, out)
+    scattermoe._gemm(d_y.to(device), 0, w.to(device).transpose(1, 2).contiguous(), seg, epi, ref)
+    assert torch.equal(out, ref)
+    seg_starts, counts, row_slot = _layout(seg)
+    for e in range(E):
+        s0, c = int(seg_starts[e]), int(counts[e])
+        if c == 0:
+            continue
+        expect = (d_y[s0 : s0 + c].double() @ w[e].double()).float()
+        got = out[s0 : s0 + c] if epilogue == "grouped" else out[torch.from_numpy(row_slot[s0 : s0 + c].astype("int64")).to(device)]
+        torch.testing.assert_close(got.float().cpu(), expect, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("align", [128, 256])
 @pytest.mark.parametrize("K,I", [(200, 72), (128, 256), (64, 136), (96, 440), (192, 440)])
 def test_grouped_gemm_swiglu_epilogues(device, dtype, align, K, I, gemm_tile):
