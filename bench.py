@@ -30,10 +30,11 @@ PEAK_HBM_GBS = 8000.0  # MI355X HBM3E
 # this same command, FETCH_SIZE scaled x2.0 and WRITE_SIZE x1.0 against transpose_batched_kernel (known size);
 # summary and commands: profiles/grouped_gemm_c3_moe_fwd_bwd.md. Not measurable from inside this process.
 TRAFFIC_BYTES_PER_LAUNCH = {
-    "grouped_gemm<scatter>": 2 * 5.727e6 * 1024 + 2.834e5 * 1024,  # 256 x 384 tiles
-    "grouped_gemm<dw>": 2 * 6.043e6 * 1024 + 1.516e6 * 1024,  # 256 x 384 tiles
-    "grouped_gemm<swiglu>": 2 * 8.842e6 * 1024 + 3.706e6 * 1024,
-    "grouped_gemm<grouped>": 2 * 4.111e6 * 1024 + 9.175e5 * 1024,
+    # scatter: mean of the two launches (c_fc dX on the contraction-strided kernel, c_proj fwd on 256 x 384 tiles)
+    "grouped_gemm<scatter>": 2 * 0.5 * (8.071e6 + 3.271e6) * 1024 + 0.5 * (2.621e5 + 2.986e5) * 1024,
+    "grouped_gemm<dw>": 2 * 6.034e6 * 1024 + 1.524e6 * 1024,  # 256 x 384 tiles
+    "grouped_gemm<swiglu>": 2 * 8.518e6 * 1024 + 3.706e6 * 1024,
+    "grouped_gemm<grouped>": 2 * 3.374e6 * 1024 + 9.175e5 * 1024,  # c_proj dX, contraction-strided weights
 }
 
 # workload: configs[2] of the baseline, the configuration its headline metric (MoE fwd+bwd TFLOP/s) is quoted on
