@@ -523,7 +523,7 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
           v.w[1] = (uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
           v.w[2] = (uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
           v.w[3] = (uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16);
-          store16(dst, v);
+          store16_nt(dst, v);
         }
       }
     };
@@ -534,7 +534,7 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
       for (int ch = tid; ch < kChunks; ch += NT) {
         const int c = ch / (BM / 8), r = (ch % (BM / 8)) * 8;
         T* dst = out_ptr(c, r);
-        if (dst != nullptr) store16(dst, load16(slab + c * kSlabLd + r));
+        if (dst != nullptr) store16_nt(dst, load16(slab + c * kSlabLd + r));
       }
     };
     auto sync_slab = [&]() { __syncthreads(); };

@@ -289,7 +289,7 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
         v.w[1] = (uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
         v.w[2] = (uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
         v.w[3] = (uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16);
-        store16(dst, v);
+        store16_nt(dst, v);
       }
     }
   };

@@ -18,7 +18,7 @@
 #include "gemm_common.h"
 
 #ifndef CK_ABLATE
-#define CK_ABLATE 0  // measurement builds only: 1 no barrier, 2 no loads in the loop, 4 no fragment reads, 8 no wait for the loads, 32 no epilogue, 64 no MFMA
+#define CK_ABLATE 0  // measurement builds only: 1 no barrier, 2 no loads in the loop, 4 no fragment reads, 8 no wait for the loads, 32 no epilogue, 64 no MFMA, 128 no row-major output stores
 #endif
 
 namespace ck {
@@ -331,28 +331,44 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
   auto tile_col = [&](int sc, int pass) {
     return (sc / (kSlabBlocks * 32)) * WN + pass * (kSlabBlocks * 32) + sc % (kSlabBlocks * 32);
   };
-  auto drain_rows = [&](auto&& out_ptr /* (tile row, slab column) -> address of 8 output columns, or nullptr */) {
-    const int l16 = tid & 15, grp = tid >> 4;
+  // Row-major drain. 16 lanes take a 4-row x 32-column block (what one transposing read pair delivers); the four lane
+  // groups of a wave take two adjacent column blocks of two adjacent row blocks, so that a store instruction writes whole
+  // 128-byte lines. The stores are non-temporal: outputs are written once and read by a later launch, and as plain
+  // stores they displace the operand panels that neighbouring tiles re-read from L2 (measured on 256 x 256 tiles with
+  // K = 2048: 7 to 13 % of the launch). Rows and column pairs are walked in unrolled loops: every address is a per-lane base plus a compile-time offset. row_ptr(tile row) -> address of the
+  // output row at the tile's first column (nullptr: pad row), block_col(cb) -> output column of slab column block cb
+  // relative to that, cols_left = valid columns from there on, tile_cols = columns the tile spans.
+  auto drain_rows = [&](auto&& row_ptr, auto&& block_col, int64_t cols_left, int tile_cols) {
+    const int l16 = tid & 15, csel = (tid >> 4) & 1, rsel = (tid >> 5) & 1;
     const int tq = l16 & 3, tj = l16 >> 2;  // as a source lane: which slab column this lane points at
     const int oq = l16 >> 2, oe = l16 & 3;  // as a destination lane: 8 columns oq of row oe of the 4 x 32 block
-    constexpr int kColBlocks = kSlabCols / 32;
-    constexpr int kBlocks = (BM / 4) * kColBlocks;
-#pragma unroll 4
-    for (int b = grp; b < kBlocks; b += NT / 16) {
-      const int rb = b / kColBlocks, cb = b % kColBlocks;
-      const T* src = slab + (cb * 32 + 8 * tq + tj) * kSlabLd + rb * 4;
-      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(src));
-      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(src + 4 * kSlabLd));
-      T* dst = out_ptr(rb * 4 + oe, cb * 32 + 8 * oq);
-      if (dst != nullptr) {
-        vec16 v;
-        v.w[0] = (uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
-        v.w[1] = (uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
-        v.w[2] = (uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
-        v.w[3] = (uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16);
-        store16(dst, v);
-      }
-    }
+    constexpr int kColPairs = kSlabCols / 64, kRowIters = (BM / 4) / (2 * NT / kWave);
+    static_assert(kSlabCols % 64 == 0 && (BM / 4) % (2 * NT / kWave) == 0, "whole column pairs and row iterations");
+    const bool cols_full = cols_left >= tile_cols;
+    auto body = [&](auto checked) {
+      static_for<kRowIters>([&](auto it) {
+        const int rb = (it * (NT / kWave) + wave) * 2 + rsel;
+        T* dst_row = row_ptr(rb * 4 + oe);
+        if (dst_row != nullptr) dst_row += 8 * oq;
+        const T* src_row = slab + (csel * 32 + 8 * tq + tj) * kSlabLd + rb * 4;
+        static_for<kColPairs>([&](auto cp) {
+          const T* src = src_row + cp * 64 * kSlabLd;
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(src));
+          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(src + 4 * kSlabLd));
+          const int col = csel ? block_col(std::integral_constant<int, 2 * decltype(cp)::value + 1>{}) : block_col(std::integral_constant<int, 2 * decltype(cp)::value>{});
+          if (dst_row != nullptr && (!checked || col + 8 * oq < cols_left) && (!(CK_ABLATE & 128) || lo[0] == 12345)) {
+            vec16 v;
+            v.w[0] = (uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
+            v.w[1] = (uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
+            v.w[2] = (uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
+            v.w[3] = (uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16);
+            store16_nt(dst_row + col, v);
+          }
+        });
+      });
+    };
+    if (cols_full) body(std::false_type{});
+    else body(std::true_type{});
   };
   auto drain_cols = [&](auto&& out_ptr /* (slab column, tile row) -> address of 8 rows of that column, or nullptr */) {
     constexpr int kChunks = kSlabCols * (BM / 8);
@@ -360,7 +376,7 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
     for (int ch = tid; ch < kChunks; ch += NT) {
       const int c = ch / (BM / 8), r = (ch % (BM / 8)) * 8;
       T* dst = out_ptr(c, r);
-      if (dst != nullptr) store16(dst, load16(slab + c * kSlabLd + r));
+      if (dst != nullptr) store16_nt(dst, load16(slab + c * kSlabLd + r));
     }
   };
 
@@ -371,10 +387,12 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
         return Elem<T>::down(acc[i][pass * kSlabBlocks + jj][4 * q + s]);
       });
       __syncthreads();
-      drain_rows([&](int r, int sc) -> T* {
-        const int64_t m = m0 + r, n = (int64_t)nt * BN + tile_col(sc, pass);
-        return (m < prm.M && n < prm.N) ? dw + m * prm.N + n : nullptr;
-      });
+      drain_rows(
+          [&](int r) -> T* {
+            const int64_t m = m0 + r;
+            return m < prm.M ? dw + m * prm.N + (int64_t)nt * BN : nullptr;
+          },
+          [&](auto cb) { return tile_col(cb * 32, pass); }, prm.N - (int64_t)nt * BN, BN);
       __syncthreads();
     });
   } else if constexpr (MODE == kGrouped || MODE == kScatter) {
@@ -391,12 +409,14 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
         });
       }
       __syncthreads();
-      drain_rows([&](int r, int sc) -> T* {
-        const int64_t p = m0 + r, n = (int64_t)nt * BN + tile_col(sc, pass);
-        if (p >= valid_end || n >= prm.N) return nullptr;
-        const int64_t row = (MODE == kScatter) ? (int64_t)scatter_rows[r] : p;
-        return y + row * prm.N + n;
-      });
+      drain_rows(
+          [&](int r) -> T* {
+            const int64_t p = m0 + r;
+            if (!tile_full && p >= valid_end) return nullptr;
+            const int64_t row = (MODE == kScatter) ? (int64_t)scatter_rows[r] : p;
+            return y + row * prm.N + (int64_t)nt * BN;
+          },
+          [&](auto cb) { return tile_col(cb * 32, pass); }, prm.N - (int64_t)nt * BN, BN);
       if (MODE == kGrouped && y_t != nullptr) {
         drain_cols([&](int sc, int r) -> T* {
           const int64_t n = (int64_t)nt * BN + tile_col(sc, pass);
@@ -431,13 +451,16 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
         });
       }
       __syncthreads();
-      drain_rows([&](int r, int sc) -> T* {
-        const int64_t p = m0 + r, col = act_col(sc);
-        if (p >= valid_end || col >= prm.I) return nullptr;
-        if (pass == 0) return pre + p * two_i + col;
-        if (pass == 1) return pre + p * two_i + prm.I + col;
-        return act + p * prm.I + col;
-      });
+      const int64_t col0 = (int64_t)nt * (BN / 2);  // the tile's first activation column
+      drain_rows(
+          [&](int r) -> T* {
+            const int64_t p = m0 + r;
+            if (!tile_full && p >= valid_end) return nullptr;
+            if (pass == 0) return pre + p * two_i + col0;
+            if (pass == 1) return pre + p * two_i + prm.I + col0;
+            return act + p * prm.I + col0;
+          },
+          [&](auto cb) { return (int)(act_col(cb * 32) - col0); }, prm.I - col0, BN / 2);
       if (pass == 2 && act_t != nullptr) {
         drain_cols([&](int sc, int r) -> T* {
           const int64_t col = act_col(sc);
