@@ -8,8 +8,9 @@
 // the LDS: step kt multiplies out of one stage while the loads of step kt + 1 fill the other.
 //
 // Workgroup = 8 waves (two per SIMD) in a 4 x 2 grid, wave tile 64 x BN/2 = 2 x (BN/64) v_mfma_f32_32x32x16 blocks.
-// Fragments are single-buffered and rotate through the four 16-wide slices of a step: a register set is reloaded for the
-// next slice as soon as the last MFMA that reads it has issued. One barrier per step, in front of the last slice: by then
+// Fragments rotate through the four 16-wide slices of a step. BN = 384 has registers for one fragment set: a register is
+// reloaded for the next slice as soon as the last MFMA that reads it has issued. BN = 256 keeps two sets and reads the
+// next slice's fragments a whole slice ahead. One barrier per step, in front of the last slice: by then
 // every wave has read the whole current stage (its last-slice fragments are in registers) and the next stage has landed,
 // so the loads of step kt + 2 go out under the last slice's MFMAs, as do the fragment reads of step kt + 1.
 // BN = 384 carries 20 % more FLOPs per loaded byte (153.6 against 128) and is used where the contraction is long.
@@ -18,7 +19,7 @@
 #include "gemm_common.h"
 
 #ifndef CK_ABLATE
-#define CK_ABLATE 0  // measurement builds only: 1 no barrier, 2 no loads in the loop, 4 no fragment reads, 8 no wait for the loads, 32 no epilogue, 64 no MFMA, 128 no row-major output stores
+#define CK_ABLATE 0  // measurement builds only: 1 no barrier, 2 no loads in the loop, 4 no fragment reads, 8 no wait for the loads, 16 every step loads the first two K steps again (L2 hits), 32 no epilogue, 64 no MFMA, 128 no row-major output stores, 512 single fragment set at BN = 256
 #endif
 
 namespace ck {
@@ -175,8 +176,8 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
   const uint32_t wave_a = __builtin_amdgcn_readfirstlane(lds_base + wave * A_LD * 1024);
   const uint32_t wave_b = __builtin_amdgcn_readfirstlane(lds_base + BM * kRowBytes + wave * B_LD * 1024);
   auto issue_one = [&](int step, int g) {
-    const int64_t kb = (int64_t)step * kRowBytes;
-    const int64_t kb_b = BT ? (int64_t)step * BK * prm.ldw * 2 : kb;  // BT: 64 contraction rows further down
+    const int64_t kb = (CK_ABLATE & 16) ? (int64_t)(step & 1) * kRowBytes : (int64_t)step * kRowBytes;
+    const int64_t kb_b = BT ? (int64_t)((CK_ABLATE & 16) ? (step & 1) : step) * BK * prm.ldw * 2 : kb;  // BT: 64 contraction rows further down
     const uint32_t st = (uint32_t)((step & (NSTAGE - 1)) * kStageBytes);
     if (g < A_LD) dma16(a_base + kb + a_off[g], wave_a + st + g * 1024);
     else dma16(b_base + kb_b + b_off[g - A_LD], wave_b + st + (g - A_LD) * 1024);
@@ -194,9 +195,12 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
   for (int sl = 0; sl < KS; ++sl) slice_off[sl] = ((2 * sl + fh) ^ fsw) * 16;
   const int fa_row = (wm * WM + (lane & 31)) * kRowBytes;
   const int fb_row = BM * kRowBytes + (wn * WN + (lane & 31)) * kRowBytes;
-  frag_t fa[MI], fb[NI];
+  // 256-wide tiles have the registers for two fragment sets: the reads for the next slice then go out a whole slice ahead
+  constexpr bool kDouble = BN == 256 && (CK_ABLATE & 512) == 0;  // (measured: 2.5 to 3.5 % faster launches)
+  constexpr int kSets = kDouble ? 2 : 1;
+  frag_t fa[kSets][MI], fb[kSets][NI];
   auto read_a = [&](int stage, int sl, int i) {
-    fa[i] = *reinterpret_cast<const frag_t*>(lds_c + stage * kStageBytes + slice_off[sl] + fa_row + i * 32 * kRowBytes);
+    fa[kDouble ? (sl & 1) : 0][i] = *reinterpret_cast<const frag_t*>(lds_c + stage * kStageBytes + slice_off[sl] + fa_row + i * 32 * kRowBytes);
   };
   // BT: lane l = 16 g + i of a transposing read points at 4 consecutive columns (4 (i % 4) ..) of contraction row i / 4
   // of a 4-row x 16-column patch and receives the 4 rows of column i; two reads (rows +0..3, +4..7) make the 8 contraction
@@ -220,17 +224,17 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
       } u;
       u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr16x4 __attribute__((address_space(3)))*)(p));
       u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr16x4 __attribute__((address_space(3)))*)(p + 4 * kBtRowBytes));
-      fb[j] = u.f;
+      fb[kDouble ? (sl & 1) : 0][j] = u.f;
     } else {
-      fb[j] = *reinterpret_cast<const frag_t*>(lds_c + stage * kStageBytes + slice_off[sl] + fb_row + j * 32 * kRowBytes);
+      fb[kDouble ? (sl & 1) : 0][j] = *reinterpret_cast<const frag_t*>(lds_c + stage * kStageBytes + slice_off[sl] + fb_row + j * 32 * kRowBytes);
     }
   };
-  auto mfma = [&](int i, int j) {
+  auto mfma = [&](int set, int i, int j) {
     if constexpr ((CK_ABLATE & 64) != 0) {
-      asm volatile("" ::"v"(fa[i]), "v"(fb[j]));
+      asm volatile("" ::"v"(fa[set][i]), "v"(fb[set][j]));
       return;
     }
-    acc[i][j] = Mfma<T>::run(fa[i], fb[j], acc[i][j]);
+    acc[i][j] = Mfma<T>::run(fa[set][i], fb[set][j], acc[i][j]);
   };
 
   if (nk > 0) {
@@ -264,25 +268,46 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
         else if constexpr ((CK_ABLATE & 8) != 0) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       }
+      constexpr int cur = kDouble ? (decltype(sl)::value & 1) : 0;
+      if constexpr (kDouble) {
+        // reads for the next slice in the order it needs them, one after each of the first MI + NI MFMAs
+        auto reload = [&](int n) {
+          if (n == 0) read_a(ns, nsl, 0);
+          else if (n <= NI) read_b(ns, nsl, n - 1);
+          else read_a(ns, nsl, 1);
+        };
 #pragma unroll
-      for (int j = 0; j < NI; ++j) {
-        mfma(0, j);
-        if constexpr (kLast && kPhase == 0 && !(CK_ABLATE & 2)) {
-          if (j < kLoadsPerStep) issue_one(kt + 2, j);
+        for (int n = 0; n < 2 * NI; ++n) {
+          mfma(cur, n / NI, n % NI);
+          if constexpr (kLast && kPhase == 0 && !(CK_ABLATE & 2)) {
+            if (n < kLoadsPerStep) issue_one(kt + 2, n);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          if constexpr (kReload) {
+            if (n < MI + NI) reload(n);
+          }
         }
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      if constexpr (kReload) read_a(ns, nsl, 0);
+      } else {
 #pragma unroll
-      for (int j = 0; j < NI; ++j) {
-        mfma(1, j);
-        if constexpr (kLast && kPhase == 0 && !(CK_ABLATE & 2)) {
-          if (NI + j < kLoadsPerStep) issue_one(kt + 2, NI + j);
+        for (int j = 0; j < NI; ++j) {
+          mfma(0, 0, j);
+          if constexpr (kLast && kPhase == 0 && !(CK_ABLATE & 2)) {
+            if (j < kLoadsPerStep) issue_one(kt + 2, j);
+          }
+          __builtin_amdgcn_sched_barrier(0);
         }
-        __builtin_amdgcn_sched_barrier(0);
-        if constexpr (kReload) read_b(ns, nsl, j);
+        if constexpr (kReload) read_a(ns, nsl, 0);
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+          mfma(0, 1, j);
+          if constexpr (kLast && kPhase == 0 && !(CK_ABLATE & 2)) {
+            if (NI + j < kLoadsPerStep) issue_one(kt + 2, NI + j);
+          }
+          __builtin_amdgcn_sched_barrier(0);
+          if constexpr (kReload) read_b(ns, nsl, j);
+        }
+        if constexpr (kReload) read_a(ns, nsl, 1);
       }
-      if constexpr (kReload) read_a(ns, nsl, 1);
       __builtin_amdgcn_sched_barrier(0);
     };
     auto k_step = [&](int kt, auto phase) { static_for<KS>([&](auto sl) { slice(kt, sl, phase); }); };
