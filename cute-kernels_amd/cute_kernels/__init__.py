@@ -22,7 +22,7 @@ from .scattermoe import (
 )
 from .softmax import softmax_cute
 from .swiglu import swiglu_cute, swiglu_packed_cute
-from .utils import ceil_divide, divide_if_divisible, get_num_elements_and_hidden_size, set_seed
+from .utils import ceil_divide, divide_if_divisible, enable_cute_tracing, get_num_elements_and_hidden_size, set_seed
 
 # torch.compile support: the public functions switch to the registered ops while a trace is being taken
 from . import compile_ops as _compile_ops
@@ -32,3 +32,5 @@ from . import softmax as _m_softmax, swiglu as _m_swiglu
 for _m in (_m_count, _m_frn, _m_rms, _m_moe, _m_softmax, _m_swiglu):
     _m._ops = _compile_ops
 del _m
+
+from .cute_inductor import CuteInductor  # noqa: E402  (after the ops are wired: its rewrites call the public functions)

@@ -9,6 +9,7 @@ from __future__ import annotations
 import torch
 
 from . import _C
+from .utils import is_tracing
 
 _ops = None  # cute_kernels.compile_ops, set by the package once it is imported (used only while torch.compile traces)
 
@@ -49,7 +50,7 @@ def continuous_count_cute(x: torch.Tensor, size: int) -> torch.Tensor:
     assert x.dim() == 1, "x should be 1-dimensional"
     assert x.dtype in [torch.int32, torch.long]
 
-    if torch.compiler.is_compiling():
+    if is_tracing():
         return _ops.continuous_count(x, size)
     return _launch(x, size, want_offsets=False)[0]
 

@@ -10,7 +10,7 @@ from __future__ import annotations
 import torch
 
 from . import _C
-from .utils import get_num_elements_and_hidden_size
+from .utils import get_num_elements_and_hidden_size, is_tracing
 
 _ops = None  # cute_kernels.compile_ops, set by the package once it is imported (used only while torch.compile traces)
 
@@ -111,7 +111,7 @@ def fused_residual_add_rmsnorm_cute(
     Returns:
         tuple[torch.Tensor, torch.Tensor]: output activations, updated residual stream
     """
-    if torch.compiler.is_compiling():
+    if is_tracing():
         if weight is not None:
             assert weight.dim() == 1, "weight should be 1D"
             assert weight.size(-1) == x.size(-1), "hidden size for x and weight tensor is different"

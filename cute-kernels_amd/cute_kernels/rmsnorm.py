@@ -9,7 +9,7 @@ from __future__ import annotations
 import torch
 
 from . import _C
-from .utils import get_num_elements_and_hidden_size
+from .utils import get_num_elements_and_hidden_size, is_tracing
 
 _ops = None  # cute_kernels.compile_ops, set by the package once it is imported (used only while torch.compile traces)
 
@@ -86,7 +86,7 @@ def rmsnorm_cute(
     Returns:
         torch.Tensor: output tensor
     """
-    if torch.compiler.is_compiling():
+    if is_tracing():
         if weight is not None:
             assert weight.dim() == 1, "weight should be 1D"
             assert weight.size(-1) == x.size(-1), "hidden size for x and weight tensor is different"

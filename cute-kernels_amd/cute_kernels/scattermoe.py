@@ -15,6 +15,7 @@ from dataclasses import dataclass
 import torch
 
 from . import _C
+from .utils import is_tracing
 
 _ops = None  # cute_kernels.compile_ops, set by the package once it is imported (used only while torch.compile traces)
 
@@ -67,7 +68,7 @@ def route_topk_softmax(logits: torch.Tensor, k: int, long_indices: bool = True) 
     """Top-k over the logits and softmax over the k selected logits in fp32, cast back to logits.dtype
     (torch_implementation.py:122-135). Equal logits: the lowest expert index wins. The indices come back as int64 like
     torch.topk's; long_indices=False keeps the kernel's int32 (what the sort consumes fastest)."""
-    if torch.compiler.is_compiling():
+    if is_tracing():
         gates, selected = _ops.route_topk_softmax(logits, k)
         return gates.to(logits.dtype), (selected.long() if long_indices else selected)
     return _RouteTopKSoftmax.apply(logits, k, long_indices)
@@ -142,7 +143,7 @@ def sort_by_expert(expert_ids: torch.Tensor, num_experts: int, align: int | None
     assert expert_ids.dtype in (torch.int32, torch.long)
     if align is None:
         align = choose_align(expert_ids.numel(), num_experts)
-    if torch.compiler.is_compiling():
+    if is_tracing():
         return _ops.sort_by_expert_segments(expert_ids, num_experts, align)
     return _sort_by_expert_eager(expert_ids, num_experts, align)
 
@@ -461,7 +462,7 @@ def experts_up(
 ) -> torch.Tensor:
     """x [T, H] -> c_fc output in padded grouped order [max_rows, N] (+ bias[e] on expert e's rows)."""
     _check_expert_dtypes(x, weight)
-    if torch.compiler.is_compiling():
+    if is_tracing():
         return _ops.experts_up(
             x, weight, bias, seg.seg_starts, seg.counts, seg.tile_expert, seg.row_slot, seg.max_rows, seg.num_experts,
             seg.align, k,
@@ -475,7 +476,7 @@ def experts_down(
 ) -> torch.Tensor:
     """h [max_rows, I] (padded grouped) -> sum_k gates * (c_proj output + bias[e]) in token order [T, N]."""
     _check_expert_dtypes(h, weight)
-    if torch.compiler.is_compiling():
+    if is_tracing():
         slot_expert = _slot_experts(seg) if bias is not None else None
         return _ops.experts_down(
             h, weight, gates.to(h.dtype), bias, slot_expert, seg.seg_starts, seg.counts, seg.tile_expert, seg.row_slot,
@@ -577,7 +578,7 @@ def swiglu_experts(
     """Fused expert block for `activation_function = swiglu_packed_cute`, `is_glu=True` (c_fc columns [up | gate])."""
     _check_expert_dtypes(x, w_fc, w_proj)
     assert w_fc.size(1) % 16 == 0, "intermediate size should be a multiple of 8"
-    if torch.compiler.is_compiling():
+    if is_tracing():
         grad = torch.is_grad_enabled()
         return _ops.swiglu_experts(
             x, w_fc, w_proj, gates.to(x.dtype), seg.seg_starts, seg.counts, seg.tile_expert, seg.row_slot, seg.max_rows,

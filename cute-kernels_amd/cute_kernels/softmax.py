@@ -9,7 +9,7 @@ from __future__ import annotations
 import torch
 
 from . import _C
-from .utils import get_num_elements_and_hidden_size
+from .utils import get_num_elements_and_hidden_size, is_tracing
 
 _ops = None  # cute_kernels.compile_ops, set by the package once it is imported (used only while torch.compile traces)
 
@@ -57,6 +57,6 @@ def softmax_cute(x: torch.Tensor, logits_multiplier: float | None = None) -> tor
     Returns:
         torch.Tensor: output tensor
     """
-    if torch.compiler.is_compiling():
+    if is_tracing():
         return _ops.softmax(x, 1.0 if logits_multiplier is None else float(logits_multiplier))
     return _Softmax_Cute.apply(x, logits_multiplier)

@@ -8,7 +8,7 @@ from __future__ import annotations
 import torch
 
 from . import _C
-from .utils import divide_if_divisible
+from .utils import divide_if_divisible, is_tracing
 
 _ops = None  # cute_kernels.compile_ops, set by the package once it is imported (used only while torch.compile traces)
 
@@ -111,7 +111,7 @@ def swiglu_cute(
     Returns:
         torch.Tensor: output tensor
     """
-    if torch.compiler.is_compiling():
+    if is_tracing():
         assert gate.size() == up.size(), "tensors gate and up should have same shape"
         assert gate.dtype == up.dtype, "tensors gate and up should have same dtype"
         return _ops.swiglu(gate, up)
@@ -128,7 +128,7 @@ def swiglu_packed_cute(x: torch.Tensor) -> torch.Tensor:
     Returns:
         torch.Tensor: output tensor
     """
-    if torch.compiler.is_compiling():
+    if is_tracing():
         divide_if_divisible(x.size(-1), 2)
         return _ops.swiglu_packed(x)
     return _SwigluPacked_Cute.apply(x)

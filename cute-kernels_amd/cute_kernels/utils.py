@@ -2,10 +2,33 @@
 
 from __future__ import annotations
 
+import contextlib
 import random
 
 import numpy as np
 import torch
+
+# True while a graph that calls this package's public functions is being re-traced outside dynamo (CuteInductor hands the
+# rewritten FX graph to AOTAutograd / inductor): the functions then take their custom-op form, as they do under dynamo.
+_IS_CUTE_TRACING = False
+
+
+@contextlib.contextmanager
+def enable_cute_tracing():
+    """Reference: cute_kernels/utils/custom_op.py:15-22."""
+    global _IS_CUTE_TRACING
+    previous = _IS_CUTE_TRACING
+    _IS_CUTE_TRACING = True
+    try:
+        yield
+    finally:
+        _IS_CUTE_TRACING = previous
+
+
+def is_tracing() -> bool:
+    """Whether the public functions must dispatch to their torch.library custom ops (dynamo or cute tracing) instead of
+    the eager autograd.Function path. Reference: cute_kernels/utils/custom_op.py:26."""
+    return _IS_CUTE_TRACING or torch.compiler.is_compiling()
 
 
 def set_seed(seed: int) -> None:

@@ -83,3 +83,57 @@ def test_moe_layer_compiled(device, act, is_glu, add_bias):
     # inference: nothing is saved, nothing breaks
     with torch.no_grad():
         assert torch.equal(compiled(x)[0], moe(x)[0])
+
+
+class _NormGluNorm(torch.nn.Module):  # examples/cute_inductor.py:21-33 of the reference, with a packed SwiGLU in the middle
+    def __init__(self) -> None:
+        super().__init__()
+        self.norm1 = torch.nn.RMSNorm(256, eps=1e-5)
+        self.linear = torch.nn.Linear(256, 1024)
+        self.norm2 = torch.nn.RMSNorm(512, eps=1e-6)  # explicit: torch's GPU kernel evaluates a None eps in fp32, rmsnorm_cute in x.dtype
+
+    def forward(self, x):
+        x = self.linear(self.norm1(x))
+        up, gate = x.chunk(2, dim=-1)
+        return self.norm2(up * torch.nn.functional.silu(gate))
+
+
+@pytest.mark.parametrize("then_inductor", [False, True])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_cute_inductor_rewrites_match_the_torch_model(device, dtype, then_inductor):
+    """The model compiled through CuteInductor (rmsnorm_cute + swiglu_packed_cute swapped in) against the same model run
+    by torch eagerly: outputs and every gradient within the elementwise-kernel tolerances (fp32 1e-5; bf16 one rounding
+    step of values of order 1: atol 2e-2, rtol 2e-2)."""
+    from cute_kernels import CuteInductor
+
+    torch.manual_seed(0)
+    model = _NormGluNorm().to(dtype).to(device)
+    x = torch.randn(333, 256, device=device, dtype=dtype)
+    g = torch.randn(333, 512, device=device, dtype=dtype)
+    x_ref = x.clone().requires_grad_()
+    model(x_ref).backward(g)
+    want = [x_ref.grad] + [p.grad.clone() for p in model.parameters()]
+    want_y = model(x)
+    for p in model.parameters():
+        p.grad = None
+
+    seen = []
+    inductor = CuteInductor(use_torch_inductor_after_cute_inductor=then_inductor)
+
+    def backend(gm, example_inputs):
+        run = inductor.compiler(gm, example_inputs)
+        seen.extend(n.target for n in gm.graph.nodes if n.op == "call_function")
+        return run
+
+    compiled = torch.compile(model, backend=backend, fullgraph=True)
+    x_got = x.clone().requires_grad_()
+    y = compiled(x_got)
+    assert seen.count(ck.rmsnorm_cute) == 2 and seen.count(ck.swiglu_packed_cute) == 1
+    y.backward(g)
+    got = [x_got.grad] + [p.grad for p in model.parameters()]
+    tol = dict(atol=1e-5, rtol=1e-5) if dtype == torch.float32 else dict(atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(y, want_y, **tol)
+    for a, b in zip(got, want):
+        # weight gradients sum 333 rows: compare in units of the gradient's own scale
+        scale = max(1.0, float(b.float().abs().max()))
+        torch.testing.assert_close(a.float() / scale, b.float() / scale, **tol)
