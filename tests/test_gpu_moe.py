@@ -360,3 +360,85 @@ def test_moe_fused_path_equals_unfused_path_at_mixtral_row_shape(device):
     with torch.no_grad():
         yp, _ = moe(x[perm])
     torch.testing.assert_close(yp, ya.detach()[perm], rtol=RTOL, atol=ATOL)
+
+
+def _close_via_truth_on_device(ours, oracle, truth, what, rtol=RTOL, atol=ATOL):
+    """Per element: within atol * s + rtol * |x| of the bf16 oracle, or no further from the fp32 truth than the oracle is
+    plus that margin; s = max(1, RMS of the tensor): at these sizes outputs and gradients are sums of thousands of O(1)
+    terms, and the absolute tolerance is stated in units of their typical magnitude. At most one element in a million may
+    miss that bound (an output element is a gate-weighted sum of per-expert rows that are themselves rounded to bf16:
+    where large rows cancel, the rounding of the parts exceeds any tolerance tied to the sum), and no element may be
+    further from the truth than 1.25 x the oracle's own worst element. Over the whole tensor: our RMS distance to the
+    truth is at most 1.1 x the oracle's."""
+    ours, oracle, truth = ours.detach().float(), oracle.detach().float(), truth.detach().float()
+    scale = max(1.0, float(truth.square().mean().sqrt()))
+    direct = (ours - oracle).abs() <= atol * scale + rtol * oracle.abs()
+    via = (ours - truth).abs() <= (oracle - truth).abs() + atol * scale + rtol * truth.abs()
+    bad = ~(direct | via)
+    err_ours = float((ours - truth).square().mean().sqrt())
+    err_oracle = float((oracle - truth).square().mean().sqrt())
+    worst_ours, worst_oracle = float((ours - truth).abs().max()), float((oracle - truth).abs().max())
+    assert int(bad.sum()) <= bad.numel() // 1_000_000 and worst_ours <= 1.25 * worst_oracle + atol * scale, (
+        f"{what}: {int(bad.sum())}/{bad.numel()} elements off; worst |ours-oracle|={float((ours - oracle).abs().max()):.4g}, "
+        f"|ours-truth|={worst_ours:.4g}, |oracle-truth|={worst_oracle:.4g}"
+    )
+    assert err_ours <= 1.1 * err_oracle + 1e-3 * scale, f"{what}: RMS error {err_ours:.4g} against the oracle's {err_oracle:.4g}"
+
+
+@pytest.mark.parametrize(
+    "name,T,E,k,H,I,skew",
+    [("C3", 16384, 8, 2, 4096, 14336, 0.5), ("C4", 8192, 64, 8, 2048, 1408, 0.0)],
+)
+def test_moe_layer_at_full_baseline_shapes(device, name, T, E, k, H, I, skew):
+    """The benchmark's own shapes, forward and every gradient, against the oracle layer evaluated by torch's library
+    routines on the same device (bf16, and fp32 as the truth that arbitrates rounding): same tolerances as the small
+    cases. `skew` > 0 adds the benchmark's rank-dependent router bias so that expert loads are ragged (Zipf-like)."""
+    torch.manual_seed(7)
+    dtype = torch.bfloat16
+    moe = cute_kernels.MoE(E, k, H, I, cute_kernels.swiglu_packed_cute, True, False, 0.02).to(dtype)
+    oracle = _OracleWithSelection(E, k, H, I, mo.swiglu_packed_torch, True, False, 0.02).to(dtype)
+    oracle.load_state_dict(moe.state_dict())
+    truth = _OracleWithSelection(E, k, H, I, mo.swiglu_packed_torch, True, False, 0.02).float()
+    truth.load_state_dict({n: v.float() for n, v in moe.state_dict().items()})
+    moe, oracle, truth = moe.to(device), oracle.to(device), truth.to(device)
+    bias = (-skew * torch.log(torch.arange(1, E + 1, dtype=torch.float32))).to(device)
+    for layer in (moe, oracle, truth):
+        layer.gate.register_forward_hook(lambda mod, inp, out: out + bias.to(out.dtype))
+
+    x = torch.randn(T, H, generator=torch.Generator().manual_seed(1)).to(dtype).to(device)
+    r = torch.randn(T, H, generator=torch.Generator().manual_seed(2)).to(dtype).to(device)
+    xg, xo, xt = x.clone().requires_grad_(), x.clone().requires_grad_(), x.clone().float().requires_grad_()
+
+    captured = {}
+    orig = moe._compute_routing_weights
+
+    def spy(hs):
+        out = orig(hs)
+        captured["sel"] = out[2].detach()
+        return out
+
+    moe._compute_routing_weights = spy
+    y, logits = moe(xg)
+    oracle.forced_selection = truth.forced_selection = captured["sel"]
+    load = torch.bincount(captured["sel"].flatten(), minlength=E).float() / (T * k)
+    if skew > 0:
+        assert float(load.max()) > 2.5 * float(load.min())  # ragged segments really are exercised
+    yo, logits_o = oracle(xo)
+    yt, _ = truth(xt)
+    torch.testing.assert_close(logits.float(), logits_o.float(), rtol=RTOL, atol=ATOL)
+    _close_via_truth_on_device(y, yo.detach(), yt.detach(), f"{name} output")
+
+    (y * r).sum().backward()
+    (yo * r).sum().backward()
+    (yt * r.float()).sum().backward()
+    _close_via_truth_on_device(xg.grad, xo.grad, xt.grad, f"{name} x.grad", atol=2e-2)
+    for pname in ["c_fc", "c_proj"]:
+        _close_via_truth_on_device(
+            getattr(moe, pname).weight.grad, getattr(oracle, pname).weight.grad, getattr(truth, pname).weight.grad,
+            f"{name} {pname}.weight.grad", atol=3e-2,
+        )
+    eps = 2.0**-8
+    floor = 2 * eps * float(truth.last_router_weights.grad.abs().max()) * float(x.float().abs().max())
+    _close_via_truth_on_device(
+        moe.gate.weight.grad, oracle.gate.weight.grad, truth.gate.weight.grad, f"{name} gate.weight.grad", atol=3e-2 + floor
+    )
