@@ -39,6 +39,15 @@ struct Vec {
     }
     return v;
   }
+  // a 16-byte chunk fetched earlier (P > 1)
+  __device__ static inline Vec unpack(const vec16& raw) {
+    Vec v;
+    Pack16<T> k;
+    k.v = raw;
+#pragma unroll
+    for (int i = 0; i < P; ++i) v.f[i] = Elem<T>::up(k.e[i]);
+    return v;
+  }
   __device__ static inline Vec ones() {
     Vec v;
 #pragma unroll
@@ -95,38 +104,85 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_fwd_kernel(const T* __restrict
   const int lane = threadIdx.x % TPR;
   const int64_t row_stride = (int64_t)gridDim.x * ROWS;
   const float inv_h = 1.0f / (float)H;
+  // Cached rows in 16-byte chunks: the next row (and its residual row) is fetched, packed, before this row's reduction
+  // and stores; a lane's weight chunks are the same in every row and are fetched once. Rows of four chunks per lane
+  // would pay for the extra registers with occupancy (measured slower), so they load in place.
+  constexpr bool kPrefetch = NC > 0 && NC <= 2 && P > 1;
+  vec16 next_x[kPrefetch ? NC : 1], next_r[kPrefetch ? NC : 1], w_raw[kPrefetch ? NC : 1];
+  auto fetch = [&](int64_t r) {
+    if constexpr (kPrefetch) {
+      if (r < B) {
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          const int ch = c * TPR + lane;
+          if (ch < chunks) {
+            next_x[c] = load16_nt(x + r * H + (int64_t)ch * P);
+            if (fuse.residual != nullptr) next_r[c] = load16_nt(fuse.residual + r * H + (int64_t)ch * P);
+          }
+        }
+      }
+    }
+  };
+  if constexpr (kPrefetch) {
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const int ch = c * TPR + lane;
+      if (weight != nullptr && ch < chunks) w_raw[c] = load16(weight + (int64_t)ch * P);
+    }
+  }
+  const int64_t first_row = (int64_t)blockIdx.x * ROWS + threadIdx.x / TPR;
+  fetch(first_row);
   // TPR == kBlock: all threads of the block share the row, so the loop trip count is block-uniform (block_sum barriers)
-  for (int64_t row = (int64_t)blockIdx.x * ROWS + threadIdx.x / TPR; row < B; row += row_stride) {
+  for (int64_t row = first_row; row < B; row += row_stride) {
     const T* xr = x + row * H;
     T* yr = out + row * H;
     const T* rr = fuse.residual ? fuse.residual + row * H : nullptr;
     T* ar = fuse.residual ? fuse.added + row * H : nullptr;
     // the row to normalise: x, or the freshly written sum with the residual stream
+    auto add_residual = [&](Vec<T, P>& v, const Vec<T, P>& r, int ch) {
+#pragma unroll
+      for (int i = 0; i < P; ++i) {
+        float t = v.f[i];
+        if (fuse.multiplier != 1.0f) t = round_to<T>(__fmul_rn(t, fuse.multiplier));  // never contracted into an fma
+        v.f[i] = round_to<T>(__fadd_rn(t, r.f[i]));
+      }
+      v.store(ar + (int64_t)ch * P);
+    };
     auto load_x = [&](int ch) {
       // cached rows (NC > 0) are read once; streaming rows come back for the second pass
       Vec<T, P> v = NC > 0 ? Vec<T, P>::load_once(xr + (int64_t)ch * P) : Vec<T, P>::load(xr + (int64_t)ch * P);
-      if (rr != nullptr) {
-        const Vec<T, P> r = Vec<T, P>::load_once(rr + (int64_t)ch * P);
-#pragma unroll
-        for (int i = 0; i < P; ++i) {
-          float t = v.f[i];
-          if (fuse.multiplier != 1.0f) t = round_to<T>(__fmul_rn(t, fuse.multiplier));  // never contracted into an fma
-          v.f[i] = round_to<T>(__fadd_rn(t, r.f[i]));
-        }
-        v.store(ar + (int64_t)ch * P);
-      }
+      if (rr != nullptr) add_residual(v, Vec<T, P>::load_once(rr + (int64_t)ch * P), ch);
       return v;
     };
     float ss = 0.f;
     if constexpr (NC > 0) {
       Vec<T, P> xv[NC];
+      if constexpr (kPrefetch) {
 #pragma unroll
-      for (int c = 0; c < NC; ++c) {
-        const int ch = c * TPR + lane;
-        if (ch < chunks) {
-          xv[c] = load_x(ch);
+        for (int c = 0; c < NC; ++c) {
+          const int ch = c * TPR + lane;
+          if (ch < chunks) {
+            xv[c] = Vec<T, P>::unpack(next_x[c]);
+            if (rr != nullptr) add_residual(xv[c], Vec<T, P>::unpack(next_r[c]), ch);
+          }
+        }
+        fetch(row + row_stride);  // the packed registers are free again: the next row is in flight from here on
 #pragma unroll
-          for (int i = 0; i < P; ++i) ss += xv[c].f[i] * xv[c].f[i];
+        for (int c = 0; c < NC; ++c) {
+          if (c * TPR + lane < chunks) {
+#pragma unroll
+            for (int i = 0; i < P; ++i) ss += xv[c].f[i] * xv[c].f[i];
+          }
+        }
+      } else {
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          const int ch = c * TPR + lane;
+          if (ch < chunks) {
+            xv[c] = load_x(ch);
+#pragma unroll
+            for (int i = 0; i < P; ++i) ss += xv[c].f[i] * xv[c].f[i];
+          }
         }
       }
       ss = row_sum<TPR>(ss, scratch);
@@ -136,7 +192,9 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_fwd_kernel(const T* __restrict
       for (int c = 0; c < NC; ++c) {
         const int ch = c * TPR + lane;
         if (ch < chunks) {
-          const Vec<T, P> wv = weight ? Vec<T, P>::load(weight + (int64_t)ch * P) : Vec<T, P>::ones();
+          Vec<T, P> wv;
+          if constexpr (kPrefetch) wv = weight ? Vec<T, P>::unpack(w_raw[c]) : Vec<T, P>::ones();
+          else wv = weight ? Vec<T, P>::load(weight + (int64_t)ch * P) : Vec<T, P>::ones();
           Vec<T, P> y;
 #pragma unroll
           for (int i = 0; i < P; ++i) y.f[i] = xv[c].f[i] * rs * wv.f[i];
@@ -194,6 +252,40 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const T* __restrict
     }
   }
 
+  // Cached rows in 16-byte chunks: the next row's x and d_y are fetched (packed, 4 registers a chunk) before this row's
+  // reductions and stores, so that a row owner always has a row of loads in flight.
+  constexpr bool kPrefetch = NC > 0 && P > 1;
+  vec16 next_x[kPrefetch ? NC : 1], next_g[kPrefetch ? NC : 1], w_raw[kPrefetch ? NC : 1];
+  float next_rs = 0.f;
+  if constexpr (kPrefetch) {  // a lane sees the same weight chunks in every row: fetched once (loads return in order, so
+                              // a weight or rstd load issued behind the prefetch would wait for the whole next row)
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const int ch = c * TPR + lane;
+      if (weight != nullptr && ch < chunks) w_raw[c] = load16(weight + (int64_t)ch * P);
+    }
+  }
+  auto weight_chunk = [&](int c, int ch) {
+    if constexpr (kPrefetch) return weight ? Vec<T, P>::unpack(w_raw[c]) : Vec<T, P>::ones();
+    else return weight ? Vec<T, P>::load(weight + (int64_t)ch * P) : Vec<T, P>::ones();
+  };
+  auto fetch = [&](int64_t r) {
+    if constexpr (kPrefetch) {
+      if (r < B) {
+        if (rstd != nullptr) next_rs = rstd[r];
+#pragma unroll
+        for (int c = 0; c < NC; ++c) {
+          const int ch = c * TPR + lane;
+          if (ch < chunks) {
+            next_x[c] = load16_nt(x + r * H + (int64_t)ch * P);
+            next_g[c] = load16_nt(d_out + r * H + (int64_t)ch * P);
+          }
+        }
+      }
+    }
+  };
+  fetch(worker);
+
   // with TPR == 64 the waves of a block may run different trip counts; nothing below synchronises the block then
   for (int64_t row = worker; row < B; row += row_stride) {
     const T* xr = x + row * H;
@@ -214,15 +306,66 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const T* __restrict
       o.store(dxr + (int64_t)ch * P);
     };
     float dot = 0.f, ss = 0.f;
-    if constexpr (NC > 0) {
-      Vec<T, P> xv[NC], gv[NC];  // gv holds d_y * w
+    if constexpr (kPrefetch) {
+      // this row's chunks stay packed (4 registers each) and are unpacked in both passes: fewer live registers than
+      // holding them as floats, which keeps four waves per SIMD next to the prefetched row
+      vec16 cur_x[NC], cur_g[NC];
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        cur_x[c] = next_x[c];
+        cur_g[c] = next_g[c];
+      }
+      const float saved_rs = next_rs;
+      fetch(row + row_stride);
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const int ch = c * TPR + lane;
+        if (ch < chunks) {
+          const Vec<T, P> xv = Vec<T, P>::unpack(cur_x[c]), gv = Vec<T, P>::unpack(cur_g[c]), wv = weight_chunk(c, ch);
+#pragma unroll
+          for (int i = 0; i < P; ++i) {
+            ss += xv.f[i] * xv.f[i];
+            dot += gv.f[i] * wv.f[i] * xv.f[i];
+          }
+        }
+      }
+      dot = row_sum<TPR>(dot, scratch);
+      float rs;
+      if (rstd != nullptr) {
+        rs = saved_rs;
+      } else {
+        ss = row_sum<TPR>(ss, scratch);
+        rs = rsqrtf(ss * inv_h + eps);
+      }
+      const float coef = dot * rs * rs * rs * inv_h;
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {  // the compiler must not carry the first pass's unpacked floats over the reductions
+        asm volatile("" : "+v"(cur_x[c].w[0]), "+v"(cur_x[c].w[1]), "+v"(cur_x[c].w[2]), "+v"(cur_x[c].w[3]));
+        asm volatile("" : "+v"(cur_g[c].w[0]), "+v"(cur_g[c].w[1]), "+v"(cur_g[c].w[2]), "+v"(cur_g[c].w[3]));
+      }
+#pragma unroll
+      for (int c = 0; c < NC; ++c) {
+        const int ch = c * TPR + lane;
+        if (ch < chunks) {
+          const Vec<T, P> xv = Vec<T, P>::unpack(cur_x[c]), gv = Vec<T, P>::unpack(cur_g[c]), wv = weight_chunk(c, ch);
+          Vec<T, P> o;
+#pragma unroll
+          for (int i = 0; i < P; ++i) {
+            o.f[i] = rs * gv.f[i] * wv.f[i] - coef * xv.f[i];
+            dw[c].f[i] += gv.f[i] * xv.f[i] * rs;
+          }
+          finish(o, ch);
+        }
+      }
+    } else if constexpr (NC > 0) {
+      Vec<T, P> xv[NC], gv[NC];
 #pragma unroll
       for (int c = 0; c < NC; ++c) {
         const int ch = c * TPR + lane;
         if (ch < chunks) {
           xv[c] = Vec<T, P>::load_once(xr + (int64_t)ch * P);
           gv[c] = Vec<T, P>::load_once(gr + (int64_t)ch * P);
-          const Vec<T, P> wv = weight ? Vec<T, P>::load(weight + (int64_t)ch * P) : Vec<T, P>::ones();
+          const Vec<T, P> wv = weight_chunk(c, ch);
 #pragma unroll
           for (int i = 0; i < P; ++i) {
             ss += xv[c].f[i] * xv[c].f[i];
@@ -243,7 +386,7 @@ __global__ __launch_bounds__(kBlock) void rmsnorm_bwd_kernel(const T* __restrict
       for (int c = 0; c < NC; ++c) {
         const int ch = c * TPR + lane;
         if (ch < chunks) {
-          const Vec<T, P> wv = weight ? Vec<T, P>::load(weight + (int64_t)ch * P) : Vec<T, P>::ones();
+          const Vec<T, P> wv = weight_chunk(c, ch);
           Vec<T, P> o;
 #pragma unroll
           for (int i = 0; i < P; ++i) {
