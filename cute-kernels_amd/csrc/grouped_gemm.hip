@@ -891,6 +891,36 @@ extern "C" int ck_grouped_gemm_nn(const void* a, const void* w, int32_t N, int32
   return launch_line(prm, epilogue, 256, true, dtype, (unsigned)blocks, static_cast<hipStream_t>(stream), name);
 }
 
+extern "C" int ck_grouped_gemm_dw_rows(const void* a, const void* b, int32_t M, int32_t N, const ck_segments* seg,
+                                       void* dw, int32_t dtype, void* stream) {
+  const char* name = "ck_grouped_gemm_dw_rows";
+  if (int rc = check_segments(seg, name)) return rc;
+  CK_REQUIRE(a && b && dw, "%s: NULL argument", name);
+  CK_REQUIRE(seg->align % kLineK == 0, "%s: segments must start at multiples of %d rows (align=%d)", name, kLineK, seg->align);
+  CK_REQUIRE(M >= kLineBM && N >= 256 && M % 8 == 0 && N % 8 == 0,
+             "%s: M=%d N=%d must be multiples of 8 and at least 256", name, M, N);
+  CK_REQUIRE(aligned16(a) && aligned16(b), "%s: operands need 16-byte alignment", name);
+  GemmParams prm = {};
+  prm.a = a;
+  prm.w = b;
+  prm.lda = M;
+  prm.ldw = N;
+  prm.M = M;
+  prm.N = N;
+  prm.align = seg->align;
+  prm.num_experts = seg->num_experts;
+  prm.seg_starts = seg->seg_starts;
+  prm.counts = seg->counts;
+  prm.tile_expert = seg->tile_expert;
+  prm.row_slot = seg->row_slot;
+  prm.y = dw;
+  prm.m_tiles = (int)ceil_div(M, kLineBM);
+  prm.n_tiles = (int)ceil_div(N, 256);
+  const int64_t blocks = (int64_t)prm.m_tiles * prm.n_tiles * seg->num_experts;
+  CK_REQUIRE(blocks < (int64_t)0x7fffffff, "%s: grid too large", name);
+  return launch_line(prm, kDw, 256, true, dtype, (unsigned)blocks, static_cast<hipStream_t>(stream), name);
+}
+
 extern "C" int ck_grouped_gemm_dw(const void* a_t, const void* b_t, int64_t ld_t, int32_t M, int32_t N,
                                   const ck_segments* seg, void* dw, int32_t dtype, void* stream) {
   const char* name = "ck_grouped_gemm_dw";

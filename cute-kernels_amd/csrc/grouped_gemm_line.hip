@@ -120,29 +120,47 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
 
   // ---- global -> LDS addressing: lane l of a wave-load fills slot l (16 bytes) of 64 consecutive slots = 8 rows of 128 B;
   // the lane fetches the chunk that belongs in its slot, so the 8 lanes of a row read one whole line of global memory
+  // AT (weight gradients from row-major operands): both operands are [grouped rows, columns], i.e. contraction-strided;
+  // the A stage then has the layout described for BT below (64 contraction rows of BM columns) and its fragments come out
+  // through the same transposing reads. Rows past the expert's count are zeroed in LDS (zero_pad_slots).
+  constexpr bool AT = BT && MODE == kDw;
   const char* a_base = static_cast<const char*>(prm.a);
   const char* b_base = static_cast<const char*>(prm.w);
   if constexpr (MODE != kDw) b_base += (int64_t)expert * prm.w_expert_stride * 2;
+  if constexpr (AT) {
+    a_base += k_begin * prm.lda * 2;
+    b_base += k_begin * prm.ldw * 2;
+  }
+  constexpr int kAtRowBytes = BM * 2;
+  auto swap02 = [](int w) { return (w & ~5) | ((w & 1) << 2) | ((w >> 2) & 1); };
   uint32_t a_off[A_LD], b_off[B_LD];
 #pragma unroll
   for (int t = 0; t < A_LD; ++t) {
-    const int r = (wave * A_LD + t) * 8 + (lane >> 3);
-    const int c = (lane & 7) ^ swz128(r);
-    int64_t row;
-    if constexpr (MODE == kDw) {
-      row = min(m0 + r, (int64_t)prm.M - 1);
+    if constexpr (AT) {
+      const int pos = (wave * A_LD + t) * 1024 + lane * 16;  // byte position of this lane's slot in the A stage
+      const int n = pos / kAtRowBytes, slot16 = (pos % kAtRowBytes) / 16;
+      const int q = swap02((slot16 >> 1) ^ (n & 3));
+      int64_t col = m0 + (2 * q + (slot16 & 1)) * 8;
+      if (col >= prm.M) col = m0;  // ragged edge: re-read a valid chunk, never stored
+      a_off[t] = (uint32_t)(((int64_t)n * prm.lda + col) * 2);
     } else {
-      int64_t p = m0 + r;
-      if (p >= valid_end) p = valid_end - 1;  // pad rows re-read a valid row; their results are never stored
-      row = prm.a_gather_div > 0 ? (int64_t)(prm.row_slot[p] / prm.a_gather_div) : p;
+      const int r = (wave * A_LD + t) * 8 + (lane >> 3);
+      const int c = (lane & 7) ^ swz128(r);
+      int64_t row;
+      if constexpr (MODE == kDw) {
+        row = min(m0 + r, (int64_t)prm.M - 1);
+      } else {
+        int64_t p = m0 + r;
+        if (p >= valid_end) p = valid_end - 1;  // pad rows re-read a valid row; their results are never stored
+        row = prm.a_gather_div > 0 ? (int64_t)(prm.row_slot[p] / prm.a_gather_div) : p;
+      }
+      a_off[t] = (uint32_t)((row * prm.lda + k_begin) * 2 + c * 16);
     }
-    a_off[t] = (uint32_t)((row * prm.lda + k_begin) * 2 + c * 16);
   }
   // BT: 32-byte window q of contraction row n sits at window position swap02(q) ^ (n & 3) of the row (swap02 exchanges
   // bits 0 and 2 of the window index): the 4 rows x 32 bytes one 16-lane group of a transposing read touches fill one
   // 128-byte block, and the neighbouring group (next 16 columns) falls into the other half of the banks.
   constexpr int kBtRowBytes = BN * 2, kBtWindows = kBtRowBytes / 32;
-  auto swap02 = [](int w) { return (w & ~5) | ((w & 1) << 2) | ((w >> 2) & 1); };
 #pragma unroll
   for (int t = 0; t < B_LD; ++t) {
     if constexpr (BT) {
@@ -178,8 +196,9 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
   auto issue_one = [&](int step, int g) {
     const int64_t kb = (CK_ABLATE & 16) ? (int64_t)(step & 1) * kRowBytes : (int64_t)step * kRowBytes;
     const int64_t kb_b = BT ? (int64_t)((CK_ABLATE & 16) ? (step & 1) : step) * BK * prm.ldw * 2 : kb;  // BT: 64 contraction rows further down
+    const int64_t kb_a = AT ? (int64_t)step * BK * prm.lda * 2 : kb;
     const uint32_t st = (uint32_t)((step & (NSTAGE - 1)) * kStageBytes);
-    if (g < A_LD) dma16(a_base + kb + a_off[g], wave_a + st + g * 1024);
+    if (g < A_LD) dma16(a_base + kb_a + a_off[g], wave_a + st + g * 1024);
     else dma16(b_base + kb_b + b_off[g - A_LD], wave_b + st + (g - A_LD) * 1024);
   };
   auto issue = [&](int step) {
@@ -199,13 +218,33 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
   constexpr bool kDouble = BN == 256 && (CK_ABLATE & 512) == 0;  // (measured: 2.5 to 3.5 % faster launches)
   constexpr int kSets = kDouble ? 2 : 1;
   frag_t fa[kSets][MI], fb[kSets][NI];
+  typedef __attribute__((__vector_size__(4 * sizeof(short)))) short tr16x4;
+  int at_off[MI];
+  if constexpr (AT) {  // as bt_off below, on the A stage
+    const int g = lane >> 4, i = lane & 15, n_low = i >> 2;
+#pragma unroll
+    for (int b = 0; b < MI; ++b) {
+      const int q = (wm * WM + b * 32) / 16 + (g & 1);
+      at_off[b] = (8 * (g >> 1) + n_low) * kAtRowBytes + (swap02(q) ^ n_low) * 32 + 8 * (i & 3);
+    }
+  }
   auto read_a = [&](int stage, int sl, int i) {
-    fa[kDouble ? (sl & 1) : 0][i] = *reinterpret_cast<const frag_t*>(lds_c + stage * kStageBytes + slice_off[sl] + fa_row + i * 32 * kRowBytes);
+    if constexpr (AT) {
+      const char* p = lds_c + stage * kStageBytes + at_off[i] + 16 * sl * kAtRowBytes;
+      union {
+        tr16x4 h[2];
+        frag_t f;
+      } u;
+      u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr16x4 __attribute__((address_space(3)))*)(p));
+      u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr16x4 __attribute__((address_space(3)))*)(p + 4 * kAtRowBytes));
+      fa[kDouble ? (sl & 1) : 0][i] = u.f;
+    } else {
+      fa[kDouble ? (sl & 1) : 0][i] = *reinterpret_cast<const frag_t*>(lds_c + stage * kStageBytes + slice_off[sl] + fa_row + i * 32 * kRowBytes);
+    }
   };
   // BT: lane l = 16 g + i of a transposing read points at 4 consecutive columns (4 (i % 4) ..) of contraction row i / 4
   // of a 4-row x 16-column patch and receives the 4 rows of column i; two reads (rows +0..3, +4..7) make the 8 contraction
   // values of column 16 (g % 2) + i for k-half g / 2 -- the MFMA's B layout.
-  typedef __attribute__((__vector_size__(4 * sizeof(short)))) short tr16x4;
   int bt_off[NI];
   if constexpr (BT) {
     const int g = lane >> 4, i = lane & 15, n_low = i >> 2;
@@ -237,13 +276,36 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
     acc[i][j] = Mfma<T>::run(fa[set][i], fb[set][j], acc[i][j]);
   };
 
+  // AT: contraction rows past the expert's count (the ragged end of its last K step) hold whatever the buffers hold.
+  // Every lane overwrites, with zeros, the slots of such rows that its own loads filled -- after those loads have
+  // landed, before the barrier that publishes the stage; both operands, so no 0 * Inf can arise.
+  auto zero_pad_slots = [&](int step) {
+    if constexpr (AT) {
+      const int rows_here = (int)prm.counts[expert] - step * BK;
+      if (rows_here >= BK) return;
+      char* stage = lds_c + (step & (NSTAGE - 1)) * kStageBytes;
+#pragma unroll
+      for (int t = 0; t < A_LD; ++t) {
+        const int pos = (wave * A_LD + t) * 1024 + lane * 16;
+        if (pos / kAtRowBytes >= rows_here) *reinterpret_cast<vec16*>(stage + pos) = zero16();
+      }
+#pragma unroll
+      for (int t = 0; t < B_LD; ++t) {
+        const int pos = (wave * B_LD + t) * 1024 + lane * 16;
+        if (pos / kBtRowBytes >= rows_here) *reinterpret_cast<vec16*>(stage + BM * kRowBytes + pos) = zero16();
+      }
+    }
+  };
+
   if (nk > 0) {
     issue(0);
     if (nk > 1) {
       issue(1);
       asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kLoadsPerStep) : "memory");  // step 0 landed, all waves
     } else {
-      asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      zero_pad_slots(0);
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }
 #pragma unroll
     for (int i = 0; i < MI; ++i) read_a(0, 0, i);
@@ -266,7 +328,11 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
       if constexpr (kLast && kPhase < 2) {
         if constexpr ((CK_ABLATE & 1) != 0) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         else if constexpr ((CK_ABLATE & 8) != 0) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        else if constexpr (AT && kPhase == 1) {  // the stage that has just landed is the last K step
+          asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+          zero_pad_slots(kt + 1);
+          asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        } else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       }
       constexpr int cur = kDouble ? (decltype(sl)::value & 1) : 0;
       if constexpr (kDouble) {
@@ -523,8 +589,9 @@ int launch_bn(const GemmParams& prm, int mode, bool bt, unsigned blocks, hipStre
     if constexpr (BN == 256) {
       if (mode == kGrouped) return launch_mode<T, kGrouped, BN, true>(prm, blocks, stream, name);
       if (mode == kScatter) return launch_mode<T, kScatter, BN, true>(prm, blocks, stream, name);
+      if (mode == kDw) return launch_mode<T, kDw, BN, true>(prm, blocks, stream, name);  // both operands row-major
     }
-    set_error("%s: the contraction-strided weight operand goes with 256-wide tiles and the grouped / scatter epilogues", name);
+    set_error("%s: contraction-strided operands go with 256-wide tiles and the grouped / scatter / dW epilogues", name);
     return CK_ERR_ARG;
   }
   switch (mode) {

@@ -62,6 +62,7 @@ _SIGNATURES = {
     ),
     "ck_grouped_gemm_nn": (c_int32, [c_void_p, c_void_p, c_int32, c_int32, POINTER(ck_segments), c_int32, c_void_p, c_int32, c_void_p]),
     "ck_grouped_gemm_dw": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_int32, POINTER(ck_segments), c_void_p, c_int32, c_void_p]),
+    "ck_grouped_gemm_dw_rows": (c_int32, [c_void_p, c_void_p, c_int32, c_int32, POINTER(ck_segments), c_void_p, c_int32, c_void_p]),
     "ck_quant_rows_e4m3": (c_int32, [c_void_p, c_int64, c_int32, c_void_p, c_void_p, c_int32, c_void_p]),
     "ck_grouped_gemm_fp8": (
         c_int32,

@@ -373,7 +373,8 @@ def swiglu_experts(
     row_slot: Tensor, max_rows: int, num_experts: int, align: int, need_x: bool, need_fc: bool, need_proj: bool,
     need_gates: bool,
 ) -> tuple[Tensor, Tensor, Tensor, Tensor]:
-    """(out [T, H], pre [max_rows, 2I], act_t [I, max_rows] or empty, expanded [T * k, H])"""
+    """(out [T, H], pre [max_rows, 2I], the activation for d_w_proj ([I, max_rows] transposed, or [max_rows, I] when the
+    weight gradients read row-major operands) or empty, expanded [T * k, H])"""
     ctx = _Ctx((need_x, need_fc, need_proj, need_gates, False))
     seg = _segments(seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, align)
     out = _moe._SwigluExperts.forward(ctx, x, w_fc, w_proj, gates, seg)
@@ -391,7 +392,13 @@ def _(x, w_fc, w_proj, gates, seg_starts, counts, tile_expert, row_slot, max_row
     two_i = w_fc.shape[1]
     if not (need_x or need_fc or need_proj or need_gates):
         return x.new_empty(T, H), x.new_empty(0), x.new_empty(0), x.new_empty(0)
-    act_t = x.new_empty(two_i // 2, max_rows) if need_proj else x.new_empty(0)
+    I = two_i // 2
+    if not need_proj:
+        act_t = x.new_empty(0)
+    elif _moe._dw_from_rows(max_rows, num_experts, align, (H, I), (two_i, H)):
+        act_t = x.new_empty(max_rows, I)  # the activation itself: d_w_proj reads row-major operands
+    else:
+        act_t = x.new_empty(I, max_rows)
     return x.new_empty(T, H), x.new_empty(max_rows, two_i), act_t, x.new_empty(T * k, H)
 
 

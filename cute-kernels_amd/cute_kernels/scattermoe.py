@@ -279,6 +279,37 @@ def _gemm_dw(a_t, b_t, seg: ExpertSegments, dw):
         launch_timer.time("grouped_gemm<dw>", (M, N), launch)
 
 
+def _gemm_dw_rows(a, b, seg: ExpertSegments, dw):
+    """dw[e] = a[rows of e]^T @ b[rows of e] from row-major padded-grouped operands (no transposed copies)."""
+    E, M, N = dw.shape
+    cs = seg.c_struct()
+
+    def launch():
+        with torch.cuda.device(dw.device):
+            _C.check(
+                _C.lib().ck_grouped_gemm_dw_rows(
+                    _C.ptr(a), _C.ptr(b), M, N, ctypes.byref(cs), _C.ptr(dw), _C.dtype_code(dw.dtype), _C.stream()
+                )
+            )
+
+    if launch_timer is None:
+        launch()
+    else:
+        launch_timer.time("grouped_gemm<dw>", (M, N), launch)
+
+
+def _dw_from_rows(max_rows: int, num_experts: int, align: int, *shapes: tuple[int, int]) -> bool:
+    """Whether the weight-gradient GEMMs of shapes (M, N), ... read row-major operands (ck_grouped_gemm_dw_rows) instead
+    of transposed copies: whenever that kernel takes the shapes. Not writing (and not holding) the transposes outweighs
+    the 384-wide tiles the transposed form can use (measured: fine-grained layer 4 % faster, Mixtral-shape layer 0.4 %).
+    A function of sizes only, so that forward, backward and the traced (fake) implementations agree on which tensors
+    exist."""
+    import os
+
+    ok = os.environ.get("CK_GEMM_DW_ROWS", "1") != "0"  # measurement knob: 0 = always the transposed form
+    return ok and align % 64 == 0 and all(min(m, n) >= 256 and m % 8 == 0 and n % 8 == 0 for m, n in shapes)
+
+
 def _group_rows(src, coeff, fan_out, seg: ExpertSegments, want_grouped: bool, want_transposed: bool):
     """Padded grouped copy of `src` rows (fan_out == 0: src is already padded-grouped) and / or its transpose."""
     H = src.size(-1)
@@ -403,10 +434,14 @@ class _ExpertsUp(torch.autograd.Function):
         if len(ctx.needs_input_grad) > 4 and ctx.needs_input_grad[4]:
             d_bias = _expert_bias_grad(d_y, seg)
         if ctx.needs_input_grad[1]:
-            _, d_y_t = _group_rows(d_y, None, 0, seg, False, True)
-            _, x_t = _group_rows(x, None, k, seg, False, True)
             d_w = torch.empty_like(w)
-            _gemm_dw(d_y_t, x_t, seg, d_w)
+            if _dw_from_rows(seg.max_rows, seg.num_experts, seg.align, tuple(w.shape[1:])):
+                x_g, _ = _group_rows(x, None, k, seg, True, False)
+                _gemm_dw_rows(d_y, x_g, seg, d_w)
+            else:
+                _, d_y_t = _group_rows(d_y, None, 0, seg, False, True)
+                _, x_t = _group_rows(x, None, k, seg, False, True)
+                _gemm_dw(d_y_t, x_t, seg, d_w)
         if ctx.needs_input_grad[0]:
             d_expanded = torch.empty(T * k, K, dtype=x.dtype, device=x.device)
             _gemm_dx(d_y, w, seg, _C.CK_EPI_SCATTER, d_expanded)
@@ -444,13 +479,17 @@ class _ExpertsDown(torch.autograd.Function):
         if ctx.needs_input_grad[2]:
             _, d_gates = _combine(expanded, None, T, k, N, grad_out=grad_out, want_out=False, want_d_gates=True)
         need_w = ctx.needs_input_grad[1]
-        d_y, d_y_t = _group_rows(grad_out, gates, k, seg, True, need_w)
+        rows_form = _dw_from_rows(seg.max_rows, seg.num_experts, seg.align, (N, K))
+        d_y, d_y_t = _group_rows(grad_out, gates, k, seg, True, need_w and not rows_form)
         if len(ctx.needs_input_grad) > 4 and ctx.needs_input_grad[4]:
             d_bias = _expert_bias_grad(d_y, seg)  # d_y: the gate-scaled grad_out rows in padded grouped order
         if need_w:
-            _, h_t = _group_rows(h, None, 0, seg, False, True)
             d_w = torch.empty_like(w)
-            _gemm_dw(d_y_t, h_t, seg, d_w)
+            if rows_form:
+                _gemm_dw_rows(d_y, h, seg, d_w)
+            else:
+                _, h_t = _group_rows(h, None, 0, seg, False, True)
+                _gemm_dw(d_y_t, h_t, seg, d_w)
         if ctx.needs_input_grad[0]:
             d_h = torch.zeros(seg.max_rows, K, dtype=h.dtype, device=h.device)
             _gemm_dx(d_y, w, seg, _C.CK_EPI_GROUPED, d_h)
@@ -508,7 +547,9 @@ class _SwigluExperts(torch.autograd.Function):
 
         pre = torch.empty(seg.max_rows, two_i, dtype=dt, device=dev)
         act = torch.empty(seg.max_rows, I, dtype=dt, device=dev)
-        act_t = torch.empty(I, seg.ld_t, dtype=dt, device=dev) if ctx.needs_input_grad[2] else None
+        # d_w_proj needs the activation: transposed (written by the same epilogue) or, in the row-major form, as it is
+        rows_form = _dw_from_rows(seg.max_rows, seg.num_experts, seg.align, (H, I), (two_i, H))
+        act_t = torch.empty(I, seg.ld_t, dtype=dt, device=dev) if ctx.needs_input_grad[2] and not rows_form else None
         _gemm(x, k, w_fc, seg, _C.CK_EPI_SWIGLU, pre, y_t=act_t, aux=act)
 
         expanded = torch.empty(T * k, H, dtype=dt, device=dev)
@@ -516,13 +557,14 @@ class _SwigluExperts(torch.autograd.Function):
         out, _ = _combine(expanded, gates, T, k, H)
 
         if need_grad:
-            ctx.save_for_backward(x, w_fc, w_proj, gates, pre, act_t, expanded)
+            act_saved = (act if ctx.needs_input_grad[2] else None) if rows_form else act_t
+            ctx.save_for_backward(x, w_fc, w_proj, gates, pre, act_saved, expanded)
         ctx.seg = seg
         return out
 
     @staticmethod
     def backward(ctx, grad_out):
-        x, w_fc, w_proj, gates, pre, act_t, expanded = ctx.saved_tensors
+        x, w_fc, w_proj, gates, pre, act_saved, expanded = ctx.saved_tensors
         seg = ctx.seg
         T, H = x.shape
         k = gates.size(1)
@@ -532,15 +574,19 @@ class _SwigluExperts(torch.autograd.Function):
         grad_out = grad_out.contiguous()
         need_x, need_fc, need_proj, need_gates = ctx.needs_input_grad[:4]
         d_x = d_w_fc = d_w_proj = d_gates = None
+        rows_form = _dw_from_rows(seg.max_rows, seg.num_experts, seg.align, (H, I), (two_i, H))  # as in forward
 
         if need_gates:
             _, d_gates = _combine(expanded, None, T, k, H, grad_out=grad_out, want_out=False, want_d_gates=True)
 
-        # gate-scaled grad_out rows in padded grouped order (+ transpose for d_w_proj)
-        d_y, d_y_t = _group_rows(grad_out, gates, k, seg, True, need_proj)
+        # gate-scaled grad_out rows in padded grouped order (+ transpose for d_w_proj unless it reads rows)
+        d_y, d_y_t = _group_rows(grad_out, gates, k, seg, True, need_proj and not rows_form)
         if need_proj:
             d_w_proj = torch.empty_like(w_proj)
-            _gemm_dw(d_y_t, act_t, seg, d_w_proj)
+            if rows_form:
+                _gemm_dw_rows(d_y, act_saved, seg, d_w_proj)
+            else:
+                _gemm_dw(d_y_t, act_saved, seg, d_w_proj)
             del d_y_t
 
         if need_x or need_fc:
@@ -551,7 +597,7 @@ class _SwigluExperts(torch.autograd.Function):
             _gemm_dx(d_y, w_proj, seg, _C.CK_EPI_GROUPED, d_act)
             del d_y
             d_pre = torch.empty(seg.max_rows, two_i, dtype=dt, device=dev)
-            d_pre_t = torch.empty(two_i, seg.ld_t, dtype=dt, device=dev) if need_fc else None
+            d_pre_t = torch.empty(two_i, seg.ld_t, dtype=dt, device=dev) if need_fc and not rows_form else None
             with torch.cuda.device(dev):
                 _C.check(
                     _C.lib().ck_swiglu_bwd_grouped(
@@ -561,10 +607,15 @@ class _SwigluExperts(torch.autograd.Function):
                 )
             del d_act
             if need_fc:
-                _, x_t = _group_rows(x, None, k, seg, False, True)
                 d_w_fc = torch.empty_like(w_fc)
-                _gemm_dw(d_pre_t, x_t, seg, d_w_fc)
-                del d_pre_t, x_t
+                if rows_form:
+                    x_g, _ = _group_rows(x, None, k, seg, True, False)
+                    _gemm_dw_rows(d_pre, x_g, seg, d_w_fc)
+                    del x_g
+                else:
+                    _, x_t = _group_rows(x, None, k, seg, False, True)
+                    _gemm_dw(d_pre_t, x_t, seg, d_w_fc)
+                    del d_pre_t, x_t
             if need_x:
                 d_expanded = torch.empty(T * k, H, dtype=dt, device=dev)
                 _gemm_dx(d_pre, w_fc, seg, _C.CK_EPI_SCATTER, d_expanded)

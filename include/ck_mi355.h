@@ -181,6 +181,16 @@ int ck_grouped_gemm_nn(const void* a, const void* w, int32_t N, int32_t K, const
 int ck_grouped_gemm_dw(const void* a_t, const void* b_t, int64_t ld_t, int32_t M, int32_t N, const ck_segments* seg,
                        void* dw, int32_t dtype, void* stream);
 
+/* The same weight gradient from row-major operands: dW[e] = A[seg_e, :]^T * B[seg_e, :] with a [max_rows, M] and
+ * b [max_rows, N] padded-grouped rows (what the other kernels write anyway); no transposed copies. Pad rows may hold
+ * anything: they are not read into the product.
+ * Replaces: group_bwd_W / groupXtY_triton_kernel, which also reads DY and X row-major --
+ *           cute_kernels/kernels/scattermoe/triton_implementation/ops.py:81-105, kernels.py:136-222.
+ * dw [E, M, N]; experts with no rows get exact zeros. Needs seg->align % 64 == 0, M % 8 == 0, N % 8 == 0,
+ * M >= 256 and N >= 256 (one 256 x 256 tile). */
+int ck_grouped_gemm_dw_rows(const void* a, const void* b, int32_t M, int32_t N, const ck_segments* seg, void* dw,
+                            int32_t dtype, void* stream);
+
 /* ---------------------------------------------------------------------------------------------------------------
  * (c, fp8) quantised-expert forward path: e4m3 operands (OCP e4m3fn, the gfx950 format), fp32 accumulation
  * No counterpart in the reference (it has no fp8 code): the semantics are those of the same layer evaluated on the

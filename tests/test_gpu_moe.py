@@ -196,6 +196,33 @@ def test_grouped_gemm_dw(device, dtype, align, M, N, gemm_tile):
     assert float(dw[3].abs().max()) == 0.0  # empty expert: exact zeros (ops.py:252, kernels.py:181)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("align", [128, 256])
+@pytest.mark.parametrize("M,N", [(256, 256), (264, 520), (1024, 1032)])
+@pytest.mark.parametrize("T", [900, 40, 100])
+def test_grouped_gemm_dw_from_row_major_operands(device, dtype, align, M, N, T):
+    """ck_grouped_gemm_dw_rows: X^T DY per expert (kernels.py:136-222) read from the padded-grouped row-major buffers.
+    Pad rows are filled with NaN: they must not reach the product. Segments are ragged (counts that are not multiples of
+    the 64-row K step, one empty; T = 40: every expert inside a single K step, T = 100: one or two steps)."""
+    k, E = 2, 5
+    g, seg = _make_case(device, dtype, T, k, E, align, seed=3)
+    seg_starts, counts, row_slot = _layout(seg)
+    a = torch.full((seg.max_rows, M), float("nan"), dtype=dtype)
+    b = torch.full((seg.max_rows, N), float("nan"), dtype=dtype)
+    expect = torch.zeros(E, M, N)
+    for e in range(E):
+        lo, n = int(seg_starts[e]), int(counts[e])
+        a[lo : lo + n] = torch.randn(n, M, generator=g).to(dtype)
+        b[lo : lo + n] = torch.randn(n, N, generator=g).to(dtype)
+        if n:
+            expect[e] = a[lo : lo + n].float().t() @ b[lo : lo + n].float()
+    assert int(counts.min()) == 0 and any(int(c) % 64 for c in counts)
+    dw = torch.full((E, M, N), float("nan"), dtype=dtype, device=device)
+    scattermoe._gemm_dw_rows(a.to(device), b.to(device), seg, dw)
+    torch.testing.assert_close(dw.float().cpu(), expect, rtol=RTOL, atol=0.3)  # sums of up to ~700 O(1) products
+    assert float(dw[3].abs().max()) == 0.0  # empty expert: exact zeros (ops.py:252, kernels.py:181)
+
+
 # ---------------------------------------------------------------------------------------------------------------
 # whole layer
 # ---------------------------------------------------------------------------------------------------------------
