@@ -27,14 +27,14 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E
 
 # Bytes per launch between L2 and the fabric (fetched + written) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# this same command, FETCH_SIZE scaled x2.0 and WRITE_SIZE x1.0 against transpose_batched_kernel (known size);
+# this same command, FETCH_SIZE scaled x2.0 and WRITE_SIZE x1.0 against a 1 GiB device copy (known size);
 # summary and commands: profiles/grouped_gemm_c3_moe_fwd_bwd.md. Not measurable from inside this process.
 TRAFFIC_BYTES_PER_LAUNCH = {
     # scatter: mean of the two launches (c_fc dX on the contraction-strided kernel, c_proj fwd on 256 x 384 tiles)
-    "grouped_gemm<scatter>": 2 * 0.5 * (8.071e6 + 3.271e6) * 1024 + 0.5 * (2.621e5 + 2.986e5) * 1024,
-    "grouped_gemm<dw>": 2 * 6.034e6 * 1024 + 1.524e6 * 1024,  # 256 x 384 tiles
-    "grouped_gemm<swiglu>": 2 * 8.518e6 * 1024 + 3.706e6 * 1024,
-    "grouped_gemm<grouped>": 2 * 3.374e6 * 1024 + 9.175e5 * 1024,  # c_proj dX, contraction-strided weights
+    "grouped_gemm<scatter>": 2 * 0.5 * (8.118e6 + 3.280e6) * 1024 + 0.5 * (2.621e5 + 3.134e5) * 1024,
+    "grouped_gemm<dw>": 2 * 5.842e6 * 1024 + 1.376e6 * 1024,  # both weight gradients, row-major operands
+    "grouped_gemm<swiglu>": 2 * 8.606e6 * 1024 + 2.753e6 * 1024,
+    "grouped_gemm<grouped>": 2 * 3.964e6 * 1024 + 9.175e5 * 1024,  # c_proj dX, contraction-strided weights
 }
 
 # workload: configs[2] of the baseline, the configuration its headline metric (MoE fwd+bwd TFLOP/s) is quoted on
