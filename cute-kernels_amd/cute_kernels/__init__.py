@@ -21,6 +21,7 @@ from .scattermoe import (
     swiglu_experts,
 )
 from .softmax import softmax_cute
+from .router_stats import load_balancing_loss, load_balancing_stats
 from .swiglu import swiglu_cute, swiglu_packed_cute
 from .utils import ceil_divide, divide_if_divisible, enable_cute_tracing, get_num_elements_and_hidden_size, set_seed
 

@@ -184,3 +184,16 @@ def moe_e4m3_forward_oracle(moe: "MoEOracle", x: torch.Tensor, selected: torch.T
             y = (w2[e] @ (aq.float()[0] * a_s)).to(dt)
             out[t] += gates[t, j].float() * y.float()
     return out.to(dt)
+
+
+def load_balancing_loss_torch(router_logits: torch.Tensor, selected_experts: torch.Tensor) -> torch.Tensor:
+    """Switch-transformer auxiliary loss written with one-hot masks (the form of the Hugging Face Mixtral loss for one
+    layer): E * sum over slots and experts of mean_t one_hot(selected)[t, slot, e] * mean_t softmax(logits)[t, e].
+    No counterpart in the reference (it returns router_logits and leaves the loss to the caller): parity unpinned
+    upstream; pinned here by the closed form in tests/test_oracle.py."""
+    E = router_logits.size(-1)
+    probs = F.softmax(router_logits.float(), dim=-1)
+    mask = F.one_hot(selected_experts.long(), E).float()  # [T, k, E]
+    tokens_per_expert = mask.mean(dim=0)  # [k, E]
+    prob_per_expert = probs.mean(dim=0)  # [E]
+    return E * torch.sum(tokens_per_expert * prob_per_expert.unsqueeze(0))

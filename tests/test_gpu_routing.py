@@ -168,3 +168,29 @@ def test_sort_empty_experts_zipf_and_golden(device):
         _check_sort(device, ids, 8, 256)
     # all rows to one expert, at the far end
     _check_sort(device, torch.full((5000,), 63, dtype=torch.int32), 64, 128)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("T,E,k", [(16384, 64, 2), (1000, 128, 8), (1, 8, 2)])
+def test_load_balancing_loss_matches_oracle(device, dtype, T, E, k):
+    """cute_kernels.load_balancing_loss (continuous_count_cute + softmax_cute) against the one-hot formulation in the
+    oracle: value and gradient w.r.t. the router logits. fp32 1e-5; bf16: the probabilities are rounded to bf16 before
+    the mean (rtol 1e-2)."""
+    from oracle import moe_oracle as mo
+
+    g = torch.Generator().manual_seed(E + k)
+    logits = torch.randn(T, E, generator=g).to(dtype)
+    sel = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(min(T, 64))])
+    sel = sel.repeat((T + sel.size(0) - 1) // sel.size(0), 1)[:T]
+    lg = logits.clone().to(device).requires_grad_()
+    loss = cute_kernels.load_balancing_loss(lg, sel.to(device))
+    loss.backward()
+    lo = logits.clone().float().requires_grad_()
+    want = mo.load_balancing_loss_torch(lo, sel)
+    want.backward()
+    tol = dict(rtol=1e-5, atol=1e-6) if dtype == torch.float32 else dict(rtol=1e-2, atol=1e-3)
+    torch.testing.assert_close(loss.cpu(), want.detach(), **tol)
+    gtol = dict(rtol=1e-4, atol=1e-7) if dtype == torch.float32 else dict(rtol=5e-2, atol=2e-4 / max(T, 1) + 1e-6)
+    torch.testing.assert_close(lg.grad.float().cpu(), lo.grad, **gtol)
+    f, P = cute_kernels.load_balancing_stats(lg.detach(), sel.to(device))
+    assert abs(float(f.sum()) - k) < 1e-5 and abs(float(P.sum()) - 1.0) < 1e-2

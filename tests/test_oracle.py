@@ -261,3 +261,26 @@ def test_softmax_closed_form_and_jacobian():
         yd = y.detach().double()
         torch.testing.assert_close(gx, m * yd * (dy - (dy * yd).sum(-1, keepdim=True)), rtol=1e-5, atol=1e-6)
     assert mo.softmax_torch(x.detach().to(torch.bfloat16), 0.7).dtype == torch.bfloat16
+
+
+def test_load_balancing_loss_closed_form_and_invariants():
+    """The auxiliary-loss oracle against the formula written with counts (no one-hot): E * sum_e (count_e / T) * P_e; a
+    perfectly balanced router gives k; a dropped factor E, a mean over the wrong axis or probabilities of the selected
+    experts only would each fail one of these."""
+    g = torch.Generator().manual_seed(11)
+    T, E, k = 97, 8, 2
+    logits = torch.randn(T, E, generator=g, dtype=torch.float64)
+    sel = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)])
+    counts = torch.bincount(sel.flatten(), minlength=E).double()
+    e = torch.exp(logits - logits.amax(-1, keepdim=True))
+    P = (e / e.sum(-1, keepdim=True)).mean(0)
+    want = E * torch.sum(counts / T * P)
+    torch.testing.assert_close(mo.load_balancing_loss_torch(logits, sel).double(), want, rtol=1e-6, atol=1e-7)
+    # uniform logits and a round-robin assignment: f_e = k / E, P_e = 1 / E -> loss = k
+    uniform = torch.zeros(96, E)
+    sel_rr = (torch.arange(96 * k).reshape(96, k)) % E
+    assert abs(float(mo.load_balancing_loss_torch(uniform, sel_rr)) - k) < 1e-6
+    # everything routed to one expert that also has all the probability mass: loss = E * k
+    peaked = torch.full((16, E), -1e4)
+    peaked[:, 3] = 0.0
+    assert abs(float(mo.load_balancing_loss_torch(peaked, torch.full((16, k), 3))) - E * k) < 1e-4
