@@ -595,7 +595,8 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
           if (pass == 0) return up;
           if (pass == 1) return gate;
           const float gf = Elem<T>::up(gate);  // from the rounded pre-activation, like the unfused path
-          const T a = Elem<T>::down(Elem<T>::up(up) * gf * sigmoid_fast(gf));
+          const float sg = sigmoid_fast(gf);
+          const T a = Elem<T>::down(prm.act_kind == CK_ACT_GLU ? Elem<T>::up(up) * sg : Elem<T>::up(up) * gf * sg);  // same association as swiglu_fwd_kernel
           return valid ? a : kZero;
         };
         if (tile_full) {
@@ -680,7 +681,8 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
               const T up = Elem<T>::down(acc[i][j][4 * q + s]);
               const T gate = Elem<T>::down(acc[i][j + NI / 2][4 * q + s]);
               const float gf = Elem<T>::up(gate);
-              v[s] = Elem<T>::down(Elem<T>::up(up) * gf * sigmoid_fast(gf));
+              const float sg = sigmoid_fast(gf);
+              v[s] = Elem<T>::down(prm.act_kind == CK_ACT_GLU ? Elem<T>::up(up) * sg : Elem<T>::up(up) * gf * sg);  // same association as swiglu_fwd_kernel
               if (p < valid_end) {
                 pre[p * two_i + col] = up;
                 pre[p * two_i + prm.I + col] = gate;
@@ -782,6 +784,11 @@ extern "C" int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* 
   if (int rc = check_segments(seg, name)) return rc;
   CK_REQUIRE(N >= 8 && K >= 8 && N % 8 == 0 && K % 8 == 0, "%s: N=%d and K=%d must be positive multiples of 8", name, N, K);
   CK_REQUIRE(a_gather_div >= 0, "%s: a_gather_div=%d is negative", name, a_gather_div);
+  int act_kind = CK_ACT_SWIGLU;
+  if (epilogue == CK_EPI_GLU) {  // same tiles and outputs as the SwiGLU epilogue, another gate function
+    act_kind = CK_ACT_GLU;
+    epilogue = CK_EPI_SWIGLU;
+  }
   CK_REQUIRE(epilogue >= CK_EPI_GROUPED && epilogue <= CK_EPI_SWIGLU_BWD, "%s: unknown epilogue %d", name, epilogue);
   if (seg->max_rows == 0) return CK_OK;
   CK_REQUIRE(a && w && y, "%s: a, w and y are required", name);
@@ -801,6 +808,7 @@ extern "C" int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* 
   prm.ldw = K;
   prm.w_expert_stride = (int64_t)N * K;
   prm.a_gather_div = a_gather_div;
+  prm.act_kind = act_kind;
   prm.N = N;
   prm.K = K;
   prm.align = seg->align;

@@ -531,7 +531,8 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
         if (pass == 0) return up;
         if (pass == 1) return gate;
         const float gf = Elem<T>::up(gate);  // from the rounded pre-activation, like the unfused path
-        const T a = Elem<T>::down(Elem<T>::up(up) * gf * sigmoid_fast(gf));
+        const float sg = sigmoid_fast(gf);
+        const T a = Elem<T>::down(prm.act_kind == CK_ACT_GLU ? Elem<T>::up(up) * sg : Elem<T>::up(up) * gf * sg);  // same association as swiglu_fwd_kernel
         return valid ? a : kZero;
       };
       if (tile_full) {

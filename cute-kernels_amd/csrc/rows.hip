@@ -163,7 +163,7 @@ template <typename T>
 __global__ __launch_bounds__(kBlock) void swiglu_bwd_grouped_kernel(
     const T* __restrict__ pre, const T* __restrict__ d_act, int I, const int32_t* __restrict__ seg_starts,
     const uint32_t* __restrict__ counts, const int32_t* __restrict__ tile_expert, int align, T* __restrict__ d_pre,
-    T* __restrict__ d_pre_t, int64_t ld_t) {
+    T* __restrict__ d_pre_t, int64_t ld_t, int act_kind) {
   __shared__ T tile_up[kTile][kTileStride];
   __shared__ T tile_gate[kTile][kTileStride];
   const int64_t p0 = (int64_t)blockIdx.y * kTile;
@@ -190,9 +190,14 @@ __global__ __launch_bounds__(kBlock) void swiglu_bwd_grouped_kernel(
       for (int i = 0; i < 8; ++i) {
         const float gf = Elem<T>::up(g.e[i]), uf = Elem<T>::up(u.e[i]), dyf = Elem<T>::up(dy.e[i]);
         const float sg = sigmoid_for<T>(gf);
-        const float gsg = gf * sg;
-        dg.e[i] = Elem<T>::down(dyf * uf * (sg + gsg * (1.0f - sg)));
-        du.e[i] = Elem<T>::down(dyf * gsg);
+        if (act_kind == CK_ACT_GLU) {  // act = up * sigmoid(gate)
+          dg.e[i] = Elem<T>::down(dyf * uf * sg * (1.0f - sg));
+          du.e[i] = Elem<T>::down(dyf * sg);
+        } else {  // act = up * gate * sigmoid(gate)
+          const float gsg = gf * sg;
+          dg.e[i] = Elem<T>::down(dyf * uf * (sg + gsg * (1.0f - sg)));
+          du.e[i] = Elem<T>::down(dyf * gsg);
+        }
       }
       store16_nt(d_pre + p * two_i + c, du.v);
       store16_nt(d_pre + p * two_i + I + c, dg.v);
@@ -389,9 +394,10 @@ extern "C" int ck_group_rows_padded(const void* src, const void* coeff, int32_t 
 
 extern "C" int ck_swiglu_bwd_grouped(const void* pre, const void* d_act, int32_t I, const int32_t* seg_starts,
                                      const uint32_t* counts, const int32_t* tile_expert, int32_t align,
-                                     int64_t max_rows, void* d_pre, void* d_pre_t, int64_t ld_t, int32_t dtype,
-                                     void* stream) {
+                                     int64_t max_rows, void* d_pre, void* d_pre_t, int64_t ld_t, int32_t act_kind,
+                                     int32_t dtype, void* stream) {
   CK_REQUIRE(I >= 8 && I % 8 == 0, "ck_swiglu_bwd_grouped: I=%d must be a positive multiple of 8", I);
+  CK_REQUIRE(act_kind == CK_ACT_SWIGLU || act_kind == CK_ACT_GLU, "ck_swiglu_bwd_grouped: unknown act_kind %d", act_kind);
   CK_REQUIRE(align >= kTile && align % kTile == 0, "ck_swiglu_bwd_grouped: align=%d must be a multiple of %d", align, kTile);
   CK_REQUIRE(max_rows >= 0 && max_rows % align == 0, "ck_swiglu_bwd_grouped: max_rows=%lld is not a multiple of align",
              (long long)max_rows);
@@ -407,7 +413,8 @@ extern "C" int ck_swiglu_bwd_grouped(const void* pre, const void* d_act, int32_t
   CK_DISPATCH_HALF(dtype, "ck_swiglu_bwd_grouped", {
     hipLaunchKernelGGL((swiglu_bwd_grouped_kernel<scalar_t>), grid, dim3(kBlock), 0, s,
                        static_cast<const scalar_t*>(pre), static_cast<const scalar_t*>(d_act), (int)I, seg_starts, counts,
-                       tile_expert, (int)align, static_cast<scalar_t*>(d_pre), static_cast<scalar_t*>(d_pre_t), ld_t);
+                       tile_expert, (int)align, static_cast<scalar_t*>(d_pre), static_cast<scalar_t*>(d_pre_t), ld_t,
+                       (int)act_kind);
   });
   CK_CHECK_LAUNCH("ck_swiglu_bwd_grouped");
   return CK_OK;

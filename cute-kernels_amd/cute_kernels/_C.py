@@ -18,6 +18,8 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), _LIB_NAME)
 
 CK_F32, CK_F16, CK_BF16 = 0, 1, 2
 CK_EPI_GROUPED, CK_EPI_SCATTER, CK_EPI_SWIGLU, CK_EPI_SWIGLU_BWD = 0, 1, 2, 3
+CK_EPI_GLU = 5
+CK_ACT_SWIGLU, CK_ACT_GLU = 0, 1
 
 _DTYPE_CODES = {torch.float32: CK_F32, torch.float16: CK_F16, torch.bfloat16: CK_BF16}
 
@@ -53,7 +55,7 @@ _SIGNATURES = {
     ),
     "ck_swiglu_bwd_grouped": (
         c_int32,
-        [c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_int64, c_int32, c_void_p],
+        [c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_void_p],
     ),
     "ck_transpose_batched": (c_int32, [c_void_p, c_int64, c_int32, c_int32, c_void_p, c_int32, c_void_p]),
     "ck_grouped_gemm": (

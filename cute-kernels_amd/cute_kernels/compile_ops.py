@@ -371,13 +371,13 @@ def _segments(seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, 
 def swiglu_experts(
     x: Tensor, w_fc: Tensor, w_proj: Tensor, gates: Tensor, seg_starts: Tensor, counts: Tensor, tile_expert: Tensor,
     row_slot: Tensor, max_rows: int, num_experts: int, align: int, need_x: bool, need_fc: bool, need_proj: bool,
-    need_gates: bool,
+    need_gates: bool, act_kind: int,
 ) -> tuple[Tensor, Tensor, Tensor, Tensor]:
     """(out [T, H], pre [max_rows, 2I], the activation for d_w_proj ([I, max_rows] transposed, or [max_rows, I] when the
     weight gradients read row-major operands) or empty, expanded [T * k, H])"""
     ctx = _Ctx((need_x, need_fc, need_proj, need_gates, False))
     seg = _segments(seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, align)
-    out = _moe._SwigluExperts.forward(ctx, x, w_fc, w_proj, gates, seg)
+    out = _moe._SwigluExperts.forward(ctx, x, w_fc, w_proj, gates, seg, act_kind)
     if not ctx.saved_tensors:
         return out, x.new_empty(0), x.new_empty(0), x.new_empty(0)
     pre, act_t, expanded = ctx.saved_tensors[4:]
@@ -386,7 +386,7 @@ def swiglu_experts(
 
 @swiglu_experts.register_fake
 def _(x, w_fc, w_proj, gates, seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, align, need_x, need_fc,
-      need_proj, need_gates):
+      need_proj, need_gates, act_kind):
     T, H = x.shape
     k = gates.shape[1]
     two_i = w_fc.shape[1]
@@ -406,20 +406,21 @@ def _(x, w_fc, w_proj, gates, seg_starts, counts, tile_expert, row_slot, max_row
 def swiglu_experts_backward(
     grad_out: Tensor, x: Tensor, w_fc: Tensor, w_proj: Tensor, gates: Tensor, pre: Tensor, act_t: Tensor, expanded: Tensor,
     seg_starts: Tensor, counts: Tensor, tile_expert: Tensor, row_slot: Tensor, max_rows: int, num_experts: int, align: int,
-    need_x: bool, need_fc: bool, need_proj: bool, need_gates: bool,
+    need_x: bool, need_fc: bool, need_proj: bool, need_gates: bool, act_kind: int,
 ) -> tuple[Tensor, Tensor, Tensor, Tensor]:
     ctx = _Ctx((need_x, need_fc, need_proj, need_gates, False))
+    ctx.act_kind = act_kind
     ctx.seg = _segments(seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, align)
     ctx.saved_tensors = (
         x.contiguous(), w_fc.contiguous(), w_proj.contiguous(), gates.contiguous(), pre, act_t if need_proj else None, expanded,
     )
-    d_x, d_w_fc, d_w_proj, d_gates, _ = _moe._SwigluExperts.backward(ctx, grad_out)
+    d_x, d_w_fc, d_w_proj, d_gates, _, _ = _moe._SwigluExperts.backward(ctx, grad_out)
     return _or_empty(d_x, x), _or_empty(d_w_fc, x), _or_empty(d_w_proj, x), _or_empty(d_gates, x)
 
 
 @swiglu_experts_backward.register_fake
 def _(grad_out, x, w_fc, w_proj, gates, pre, act_t, expanded, seg_starts, counts, tile_expert, row_slot, max_rows,
-      num_experts, align, need_x, need_fc, need_proj, need_gates):
+      num_experts, align, need_x, need_fc, need_proj, need_gates, act_kind):
     e = x.new_empty(0)
     return (
         torch.empty_like(x) if need_x else e,
@@ -437,10 +438,10 @@ def _swiglu_experts_setup(ctx, inputs, output):
 
 
 def _swiglu_experts_bwd(ctx, grad_out, _pre_grad, _act_t_grad, _expanded_grad):
-    need_x, need_fc, need_proj, need_gates = ctx.rest[3:]
+    need_x, need_fc, need_proj, need_gates = ctx.rest[3:7]
     grads = swiglu_experts_backward(grad_out.contiguous(), *ctx.saved_tensors, *ctx.rest)
     needs = (need_x, need_fc, need_proj, need_gates)
-    return tuple(g if n else None for g, n in zip(grads, needs)) + (None,) * 11
+    return tuple(g if n else None for g, n in zip(grads, needs)) + (None,) * 12
 
 
 swiglu_experts.register_autograd(_swiglu_experts_bwd, setup_context=_swiglu_experts_setup)

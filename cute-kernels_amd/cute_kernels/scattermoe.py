@@ -533,7 +533,7 @@ class _SwigluExperts(torch.autograd.Function):
     epilogue and the SwiGLU backward fused into the epilogue of the c_proj input-gradient GEMM."""
 
     @staticmethod
-    def forward(ctx, x, w_fc, w_proj, gates, seg: ExpertSegments):
+    def forward(ctx, x, w_fc, w_proj, gates, seg: ExpertSegments, act_kind: int = _C.CK_ACT_SWIGLU):
         x = x.contiguous()
         w_fc = w_fc.contiguous()
         w_proj = w_proj.contiguous()
@@ -550,7 +550,7 @@ class _SwigluExperts(torch.autograd.Function):
         # d_w_proj needs the activation: transposed (written by the same epilogue) or, in the row-major form, as it is
         rows_form = _dw_from_rows(seg.max_rows, seg.num_experts, seg.align, (H, I), (two_i, H))
         act_t = torch.empty(I, seg.ld_t, dtype=dt, device=dev) if ctx.needs_input_grad[2] and not rows_form else None
-        _gemm(x, k, w_fc, seg, _C.CK_EPI_SWIGLU, pre, y_t=act_t, aux=act)
+        _gemm(x, k, w_fc, seg, _C.CK_EPI_GLU if act_kind == _C.CK_ACT_GLU else _C.CK_EPI_SWIGLU, pre, y_t=act_t, aux=act)
 
         expanded = torch.empty(T * k, H, dtype=dt, device=dev)
         _gemm(act, 0, w_proj, seg, _C.CK_EPI_SCATTER, expanded)
@@ -559,13 +559,13 @@ class _SwigluExperts(torch.autograd.Function):
         if need_grad:
             act_saved = (act if ctx.needs_input_grad[2] else None) if rows_form else act_t
             ctx.save_for_backward(x, w_fc, w_proj, gates, pre, act_saved, expanded)
-        ctx.seg = seg
+        ctx.seg, ctx.act_kind = seg, act_kind
         return out
 
     @staticmethod
     def backward(ctx, grad_out):
         x, w_fc, w_proj, gates, pre, act_saved, expanded = ctx.saved_tensors
-        seg = ctx.seg
+        seg, act_kind = ctx.seg, ctx.act_kind
         T, H = x.shape
         k = gates.size(1)
         E, two_i, _ = w_fc.shape
@@ -602,7 +602,8 @@ class _SwigluExperts(torch.autograd.Function):
                 _C.check(
                     _C.lib().ck_swiglu_bwd_grouped(
                         _C.ptr(pre), _C.ptr(d_act), I, _C.ptr(seg.seg_starts), _C.ptr(seg.counts), _C.ptr(seg.tile_expert),
-                        seg.align, seg.max_rows, _C.ptr(d_pre), _C.ptr(d_pre_t), seg.ld_t, _C.dtype_code(dt), _C.stream(),
+                        seg.align, seg.max_rows, _C.ptr(d_pre), _C.ptr(d_pre_t), seg.ld_t, act_kind, _C.dtype_code(dt),
+                        _C.stream(),
                     )
                 )
             del d_act
@@ -620,13 +621,15 @@ class _SwigluExperts(torch.autograd.Function):
                 d_expanded = torch.empty(T * k, H, dtype=dt, device=dev)
                 _gemm_dx(d_pre, w_fc, seg, _C.CK_EPI_SCATTER, d_expanded)
                 d_x = d_expanded if k == 1 else _combine(d_expanded, None, T, k, H)[0]
-        return d_x, d_w_fc, d_w_proj, d_gates, None
+        return d_x, d_w_fc, d_w_proj, d_gates, None, None
 
 
 def swiglu_experts(
-    x: torch.Tensor, w_fc: torch.Tensor, w_proj: torch.Tensor, gates: torch.Tensor, seg: ExpertSegments
+    x: torch.Tensor, w_fc: torch.Tensor, w_proj: torch.Tensor, gates: torch.Tensor, seg: ExpertSegments,
+    act_kind: int = _C.CK_ACT_SWIGLU,
 ) -> torch.Tensor:
-    """Fused expert block for `activation_function = swiglu_packed_cute`, `is_glu=True` (c_fc columns [up | gate])."""
+    """Fused expert block for `is_glu=True` (c_fc columns [up | gate]) with `activation_function = swiglu_packed_cute`
+    (act_kind CK_ACT_SWIGLU: up * silu(gate)) or `torch.nn.GLU()` (CK_ACT_GLU: up * sigmoid(gate))."""
     _check_expert_dtypes(x, w_fc, w_proj)
     assert w_fc.size(1) % 16 == 0, "intermediate size should be a multiple of 8"
     if is_tracing():
@@ -634,7 +637,7 @@ def swiglu_experts(
         return _ops.swiglu_experts(
             x, w_fc, w_proj, gates.to(x.dtype), seg.seg_starts, seg.counts, seg.tile_expert, seg.row_slot, seg.max_rows,
             seg.num_experts, seg.align, grad and x.requires_grad, grad and w_fc.requires_grad,
-            grad and w_proj.requires_grad, grad and gates.requires_grad,
+            grad and w_proj.requires_grad, grad and gates.requires_grad, act_kind,
         )[0]
     _C.require_gpu(x, w_fc, w_proj, gates)
-    return _SwigluExperts.apply(x, w_fc, w_proj, gates.to(x.dtype), seg)
+    return _SwigluExperts.apply(x, w_fc, w_proj, gates.to(x.dtype), seg, act_kind)

@@ -118,10 +118,12 @@ int ck_group_rows_padded(const void* src, const void* coeff, int32_t fan_out, in
 /* SwiGLU backward over padded grouped rows (formula: cute_kernels/kernels/swiglu/cuda_implementation/backward.cu:27-41),
  * writing what the weight-gradient GEMM consumes in the same pass:
  *   pre [max_rows, 2I] packed [up | gate], d_act [max_rows, I]  ->  d_pre [max_rows, 2I] (valid rows only) and
- *   d_pre_t [2I, ld_t] = d_pre^T with zeros in the pad rows of live tiles (may be NULL). I % 8 == 0. 16-bit dtypes. */
+ *   d_pre_t [2I, ld_t] = d_pre^T with zeros in the pad rows of live tiles (may be NULL). I % 8 == 0. 16-bit dtypes.
+ * act_kind: CK_ACT_SWIGLU (act = up * gate * sigmoid(gate)) or CK_ACT_GLU (act = up * sigmoid(gate), torch.nn.GLU on the
+ * packed tensor: the activation of the reference's own MoE test, tests/test_commons.py:85). */
 int ck_swiglu_bwd_grouped(const void* pre, const void* d_act, int32_t I, const int32_t* seg_starts,
                           const uint32_t* counts, const int32_t* tile_expert, int32_t align, int64_t max_rows,
-                          void* d_pre, void* d_pre_t, int64_t ld_t, int32_t dtype, void* stream);
+                          void* d_pre, void* d_pre_t, int64_t ld_t, int32_t act_kind, int32_t dtype, void* stream);
 /* Batched 2-D transpose: dst[b, c, r] = src[b, r, c]; src [batch, rows, cols]. 16-bit dtypes only. */
 int ck_transpose_batched(const void* src, int64_t batch, int32_t rows, int32_t cols, void* dst, int32_t dtype,
                          void* stream);
@@ -163,6 +165,9 @@ typedef struct ck_segments {
 #define CK_EPI_SCATTER 1
 #define CK_EPI_SWIGLU 2
 #define CK_EPI_SWIGLU_BWD 3
+#define CK_EPI_GLU 5 /* as CK_EPI_SWIGLU with act = up * sigmoid(gate): torch.nn.GLU() on the packed c_fc output */
+#define CK_ACT_SWIGLU 0
+#define CK_ACT_GLU 1
 int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* w, int32_t N, int32_t K,
                     const ck_segments* seg, int32_t epilogue, void* y, void* y_t, int64_t ld_t, void* aux,
                     const void* aux_in, int32_t dtype, void* stream);

@@ -124,20 +124,25 @@ def test_grouped_gemm_input_gradient_form(device, dtype, epilogue, n_out, n_in):
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("align", [128, 256])
 @pytest.mark.parametrize("K,I", [(200, 72), (128, 256), (64, 136), (96, 440), (192, 440)])
-def test_grouped_gemm_swiglu_epilogues(device, dtype, align, K, I, gemm_tile):
+@pytest.mark.parametrize("kind", ["swiglu", "glu"])
+def test_grouped_gemm_swiglu_epilogues(device, dtype, align, K, I, gemm_tile, kind):
+    """Gated-activation epilogues of the c_fc GEMM: packed SwiGLU (up * silu(gate)) and torch.nn.GLU (up * sigmoid(gate),
+    the activation of the reference's MoE test, tests/test_commons.py:85), forward and both backward forms."""
     T, k, E = 300, 2, 5
+    glu = kind == "glu"
+    act_fn = (lambda t: F.glu(t, dim=-1)) if glu else mo.swiglu_packed_torch
     g, seg = _make_case(device, dtype, T, k, E, align, seed=2)
     x = torch.randn(T, K, generator=g).to(dtype)
     w = (0.1 * torch.randn(E, 2 * I, K, generator=g)).to(dtype)
     pre = torch.zeros(seg.max_rows, 2 * I, dtype=dtype, device=device)
     act = torch.zeros(seg.max_rows, I, dtype=dtype, device=device)
     act_t = torch.full((I, seg.ld_t), 7.0, dtype=dtype, device=device)
-    scattermoe._gemm(x.to(device), k, w.to(device), seg, _C.CK_EPI_SWIGLU, pre, y_t=act_t, aux=act)
+    scattermoe._gemm(x.to(device), k, w.to(device), seg, _C.CK_EPI_GLU if glu else _C.CK_EPI_SWIGLU, pre, y_t=act_t, aux=act)
     live = int(seg.seg_starts[E])
     expect_pre = _expected_grouped(lambda p, slot: x[slot // k], w, seg, 2 * I)
     torch.testing.assert_close(pre.float().cpu()[:live], expect_pre[:live], rtol=RTOL, atol=ATOL)
     # the activation is computed from the ROUNDED pre-activation, like the unfused path
-    expect_act = mo.swiglu_packed_torch(pre.cpu())
+    expect_act = act_fn(pre.cpu().float()).to(dtype)
     torch.testing.assert_close(act.cpu()[:live], expect_act[:live], rtol=RTOL, atol=1e-3)
     assert torch.equal(act_t.cpu()[:, :live], act.cpu()[:live].t())
 
@@ -147,16 +152,17 @@ def test_grouped_gemm_swiglu_epilogues(device, dtype, align, K, I, gemm_tile):
     w_proj_t = (0.1 * torch.randn(E, I, H, generator=g)).to(dtype)  # [E, I, H]: d_act = d_y @ w_proj
     d_pre = torch.zeros(seg.max_rows, 2 * I, dtype=dtype, device=device)
     d_pre_t = torch.full((2 * I, seg.ld_t), 7.0, dtype=dtype, device=device)
-    scattermoe._gemm(d_y.to(device), 0, w_proj_t.to(device), seg, _C.CK_EPI_SWIGLU_BWD, d_pre, y_t=d_pre_t, aux_in=pre)
     d_act = _expected_grouped(lambda p, slot: d_y[p], w_proj_t, seg, I).to(dtype)
     pre_c = pre.cpu().float().requires_grad_()
-    mo.swiglu_packed_torch(pre_c).backward(d_act.float())
+    act_fn(pre_c).backward(d_act.float())
     seg_starts, counts, _ = _layout(seg)
     valid = torch.zeros(seg.max_rows, dtype=torch.bool)
     for e in range(E):
         valid[int(seg_starts[e]) : int(seg_starts[e]) + int(counts[e])] = True
-    torch.testing.assert_close(d_pre.float().cpu()[valid], pre_c.grad[valid], rtol=2e-2, atol=2e-2)
-    assert torch.equal(d_pre_t.cpu()[:, :live], (d_pre.cpu()[:live] * valid[:live, None]).t())
+    if not glu:  # the fused backward epilogue exists for SwiGLU only
+        scattermoe._gemm(d_y.to(device), 0, w_proj_t.to(device), seg, _C.CK_EPI_SWIGLU_BWD, d_pre, y_t=d_pre_t, aux_in=pre)
+        torch.testing.assert_close(d_pre.float().cpu()[valid], pre_c.grad[valid], rtol=2e-2, atol=2e-2)
+        assert torch.equal(d_pre_t.cpu()[:, :live], (d_pre.cpu()[:live] * valid[:live, None]).t())
 
     # the same backward as a plain GEMM followed by the streaming SwiGLU-backward pass (what the layer uses)
     d_act_gpu = torch.zeros(seg.max_rows, I, dtype=dtype, device=device)
@@ -167,7 +173,7 @@ def test_grouped_gemm_swiglu_epilogues(device, dtype, align, K, I, gemm_tile):
         _C.lib().ck_swiglu_bwd_grouped(
             pre.data_ptr(), d_act_gpu.data_ptr(), I, seg.seg_starts.data_ptr(), seg.counts.data_ptr(),
             seg.tile_expert.data_ptr(), seg.align, seg.max_rows, d_pre2.data_ptr(), d_pre2_t.data_ptr(), seg.ld_t,
-            _C.dtype_code(dtype), torch.cuda.current_stream().cuda_stream,
+            _C.CK_ACT_GLU if glu else _C.CK_ACT_SWIGLU, _C.dtype_code(dtype), torch.cuda.current_stream().cuda_stream,
         )
     )
     torch.testing.assert_close(d_pre2.float().cpu()[valid], pre_c.grad[valid], rtol=2e-2, atol=2e-2)
@@ -469,3 +475,18 @@ def test_moe_layer_at_full_baseline_shapes(device, name, T, E, k, H, I, skew):
     _close_via_truth_on_device(
         moe.gate.weight.grad, oracle.gate.weight.grad, truth.gate.weight.grad, f"{name} gate.weight.grad", atol=3e-2 + floor
     )
+
+
+@pytest.mark.parametrize("act,kind", [("swiglu", _C.CK_ACT_SWIGLU), ("glu", _C.CK_ACT_GLU), ("gelu", None)])
+def test_gated_activations_take_the_fused_expert_block(device, monkeypatch, act, kind):
+    """Packed SwiGLU and torch.nn.GLU run inside the c_fc epilogue (swiglu_experts with the matching act_kind); any other
+    callable goes GEMM -> callable -> GEMM. Results of both routes are covered by the layer parity tests above."""
+    from cute_kernels.modules import moe as moe_module
+
+    act_gpu, _, is_glu = _acts(act)
+    layer = cute_kernels.MoE(4, 2, 128, 256, act_gpu, is_glu, False, 0.02).to(torch.bfloat16).to(device)
+    seen = []
+    real = moe_module.swiglu_experts
+    monkeypatch.setattr(moe_module, "swiglu_experts", lambda *a: (seen.append(a[5]), real(*a))[1])
+    layer(torch.randn(300, 128, device=device, dtype=torch.bfloat16))
+    assert seen == ([kind] if kind is not None else [])
