@@ -52,6 +52,22 @@ int launch_line(const GemmParams& prm, int mode, int bn, bool bt, int dtype, uns
 
 namespace {
 
+// The dynamic-LDS limit of a kernel is a per-device attribute: set it once per (instantiation, device). `done` is the
+// instantiation's own table; the call is idempotent, so a race between host threads only repeats it.
+constexpr int kMaxDevices = 64;
+inline int reserve_lds(const void* kernel, size_t bytes, bool (&done)[kMaxDevices], const char* name) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) dev = -1;
+  if (dev >= 0 && done[dev]) return CK_OK;
+  hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+  if (e != hipSuccess) {
+    set_error("%s: cannot reserve %zu bytes of LDS: %s", name, bytes, hipGetErrorString(e));
+    return CK_ERR_LAUNCH;
+  }
+  if (dev >= 0) done[dev] = true;
+  return CK_OK;
+}
+
 template <typename T>
 struct Mfma;
 template <>

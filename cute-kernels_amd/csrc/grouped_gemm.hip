@@ -738,16 +738,8 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
 template <typename T, int BM, int BN, int MODE, int PIPE, int WGM>
 int launch_pipe(const GemmParams& prm, unsigned blocks, hipStream_t s, const char* name) {
   auto kernel = grouped_gemm_kernel<T, BM, BN, MODE, PIPE, WGM>;
-  static bool attr_set = false;  // per instantiation; the attribute is idempotent, a race only repeats the call
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)lds_bytes<BM, BN, PIPE>());
-    if (e != hipSuccess) {
-      set_error("%s: cannot reserve %zu bytes of LDS: %s", name, lds_bytes<BM, BN, PIPE>(), hipGetErrorString(e));
-      return CK_ERR_LAUNCH;
-    }
-    attr_set = true;
-  }
+  static bool lds_reserved[kMaxDevices] = {};
+  if (int rc = reserve_lds(reinterpret_cast<const void*>(kernel), lds_bytes<BM, BN, PIPE>(), lds_reserved, name)) return rc;
   constexpr size_t kLds = lds_bytes<BM, BN, PIPE>();
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(64 * WGM * 2), kLds, s, prm);
   CK_CHECK_LAUNCH(name);

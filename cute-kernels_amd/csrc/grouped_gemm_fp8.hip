@@ -346,16 +346,8 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
 template <typename TO, int MODE>
 int launch_fp8(const GemmParams& prm, unsigned blocks, hipStream_t s, const char* name) {
   auto kernel = grouped_gemm_fp8_kernel<TO, MODE>;
-  static bool attr_set = false;
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)kLdsBytes);
-    if (e != hipSuccess) {
-      set_error("%s: cannot reserve %zu bytes of LDS: %s", name, kLdsBytes, hipGetErrorString(e));
-      return CK_ERR_LAUNCH;
-    }
-    attr_set = true;
-  }
+  static bool lds_reserved[kMaxDevices] = {};
+  if (int rc = reserve_lds(reinterpret_cast<const void*>(kernel), kLdsBytes, lds_reserved, name)) return rc;
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(NT), kLdsBytes, s, prm);
   CK_CHECK_LAUNCH(name);
   return CK_OK;

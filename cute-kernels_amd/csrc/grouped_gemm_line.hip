@@ -568,16 +568,8 @@ template <typename T, int MODE, int BN, bool BT>
 int launch_mode(const GemmParams& prm, unsigned blocks, hipStream_t s, const char* name) {
   auto kernel = grouped_gemm_line_kernel<T, MODE, BN, BT>;
   constexpr size_t kLds = Tile<BN>::kLdsBytes;
-  static bool attr_set = false;  // per instantiation; the attribute is idempotent, a race only repeats the call
-  if (!attr_set) {
-    hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                                       (int)kLds);
-    if (e != hipSuccess) {
-      set_error("%s: cannot reserve %zu bytes of LDS: %s", name, kLds, hipGetErrorString(e));
-      return CK_ERR_LAUNCH;
-    }
-    attr_set = true;
-  }
+  static bool lds_reserved[kMaxDevices] = {};
+  if (int rc = reserve_lds(reinterpret_cast<const void*>(kernel), kLds, lds_reserved, name)) return rc;
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(NT), kLds, s, prm);
   CK_CHECK_LAUNCH(name);
   return CK_OK;
