@@ -791,7 +791,10 @@ extern "C" int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* 
 
   // rows are addressed with 32-bit byte offsets: from the operand base for a, from the expert's slice for w
   CK_REQUIRE((int64_t)N * K * 2 < ((int64_t)1 << 32), "%s: one expert's weight matrix must stay below 4 GiB", name);
-  CK_REQUIRE(a_gather_div > 0 || seg->max_rows * (int64_t)K * 2 < ((int64_t)1 << 32),
+  const bool line_kernel = seg->align == kLineBM && K % kLineK == 0 && epilogue != CK_EPI_SWIGLU_BWD && !g_force_pipe0 &&
+                           line_kernel_enabled();
+  // the 128-byte-row kernel addresses a grouped input from each tile's first row; the general kernel from the operand base
+  CK_REQUIRE(a_gather_div > 0 || line_kernel || seg->max_rows * (int64_t)K * 2 < ((int64_t)1 << 32),
              "%s: the grouped input must stay below 4 GiB", name);
   GemmParams prm = {};
   prm.a = a;
@@ -830,7 +833,7 @@ extern "C" int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* 
   hipStream_t s = static_cast<hipStream_t>(stream);
   // kSwiglu tiles cover BN/2 activation columns each
   auto n_tiles_for = [&](int bn) { return (int)ceil_div(out_cols, epilogue == CK_EPI_SWIGLU ? bn / 2 : bn); };
-  if (seg->align == kLineBM && K % kLineK == 0 && epilogue != CK_EPI_SWIGLU_BWD && !g_force_pipe0 && line_kernel_enabled()) {
+  if (line_kernel) {
     const bool swiglu = epilogue == CK_EPI_SWIGLU;
     const int bn = epilogue == CK_EPI_SCATTER ? line_tile_width(out_cols, 256, 384, K >= 8192 ? K : 0)
                                               : (forced_tile() == 384 ? 384 : 256);
@@ -868,8 +871,7 @@ extern "C" int ck_grouped_gemm_nn(const void* a, const void* w, int32_t N, int32
              epilogue);
   if (seg->max_rows == 0) return CK_OK;
   CK_REQUIRE(a && w && y && aligned16(a) && aligned16(w), "%s: NULL or misaligned pointer", name);
-  CK_REQUIRE((int64_t)N * K * 2 < ((int64_t)1 << 32) && seg->max_rows * (int64_t)K * 2 < ((int64_t)1 << 32),
-             "%s: one expert's weight matrix and the grouped input must each stay below 4 GiB", name);
+  CK_REQUIRE((int64_t)N * K * 2 < ((int64_t)1 << 32), "%s: one expert's weight matrix must stay below 4 GiB", name);
   GemmParams prm = {};
   prm.a = a;
   prm.w = w;

@@ -131,6 +131,9 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
     a_base += k_begin * prm.lda * 2;
     b_base += k_begin * prm.ldw * 2;
   }
+  if constexpr (MODE != kDw) {
+    if (prm.a_gather_div <= 0) a_base += m0 * prm.lda * 2;
+  }
   constexpr int kAtRowBytes = BM * 2;
   auto swap02 = [](int w) { return (w & ~5) | ((w & 1) << 2) | ((w >> 2) & 1); };
   uint32_t a_off[A_LD], b_off[B_LD];
@@ -152,7 +155,9 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
       } else {
         int64_t p = m0 + r;
         if (p >= valid_end) p = valid_end - 1;  // pad rows re-read a valid row; their results are never stored
-        row = prm.a_gather_div > 0 ? (int64_t)(prm.row_slot[p] / prm.a_gather_div) : p;
+        // grouped input: offsets are taken from the tile's first row (a_base is moved there below), so that only a tile,
+        // not the whole operand, has to fit 32-bit offsets; gathered input: from the start of the token-order tensor
+        row = prm.a_gather_div > 0 ? (int64_t)(prm.row_slot[p] / prm.a_gather_div) : p - m0;
       }
       a_off[t] = (uint32_t)((row * prm.lda + k_begin) * 2 + c * 16);
     }

@@ -213,6 +213,9 @@ _EPILOGUE_NAMES = {
 def _gemm(a, gather_div, w, seg: ExpertSegments, epilogue, y, y_t=None, aux=None, aux_in=None):
     E, N, K = w.shape
     cs = seg.c_struct()
+    if gather_div > 0:  # gathered rows are addressed with 32-bit byte offsets from the start of `a` (the library is not
+        # told how many rows `a` has, so this limit is checked here)
+        assert a.numel() * a.element_size() < 2**32, "the token-order input of a grouped GEMM must stay below 4 GiB"
 
     def launch():
         with torch.cuda.device(w.device):

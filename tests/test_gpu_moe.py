@@ -229,6 +229,33 @@ def test_grouped_gemm_dw_from_row_major_operands(device, dtype, align, M, N, T):
     assert float(dw[3].abs().max()) == 0.0  # empty expert: exact zeros (ops.py:252, kernels.py:181)
 
 
+def test_grouped_gemm_grouped_input_beyond_4_gib(device):
+    """A padded-grouped input of 4.9 GB (600,000 rows x 4,096 bf16): rows are addressed from each tile's first row, so the
+    32-bit offsets inside the kernels never see the size of the whole operand. Checked on the last rows of the last expert
+    (byte offsets past 2^32) and on the first rows, for the forward form and the input-gradient form, against torch's
+    GEMM on the same device."""
+    torch.manual_seed(5)
+    R, E, K, N = 600_000, 2, 4096, 256
+    ids = (torch.arange(R, dtype=torch.int32) >= 250_000).to(torch.int32)  # expert 0: 250,000 rows, expert 1: 350,000
+    seg = cute_kernels.sort_by_expert(ids.to(device), E, 256)
+    assert seg.max_rows * K * 2 > 2**32
+    a = torch.randn(seg.max_rows, K, device=device, dtype=torch.bfloat16)
+    w = (0.05 * torch.randn(E, N, K, device=device)).to(torch.bfloat16)
+    y = torch.zeros(seg.max_rows, N, dtype=torch.bfloat16, device=device)
+    scattermoe._gemm(a, 0, w, seg, _C.CK_EPI_GROUPED, y)
+    seg_starts, counts, _ = _layout(seg)
+    last = int(seg_starts[1]) + int(counts[1])
+    for lo, hi, e in ((0, 512, 0), (last - 1000, last, 1)):
+        want = a[lo:hi].float() @ w[e].float().t()
+        torch.testing.assert_close(y[lo:hi].float(), want, rtol=RTOL, atol=2e-2)
+    # input-gradient form: x = a @ w_nn[e] with w_nn [E, K, N2] read as stored
+    w_nn = (0.05 * torch.randn(E, K, 512, device=device)).to(torch.bfloat16)
+    y2 = torch.zeros(seg.max_rows, 512, dtype=torch.bfloat16, device=device)
+    scattermoe._gemm_dx(a, w_nn, seg, _C.CK_EPI_GROUPED, y2)
+    want = a[last - 1000 : last].float() @ w_nn[1].float()
+    torch.testing.assert_close(y2[last - 1000 : last].float(), want, rtol=RTOL, atol=2e-2)
+
+
 # ---------------------------------------------------------------------------------------------------------------
 # whole layer
 # ---------------------------------------------------------------------------------------------------------------
