@@ -833,6 +833,9 @@ extern "C" int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* 
   hipStream_t s = static_cast<hipStream_t>(stream);
   // kSwiglu tiles cover BN/2 activation columns each
   auto n_tiles_for = [&](int bn) { return (int)ceil_div(out_cols, epilogue == CK_EPI_SWIGLU ? bn / 2 : bn); };
+  CK_REQUIRE(aux_in == nullptr || epilogue == CK_EPI_SWIGLU_BWD || (line_kernel && epilogue != CK_EPI_SWIGLU),
+             "%s: the bias operand (aux_in) goes with the grouped / scatter epilogues of the 256-row-tile kernel "
+             "(align = 256, K %% 64 == 0)", name);
   if (line_kernel) {
     const bool swiglu = epilogue == CK_EPI_SWIGLU;
     const int bn = epilogue == CK_EPI_SCATTER ? line_tile_width(out_cols, 256, 384, K >= 8192 ? K : 0)

@@ -494,6 +494,22 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
   } else if constexpr (MODE == kGrouped || MODE == kScatter) {
     T* y = static_cast<T*>(prm.y);
     T* y_t = static_cast<T*>(prm.y_t);
+    // optional per-expert bias row (aux_in = bias [E, N]): added to the fp32 accumulators, so that the output is rounded
+    // once, like F.linear with a bias. A lane's accumulators of one column block all belong to one output column.
+    if constexpr (!BT) {
+      if (prm.aux_in != nullptr) {
+        const T* bias = static_cast<const T*>(prm.aux_in) + (int64_t)expert * prm.N;
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {
+          const int64_t n = (int64_t)nt * BN + wn * WN + j * 32 + col_in_block;
+          const float b = n < prm.N ? Elem<T>::up(bias[n]) : 0.f;
+#pragma unroll
+          for (int i = 0; i < MI; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] += b;
+        }
+      }
+    }
     static_for<2>([&](auto pass) {
       // pad rows are staged as zeros: the transposed copy must hold zeros there
       if (tile_full) {

@@ -232,6 +232,18 @@ def _gemm(a, gather_div, w, seg: ExpertSegments, epilogue, y, y_t=None, aux=None
         launch_timer.time(_EPILOGUE_NAMES[epilogue], (N, K), launch)
 
 
+def _bias_in_epilogue(seg: ExpertSegments, K: int) -> bool:
+    """Whether ck_grouped_gemm takes the per-expert bias as an operand of its grouped / scatter epilogue (the
+    256-row-tile kernel: the bias joins the fp32 accumulators and the output is rounded once, like F.linear); otherwise
+    the bias is added by its own kernel after the GEMM."""
+    import os
+
+    return (
+        seg.align == 256 and K % 64 == 0 and os.environ.get("CK_GEMM_LINE", "1") != "0"
+        and os.environ.get("CK_GEMM_PIPE", "1") != "0" and os.environ.get("CK_GEMM_BIAS_FUSED", "1") != "0"
+    )
+
+
 def _gemm_dx(d_y, w, seg: ExpertSegments, epilogue, out):
     """out = d_y @ w[e] per expert, w [E, out_features, in_features] as the forward stores it: the input-gradient GEMM.
     Reads w contraction-strided where the kernel for that exists (256-row tiles, out_features % 64 == 0); otherwise
@@ -420,8 +432,9 @@ class _ExpertsUp(torch.autograd.Function):
         E, N, K = w.shape
         # pad rows are never written by the kernel; zeros keep any activation applied on top finite
         y = torch.zeros(seg.max_rows, N, dtype=x.dtype, device=x.device)
-        _gemm(x, k, w, seg, _C.CK_EPI_GROUPED, y)
-        if bias is not None:
+        fused_bias = bias is not None and _bias_in_epilogue(seg, K)
+        _gemm(x, k, w, seg, _C.CK_EPI_GROUPED, y, aux_in=bias.contiguous() if fused_bias else None)
+        if bias is not None and not fused_bias:
             _add_expert_bias(y, bias.contiguous(), seg, None)
         ctx.save_for_backward(x, w)
         ctx.seg, ctx.k = seg, k
@@ -463,8 +476,9 @@ class _ExpertsDown(torch.autograd.Function):
         T, k = gates.shape
         E, N, K = w.shape
         expanded = torch.empty(T * k, N, dtype=h.dtype, device=h.device)
-        _gemm(h, 0, w, seg, _C.CK_EPI_SCATTER, expanded)
-        if bias is not None:  # before the gate multiply, as torch_implementation.py:160-163
+        fused_bias = bias is not None and _bias_in_epilogue(seg, K)
+        _gemm(h, 0, w, seg, _C.CK_EPI_SCATTER, expanded, aux_in=bias.contiguous() if fused_bias else None)
+        if bias is not None and not fused_bias:  # before the gate multiply, as torch_implementation.py:160-163
             _add_expert_bias(expanded, bias.contiguous(), seg, slot_expert if slot_expert is not None else _slot_experts(seg))
         out, _ = _combine(expanded, gates, T, k, N)
         ctx.save_for_backward(h, w, gates, expanded)

@@ -153,6 +153,9 @@ typedef struct ck_segments {
  *   CK_EPI_GROUPED        : y [max_rows, N] padded-grouped (valid rows only); y_t [N, ld_t] transposed copy with
  *                           zeros in pad rows, optional (NULL to skip)
  *   CK_EPI_SCATTER        : y [R, N]: valid row p is written to row row_slot[p] (back to (token, slot) order)
+ *                           both: aux_in, if not NULL, is a bias [E, N] whose row e joins the fp32 accumulators of expert
+ *                           e's rows before the one rounding (F.linear with a bias, torch_implementation.py:42); needs
+ *                           seg->align == 256 and K % 64 == 0 (ck_add_expert_bias covers the other cases)
  *   CK_EPI_SWIGLU         : N = 2*I packed [up | gate] (cute_kernels/kernels/swiglu/__init__.py:121): writes the
  *                           pre-activation to y [max_rows, 2I], act = up*silu(gate) (computed from the rounded
  *                           pre-activation, as the unfused path would) to aux [max_rows, I], and act^T to

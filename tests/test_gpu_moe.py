@@ -384,10 +384,12 @@ def test_moe_layer_3d_input_top1_and_large_tiles(device):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("act", ["swiglu", "glu", "gelu"])
-@pytest.mark.parametrize("T,E,k,H,I", [(257, 8, 2, 128, 256), (33, 4, 4, 64, 72), (700, 64, 8, 128, 136)])
+@pytest.mark.parametrize("T,E,k,H,I", [(257, 8, 2, 128, 256), (33, 4, 4, 64, 72), (700, 64, 8, 128, 136), (3000, 4, 2, 128, 256)])
 def test_moe_layer_with_expert_biases(device, dtype, act, T, E, k, H, I):
     # add_bias=True: the reference's torch path applies one bias row per expert (torch_implementation.py:20-22,42); its
-    # Triton path drops them, so the reference's own test only runs add_bias=False (scattermoe_test.py:62-77)
+    # Triton path drops them, so the reference's own test only runs add_bias=False (scattermoe_test.py:62-77).
+    # The last shape has 256-row tiles and contraction lengths that are multiples of 64: there the bias is an operand of
+    # the GEMM epilogues; the others add it with its own kernel.
     _run_layer_case(device, dtype, T, E, k, H, I, act, add_bias=True)
 
 
@@ -517,3 +519,26 @@ def test_gated_activations_take_the_fused_expert_block(device, monkeypatch, act,
     monkeypatch.setattr(moe_module, "swiglu_experts", lambda *a: (seen.append(a[5]), real(*a))[1])
     layer(torch.randn(300, 128, device=device, dtype=torch.bfloat16))
     assert seen == ([kind] if kind is not None else [])
+
+
+def test_bias_in_the_gemm_epilogue_equals_the_separate_bias_kernel(device, monkeypatch):
+    """Same layer, same input, biases on: the epilogue form (one rounding of accumulator + bias) against the GEMM followed
+    by ck_add_expert_bias (two roundings): equal within one bf16 rounding step of the outputs, forward and gradients."""
+    torch.manual_seed(1)
+    layer = cute_kernels.MoE(4, 2, 128, 256, nn.GELU(approximate="tanh"), False, True, 0.02).to(torch.bfloat16).to(device)
+    with torch.no_grad():
+        layer.c_fc.bias.normal_(0, 0.2)
+        layer.c_proj.bias.normal_(0, 0.2)
+    x = torch.randn(3000, 128, device=device, dtype=torch.bfloat16)
+    results = []
+    for fused in ("1", "0"):
+        monkeypatch.setenv("CK_GEMM_BIAS_FUSED", fused)
+        for p in layer.parameters():
+            p.grad = None
+        xi = x.clone().requires_grad_()
+        y, _ = layer(xi)
+        y.float().square().sum().backward()
+        results.append((y.detach(), xi.grad, layer.c_fc.bias.grad.clone(), layer.c_proj.bias.grad.clone()))
+    for a, b in zip(*results):
+        torch.testing.assert_close(a.float(), b.float(), rtol=2e-2, atol=2e-2 * max(1.0, float(b.float().abs().max()) / 8))
+    assert not torch.equal(results[0][0], results[1][0])  # the two forms really differ in rounding: both paths ran
