@@ -518,6 +518,7 @@ def experts_up(
 ) -> torch.Tensor:
     """x [T, H] -> c_fc output in padded grouped order [max_rows, N] (+ bias[e] on expert e's rows)."""
     _check_expert_dtypes(x, weight)
+    assert bias is None or (bias.dtype == x.dtype and bias.shape == weight.shape[:2]), "bias should be [E, out] in x.dtype"
     if is_tracing():
         return _ops.experts_up(
             x, weight, bias, seg.seg_starts, seg.counts, seg.tile_expert, seg.row_slot, seg.max_rows, seg.num_experts,
@@ -532,6 +533,7 @@ def experts_down(
 ) -> torch.Tensor:
     """h [max_rows, I] (padded grouped) -> sum_k gates * (c_proj output + bias[e]) in token order [T, N]."""
     _check_expert_dtypes(h, weight)
+    assert bias is None or (bias.dtype == h.dtype and bias.shape == weight.shape[:2]), "bias should be [E, out] in h.dtype"
     if is_tracing():
         slot_expert = _slot_experts(seg) if bias is not None else None
         return _ops.experts_down(
