@@ -271,27 +271,43 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
       });
     });
   };
-  auto drain_rows = [&](auto&& out_ptr) {
-    const int l16 = tid & 15, grp = tid >> 4;
+  // Row-major drain as in the 16-bit kernel: 16 lanes take a 4-row x 32-column block, the four lane groups of a wave two
+  // adjacent column blocks of two adjacent row blocks (whole 128-byte lines per store instruction); rows and column pairs
+  // are walked in unrolled loops, so every address is a per-lane base plus a compile-time offset. row_ptr(tile row) ->
+  // address of the output row at the tile's first column (nullptr: pad row), block_col(cb) -> output column of slab
+  // column block cb relative to that, cols_left = valid columns from there on, tile_cols = columns the tile spans.
+  auto drain_rows = [&](auto&& row_ptr, auto&& block_col, int64_t cols_left, int tile_cols) {
+    const int l16 = tid & 15, csel = (tid >> 4) & 1, rsel = (tid >> 5) & 1;
     const int tq = l16 & 3, tj = l16 >> 2;
     const int oq = l16 >> 2, oe = l16 & 3;
-    constexpr int kBlocks = (BM / 4) * (kSlabCols / 32);
-#pragma unroll 4
-    for (int b = grp; b < kBlocks; b += NT / 16) {
-      const int rb = b >> 2, cb = b & 3;
-      const TO* src = slab + (cb * 32 + 8 * tq + tj) * kSlabLd + rb * 4;
-      const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(src));
-      const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(src + 4 * kSlabLd));
-      TO* dst = out_ptr(rb * 4 + oe, cb * 32 + 8 * oq);
-      if (dst != nullptr) {
-        vec16 v;
-        v.w[0] = (uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
-        v.w[1] = (uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
-        v.w[2] = (uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
-        v.w[3] = (uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16);
-        store16_nt(dst, v);
-      }
-    }
+    constexpr int kColPairs = kSlabCols / 64, kRowIters = (BM / 4) / (2 * NT / kWave);
+    static_assert(kSlabCols % 64 == 0 && (BM / 4) % (2 * NT / kWave) == 0, "whole column pairs and row iterations");
+    const bool cols_full = cols_left >= tile_cols;
+    auto body = [&](auto checked) {
+      static_for<kRowIters>([&](auto it) {
+        const int rb = (it * (NT / kWave) + wave) * 2 + rsel;
+        TO* dst_row = row_ptr(rb * 4 + oe);
+        if (dst_row != nullptr) dst_row += 8 * oq;
+        const TO* src_row = slab + (csel * 32 + 8 * tq + tj) * kSlabLd + rb * 4;
+        static_for<kColPairs>([&](auto cp) {
+          const TO* src = src_row + cp * 64 * kSlabLd;
+          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(src));
+          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(src + 4 * kSlabLd));
+          const int col = csel ? block_col(std::integral_constant<int, 2 * decltype(cp)::value + 1>{})
+                               : block_col(std::integral_constant<int, 2 * decltype(cp)::value>{});
+          if (dst_row != nullptr && (!checked || col + 8 * oq < cols_left)) {
+            vec16 v;
+            v.w[0] = (uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
+            v.w[1] = (uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
+            v.w[2] = (uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
+            v.w[3] = (uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16);
+            store16_nt(dst_row + col, v);
+          }
+        });
+      });
+    };
+    if (cols_full) body(std::false_type{});
+    else body(std::true_type{});
   };
   const float* w_sc = meta_f + BM;
 
@@ -309,13 +325,14 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
       });
       __syncthreads();
       if constexpr (pass == 0) stamp(6);
-      drain_rows([&](int r, int sc) -> TO* {
-        const int64_t n = (int64_t)nt * BN + (sc >> 6) * WN + pass * 64 + (sc & 63);
-        const int out_row = meta_rows[r];
-        if (out_row < 0 || n >= prm.N) return nullptr;
-        const int64_t row = (MODE == kScatter) ? (int64_t)out_row : m0 + r;
-        return y + row * prm.N + n;
-      });
+      drain_rows(
+          [&](int r) -> TO* {
+            const int out_row = meta_rows[r];
+            if (out_row < 0) return nullptr;
+            const int64_t row = (MODE == kScatter) ? (int64_t)out_row : m0 + r;
+            return y + row * prm.N + (int64_t)nt * BN;
+          },
+          [&](auto cb) { return ((cb * 32) >> 6) * WN + pass * 64 + ((cb * 32) & 63); }, prm.N - (int64_t)nt * BN, BN);
       if constexpr (pass == 0) stamp(7);
       __syncthreads();
     });
@@ -334,11 +351,12 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
       return Elem<TO>::down(Elem<TO>::up(up) * gf * sigmoid_fast(gf));
     });
     __syncthreads();
-    drain_rows([&](int r, int sc) -> TO* {
-      const int64_t p = m0 + r, col = (int64_t)nt * (BN / 2) + (sc >> 6) * (WN / 2) + (sc & 63);
-      if (p >= valid_end || col >= prm.I) return nullptr;
-      return act + p * prm.I + col;
-    });
+    drain_rows(
+        [&](int r) -> TO* {
+          const int64_t p = m0 + r;
+          return p < valid_end ? act + p * prm.I + (int64_t)nt * (BN / 2) : nullptr;
+        },
+        [&](auto cb) { return ((cb * 32) >> 6) * (WN / 2) + ((cb * 32) & 63); }, prm.I - (int64_t)nt * (BN / 2), BN / 2);
   }
   stamp(5);
 }
