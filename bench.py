@@ -212,7 +212,29 @@ def secondary_hbm_kernels(dev):
     yn = cute_kernels.rmsnorm_cute(xn, wn, 1e-6)
     gn = torch.randn_like(yn)
     rec("rmsnorm_bwd_C5", timed(lambda: torch.autograd.grad(yn, (xn, wn), gn, retain_graph=True)), 3 * Bn * Hn * 2 + 4 * Bn)
-    del xn, wn, yn, gn
+    # the step that precedes an MoE block in a transformer: residual add fused into the norm (same rows); algorithmic
+    # bytes: forward reads x, residual and writes y, added; backward reads added, d_y, d_added and writes d_x, d_residual
+    rn = torch.randn(Bn, Hn, device=dev, dtype=torch.bfloat16, requires_grad=True)
+    rec(
+        "fused_residual_add_rmsnorm_fwd_C5",
+        timed(lambda: cute_kernels.fused_residual_add_rmsnorm_cute(xn.detach(), rn.detach(), wn.detach(), 1e-6)),
+        4 * Bn * Hn * 2 + 4 * Bn,
+    )
+    yf, af = cute_kernels.fused_residual_add_rmsnorm_cute(xn, rn, wn, 1e-6)
+    ga = torch.randn_like(af)
+    rec(
+        "fused_residual_add_rmsnorm_bwd_C5",
+        timed(lambda: torch.autograd.grad((yf, af), (xn, rn, wn), (gn, ga), retain_graph=True)),
+        5 * Bn * Hn * 2 + 4 * Bn,
+    )
+    del xn, wn, yn, gn, rn, yf, af, ga
+    # router-logit statistics: softmax over all experts at the C5 router shape (65,536 x 128)
+    lg = torch.randn(Bn, 128, device=dev, dtype=torch.bfloat16, requires_grad=True)
+    rec("softmax_fwd_C5_router", timed(lambda: cute_kernels.softmax_cute(lg.detach())), 2 * Bn * 128 * 2)
+    sm = cute_kernels.softmax_cute(lg)
+    gs = torch.randn_like(sm)
+    rec("softmax_bwd_C5_router", timed(lambda: torch.autograd.grad(sm, lg, gs, retain_graph=True)), 3 * Bn * 128 * 2)
+    del lg, sm, gs
     torch.cuda.empty_cache()
 
     # C4: fine-grained MoE fwd+bwd behind an RMSNorm prologue (T=8192, H=2048, E=64, top-8, I=1408, uniform routing)
