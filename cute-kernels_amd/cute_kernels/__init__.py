@@ -23,7 +23,14 @@ from .scattermoe import (
 from .softmax import softmax_cute
 from .router_stats import load_balancing_loss, load_balancing_stats
 from .swiglu import swiglu_cute, swiglu_packed_cute
-from .utils import ceil_divide, divide_if_divisible, enable_cute_tracing, get_num_elements_and_hidden_size, set_seed
+from .utils import (
+    KernelBackend,
+    ceil_divide,
+    divide_if_divisible,
+    enable_cute_tracing,
+    get_num_elements_and_hidden_size,
+    set_seed,
+)
 
 # torch.compile support: the public functions switch to the registered ops while a trace is being taken
 from . import compile_ops as _compile_ops

@@ -3,6 +3,7 @@
 from __future__ import annotations
 
 import contextlib
+import enum
 import random
 
 import numpy as np
@@ -29,6 +30,14 @@ def is_tracing() -> bool:
     """Whether the public functions must dispatch to their torch.library custom ops (dynamo or cute tracing) instead of
     the eager autograd.Function path. Reference: cute_kernels/utils/custom_op.py:26."""
     return _IS_CUTE_TRACING or torch.compiler.is_compiling()
+
+
+class KernelBackend(enum.Enum):
+    """The reference's backend selector (cute_kernels/kernel_backend.py:11-13), kept so that calls which pass
+    `kernel_backend_forward=KernelBackend.cuda` still read; this build has one backend (HIP) and ignores the choice."""
+
+    cuda = "cuda"
+    triton = "triton"
 
 
 def set_seed(seed: int) -> None:

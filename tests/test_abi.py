@@ -75,6 +75,8 @@ def test_python_api_surface_matches_reference_names_and_signatures():
     sig = inspect.signature(cute_kernels.swiglu_cute)
     assert list(sig.parameters) == ["gate", "up", "kernel_backend_forward", "kernel_backend_backward"]
     assert sig.parameters["kernel_backend_forward"].kind is inspect.Parameter.KEYWORD_ONLY
+    # the selector enum of the reference (kernel_backend.py:11-13) exists so that such calls still read
+    assert {m.name for m in cute_kernels.KernelBackend} == {"cuda", "triton"}
     sig = inspect.signature(cute_kernels.rmsnorm_cute)
     assert list(sig.parameters) == ["x", "weight", "eps", "memory_efficient"]
     assert sig.parameters["memory_efficient"].default is False
