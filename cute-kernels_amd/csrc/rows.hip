@@ -214,6 +214,71 @@ __global__ __launch_bounds__(kBlock) void swiglu_bwd_grouped_kernel(
   store_tile_transposed<T>(tile_gate, d_pre_t, ld_t, p0, (int64_t)I + c0, cols_ok, p0 + kTile);
 }
 
+// Whole-row forms of the two kernels above for callers that take no transposed copy (the weight-gradient GEMM reads
+// row-major operands): consecutive lanes walk consecutive 16-byte chunks of a row, so a wave touches 1 KiB of each
+// stream at a time instead of 64 rows x 128 bytes. Same results as the tiled kernels, pad rows included.
+template <typename T>
+__global__ __launch_bounds__(kBlock) void group_rows_stream_kernel(
+    const T* __restrict__ src, const T* __restrict__ coeff, int fan_out, const int32_t* __restrict__ row_slot,
+    const int32_t* __restrict__ seg_starts, const uint32_t* __restrict__ counts, const int32_t* __restrict__ tile_expert,
+    int align, int64_t max_rows, int chunks_per_row, T* __restrict__ grouped) {
+  const int64_t total = max_rows * chunks_per_row;
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  for (int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x; c < total; c += stride) {
+    const int64_t p = c / chunks_per_row;
+    const int ch = (int)(c - p * chunks_per_row);
+    const int e = tile_expert[p / align];
+    if (e < 0) continue;  // past the last segment: nothing reads these rows
+    vec16 v = zero16();
+    if (p < (int64_t)seg_starts[e] + counts[e]) {
+      if (fan_out > 0) {
+        const int32_t slot = row_slot[p];
+        v = load16(src + ((int64_t)(slot / fan_out) * chunks_per_row + ch) * 8);
+        if (coeff != nullptr) v = scale16<T>(v, Elem<T>::up(coeff[slot]));
+      } else {
+        v = load16(src + c * 8);
+      }
+    }
+    store16_nt(grouped + c * 8, v);
+  }
+}
+
+template <typename T>
+__global__ __launch_bounds__(kBlock) void swiglu_bwd_stream_kernel(
+    const T* __restrict__ pre, const T* __restrict__ d_act, int chunks_per_row, const int32_t* __restrict__ seg_starts,
+    const uint32_t* __restrict__ counts, const int32_t* __restrict__ tile_expert, int align, int64_t max_rows,
+    T* __restrict__ d_pre, int act_kind) {
+  const int64_t total = max_rows * chunks_per_row;
+  const int64_t stride = (int64_t)gridDim.x * kBlock;
+  const int I = chunks_per_row * 8;
+  for (int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x; c < total; c += stride) {
+    const int64_t p = c / chunks_per_row;
+    const int col = (int)(c - p * chunks_per_row) * 8;
+    const int e = tile_expert[p / align];
+    if (e < 0 || p >= (int64_t)seg_starts[e] + counts[e]) continue;  // pad rows of d_pre are left as they are
+    const int64_t up_at = p * 2 * I + col;
+    Pack16<T> u, g, dy, du, dg;
+    u.v = load16_nt(pre + up_at);  // all three are read once
+    g.v = load16_nt(pre + up_at + I);
+    dy.v = load16_nt(d_act + c * 8);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float gf = Elem<T>::up(g.e[i]), uf = Elem<T>::up(u.e[i]), dyf = Elem<T>::up(dy.e[i]);
+      const float sg = sigmoid_for<T>(gf);
+      if (act_kind == CK_ACT_GLU) {  // act = up * sigmoid(gate)
+        dg.e[i] = Elem<T>::down(dyf * uf * sg * (1.0f - sg));
+        du.e[i] = Elem<T>::down(dyf * sg);
+      } else {  // act = up * gate * sigmoid(gate)
+        const float gsg = gf * sg;
+        dg.e[i] = Elem<T>::down(dyf * uf * (sg + gsg * (1.0f - sg)));
+        du.e[i] = Elem<T>::down(dyf * gsg);
+      }
+    }
+    store16_nt(d_pre + up_at, du.v);
+    store16_nt(d_pre + up_at + I, dg.v);
+  }
+}
+
 // dst[b, c, r] = src[b, r, c]; grid: (ceil(cols/64), ceil(rows/64), batch); rows % 8 == 0 and cols % 8 == 0
 template <typename T>
 __global__ __launch_bounds__(kBlock) void transpose_batched_kernel(const T* __restrict__ src, int rows, int cols,
@@ -382,6 +447,16 @@ extern "C" int ck_group_rows_padded(const void* src, const void* coeff, int32_t 
   CK_REQUIRE(max_rows / kTile <= 65535, "ck_group_rows_padded: too many rows for one launch");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)ceil_div(H, kTile), (unsigned)(max_rows / kTile));
+  if (grouped_t == nullptr) {
+    CK_DISPATCH_HALF(dtype, "ck_group_rows_padded", {
+      hipLaunchKernelGGL((group_rows_stream_kernel<scalar_t>), dim3(grid_for(max_rows * (H / 8), 2)), dim3(kBlock), 0, s,
+                         static_cast<const scalar_t*>(src), static_cast<const scalar_t*>(coeff), (int)fan_out, row_slot,
+                         seg_starts, counts, tile_expert, (int)align, max_rows, (int)(H / 8),
+                         static_cast<scalar_t*>(grouped));
+    });
+    CK_CHECK_LAUNCH("ck_group_rows_padded");
+    return CK_OK;
+  }
   CK_DISPATCH_HALF(dtype, "ck_group_rows_padded", {
     hipLaunchKernelGGL((group_rows_padded_kernel<scalar_t>), grid, dim3(kBlock), 0, s,
                        static_cast<const scalar_t*>(src), static_cast<const scalar_t*>(coeff), (int)fan_out, (int)H,
@@ -410,6 +485,15 @@ extern "C" int ck_swiglu_bwd_grouped(const void* pre, const void* d_act, int32_t
   CK_REQUIRE(max_rows / kTile <= 65535, "ck_swiglu_bwd_grouped: too many rows for one launch");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)ceil_div(I, kTile), (unsigned)(max_rows / kTile));
+  if (d_pre_t == nullptr) {
+    CK_DISPATCH_HALF(dtype, "ck_swiglu_bwd_grouped", {
+      hipLaunchKernelGGL((swiglu_bwd_stream_kernel<scalar_t>), dim3(grid_for(max_rows * (I / 8), 2)), dim3(kBlock), 0, s,
+                         static_cast<const scalar_t*>(pre), static_cast<const scalar_t*>(d_act), (int)(I / 8), seg_starts,
+                         counts, tile_expert, (int)align, max_rows, static_cast<scalar_t*>(d_pre), (int)act_kind);
+    });
+    CK_CHECK_LAUNCH("ck_swiglu_bwd_grouped");
+    return CK_OK;
+  }
   CK_DISPATCH_HALF(dtype, "ck_swiglu_bwd_grouped", {
     hipLaunchKernelGGL((swiglu_bwd_grouped_kernel<scalar_t>), grid, dim3(kBlock), 0, s,
                        static_cast<const scalar_t*>(pre), static_cast<const scalar_t*>(d_act), (int)I, seg_starts, counts,

@@ -178,6 +178,17 @@ def test_grouped_gemm_swiglu_epilogues(device, dtype, align, K, I, gemm_tile, ki
     )
     torch.testing.assert_close(d_pre2.float().cpu()[valid], pre_c.grad[valid], rtol=2e-2, atol=2e-2)
     assert torch.equal(d_pre2_t.cpu()[:, :live], (d_pre2.cpu()[:live] * valid[:live, None]).t())
+    # without a transposed copy (the layer's call) the whole-row kernel runs: bit-identical rows, pad rows untouched
+    d_pre3 = torch.full((seg.max_rows, 2 * I), 5.0, dtype=dtype, device=device)
+    _C.check(
+        _C.lib().ck_swiglu_bwd_grouped(
+            pre.data_ptr(), d_act_gpu.data_ptr(), I, seg.seg_starts.data_ptr(), seg.counts.data_ptr(),
+            seg.tile_expert.data_ptr(), seg.align, seg.max_rows, d_pre3.data_ptr(), None, seg.ld_t,
+            _C.CK_ACT_GLU if glu else _C.CK_ACT_SWIGLU, _C.dtype_code(dtype), torch.cuda.current_stream().cuda_stream,
+        )
+    )
+    assert torch.equal(d_pre3.cpu()[valid], d_pre2.cpu()[valid])
+    assert bool((d_pre3.cpu()[~valid] == 5.0).all())
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

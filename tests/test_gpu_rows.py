@@ -67,6 +67,14 @@ def test_group_rows_padded_and_transposes(device, dtype, align):
             expect[p] = (src[slot // k].float() * coeff[slot].float()).to(dtype)
     assert torch.equal(grouped.cpu()[:live], expect[:live])  # pad rows of live tiles are zero
     assert torch.equal(grouped_t.cpu()[:, :live], expect[:live].t())
+    # without a transposed copy the whole-row kernel runs: same rows, same zero pad rows, identity mode too
+    only_rows, none_t = scattermoe._group_rows(src.to(device), coeff.to(device), k, seg, True, False)
+    assert none_t is None and torch.equal(only_rows.cpu()[:live], expect[:live])
+    no_coeff, _ = scattermoe._group_rows(src.to(device), None, k, seg, True, False)
+    tiled_no_coeff, _ = scattermoe._group_rows(src.to(device), None, k, seg, True, True)
+    assert torch.equal(no_coeff.cpu()[:live], tiled_no_coeff.cpu()[:live])
+    same, _ = scattermoe._group_rows(grouped, None, 0, seg, True, False)
+    assert torch.equal(same.cpu()[:live], expect[:live])
     # identity mode (source already padded-grouped) and the batched weight transpose
     _, again_t = scattermoe._group_rows(grouped, None, 0, seg, False, True)
     assert torch.equal(again_t.cpu()[:, :live], expect[:live].t())
