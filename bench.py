@@ -75,6 +75,7 @@ def build_layer(dev):
     bias = bias.to(torch.bfloat16)
     # the router has no bias parameter (torch_implementation.py:83 of the reference): skew goes in through a hook
     moe.gate.register_forward_hook(lambda mod, inp, out: out + bias)
+    moe.zipf_logit_bias = bias
     grad_out = torch.randn(T, H, generator=torch.Generator().manual_seed(SEED + 1)).to(torch.bfloat16).to(dev)
     return moe, x, grad_out, freq.tolist(), c
 
@@ -87,8 +88,9 @@ def step(moe, x, grad_out):
     y.backward(grad_out)
 
 
-def cpu_baseline(moe_gpu, bias_fn_freq, sample_tokens: int = 512):
-    """The torch CPU path (restated in oracle/moe_oracle.py) on `sample_tokens` tokens of the same layer."""
+def cpu_baseline(moe_gpu, bias_fn_freq, sample_tokens: int = T):
+    """The torch CPU path (restated in oracle/moe_oracle.py) on `sample_tokens` tokens of the same layer (default: the
+    whole batch, one forward+backward, 10 to 20 s on 16 host threads), same router skew."""
     import torch
     import torch.nn.functional as F
 
@@ -96,6 +98,8 @@ def cpu_baseline(moe_gpu, bias_fn_freq, sample_tokens: int = 512):
 
     oracle = mo.MoEOracle(E, TOP_K, H, I, mo.swiglu_packed_torch, True, False, 0.02).to(torch.bfloat16)
     oracle.load_state_dict({k: v.cpu() for k, v in moe_gpu.state_dict().items()})
+    cpu_bias = moe_gpu.zipf_logit_bias.cpu()
+    oracle.gate.register_forward_hook(lambda mod, inp, out: out + cpu_bias)
     xs = torch.randn(sample_tokens, H, generator=torch.Generator().manual_seed(SEED)).to(torch.bfloat16).requires_grad_()
     g = torch.randn(sample_tokens, H, generator=torch.Generator().manual_seed(SEED + 1)).to(torch.bfloat16)
     warm = xs[:32].detach().clone().requires_grad_()
@@ -112,7 +116,7 @@ def cpu_baseline(moe_gpu, bias_fn_freq, sample_tokens: int = 512):
         "unit": "TFLOP/s",
         "cores": torch.get_num_threads(),
         "kind": "port",
-        "sample": f"1 fwd+bwd of the same layer on T={sample_tokens} tokens (of {T}), bf16, unskewed router, {dt:.2f} s; "
+        "sample": f"1 fwd+bwd of the same layer on T={sample_tokens} tokens (of {T}), bf16, same Zipf router bias, {dt:.2f} s; "
         f"os.cpu_count()={os.cpu_count()}",
     }
 

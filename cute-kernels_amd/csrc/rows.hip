@@ -487,7 +487,7 @@ extern "C" int ck_swiglu_bwd_grouped(const void* pre, const void* d_act, int32_t
   const dim3 grid((unsigned)ceil_div(I, kTile), (unsigned)(max_rows / kTile));
   if (d_pre_t == nullptr) {
     CK_DISPATCH_HALF(dtype, "ck_swiglu_bwd_grouped", {
-      hipLaunchKernelGGL((swiglu_bwd_stream_kernel<scalar_t>), dim3(grid_for(max_rows * (I / 8), 2)), dim3(kBlock), 0, s,
+      hipLaunchKernelGGL((swiglu_bwd_stream_kernel<scalar_t>), dim3(grid_for(max_rows * (I / 8), 1)), dim3(kBlock), 0, s,
                          static_cast<const scalar_t*>(pre), static_cast<const scalar_t*>(d_act), (int)(I / 8), seg_starts,
                          counts, tile_expert, (int)align, max_rows, static_cast<scalar_t*>(d_pre), (int)act_kind);
     });
