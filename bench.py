@@ -31,10 +31,10 @@ PEAK_HBM_GBS = 8000.0  # MI355X HBM3E
 # summary and commands: profiles/grouped_gemm_c3_moe_fwd_bwd.md. Not measurable from inside this process.
 TRAFFIC_BYTES_PER_LAUNCH = {
     # scatter: mean of the two launches (c_fc dX on the contraction-strided kernel, c_proj fwd on 256 x 384 tiles)
-    "grouped_gemm<scatter>": 2 * 0.5 * (8.118e6 + 3.280e6) * 1024 + 0.5 * (2.621e5 + 3.134e5) * 1024,
-    "grouped_gemm<dw>": 2 * 5.842e6 * 1024 + 1.376e6 * 1024,  # both weight gradients, row-major operands
-    "grouped_gemm<swiglu>": 2 * 8.606e6 * 1024 + 2.753e6 * 1024,
-    "grouped_gemm<grouped>": 2 * 3.964e6 * 1024 + 9.175e5 * 1024,  # c_proj dX, contraction-strided weights
+    "grouped_gemm<scatter>": 2 * 0.5 * (8.130e6 + 3.316e6) * 1024 + 0.5 * (2.622e5 + 3.275e5) * 1024,
+    "grouped_gemm<dw>": 2 * 5.883e6 * 1024 + 1.376e6 * 1024,  # both weight gradients, row-major operands
+    "grouped_gemm<swiglu>": 2 * 8.886e6 * 1024 + 2.753e6 * 1024,
+    "grouped_gemm<grouped>": 2 * 3.811e6 * 1024 + 9.175e5 * 1024,  # c_proj dX, contraction-strided weights
 }
 
 # workload: configs[2] of the baseline, the configuration its headline metric (MoE fwd+bwd TFLOP/s) is quoted on
