@@ -324,12 +324,13 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
     //   (the only loads in flight) and for this wave's own fragment reads, then meet the other waves -- the whole current
     //   stage has been read by everyone, so in phase 0 the loads of step kt + 2 overwrite it under this slice's MFMAs.
     //   Phase 1 is step nk - 2 (nothing left to fetch), phase 2 the last step (nothing to wait for, nothing to reload).
-    auto slice = [&](int kt, auto sl, auto phase) {
+    auto slice = [&](int kt, auto sl, auto phase, auto idle) {
+      constexpr bool kIdle = decltype(idle)::value;  // this wave's 64 rows are all pad rows: no fragments, no MFMAs
       constexpr bool kLast = decltype(sl)::value == KS - 1;
       constexpr int kPhase = decltype(phase)::value;
       const int ns = kLast ? (kt + 1) & (NSTAGE - 1) : kt & (NSTAGE - 1);
       constexpr int nsl = kLast ? 0 : decltype(sl)::value + 1;
-      constexpr bool kReload = !(kLast && kPhase == 2) && !(CK_ABLATE & 4);
+      constexpr bool kReload = !(kLast && kPhase == 2) && !(CK_ABLATE & 4) && !kIdle;
       if constexpr (kLast && kPhase < 2) {
         if constexpr ((CK_ABLATE & 1) != 0) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         else if constexpr ((CK_ABLATE & 8) != 0) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
@@ -349,7 +350,7 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
         };
 #pragma unroll
         for (int n = 0; n < 2 * NI; ++n) {
-          mfma(cur, n / NI, n % NI);
+          if constexpr (!kIdle) mfma(cur, n / NI, n % NI);
           if constexpr (kLast && kPhase == 0 && !(CK_ABLATE & 2)) {
             if (n < kLoadsPerStep) issue_one(kt + 2, n);
           }
@@ -361,7 +362,7 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
       } else {
 #pragma unroll
         for (int j = 0; j < NI; ++j) {
-          mfma(0, 0, j);
+          if constexpr (!kIdle) mfma(0, 0, j);
           if constexpr (kLast && kPhase == 0 && !(CK_ABLATE & 2)) {
             if (j < kLoadsPerStep) issue_one(kt + 2, j);
           }
@@ -370,7 +371,7 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
         if constexpr (kReload) read_a(ns, nsl, 0);
 #pragma unroll
         for (int j = 0; j < NI; ++j) {
-          mfma(0, 1, j);
+          if constexpr (!kIdle) mfma(0, 1, j);
           if constexpr (kLast && kPhase == 0 && !(CK_ABLATE & 2)) {
             if (NI + j < kLoadsPerStep) issue_one(kt + 2, NI + j);
           }
@@ -381,11 +382,20 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
       }
       __builtin_amdgcn_sched_barrier(0);
     };
-    auto k_step = [&](int kt, auto phase) { static_for<KS>([&](auto sl) { slice(kt, sl, phase); }); };
-    int kt = 0;
-    for (; kt + 2 < nk; ++kt) k_step(kt, std::integral_constant<int, 0>{});
-    if (kt + 2 == nk) k_step(kt++, std::integral_constant<int, 1>{});
-    k_step(kt, std::integral_constant<int, 2>{});
+    auto k_loop = [&](auto idle) {
+      auto k_step = [&](int kt, auto phase) { static_for<KS>([&](auto sl) { slice(kt, sl, phase, idle); }); };
+      int kt = 0;
+      for (; kt + 2 < nk; ++kt) k_step(kt, std::integral_constant<int, 0>{});
+      if (kt + 2 == nk) k_step(kt++, std::integral_constant<int, 1>{});
+      k_step(kt, std::integral_constant<int, 2>{});
+    };
+    // A wave whose 64 tile rows all lie past the expert's last row (the tile is the ragged end of a segment) still
+    // issues its share of the loads and meets every barrier, but multiplies nothing: the wave it shares a SIMD with
+    // then has the matrix pipe to itself. Its accumulators stay zero and its rows are never stored.
+    bool wave_idle = false;
+    if constexpr (MODE != kDw) wave_idle = m0 + wm * WM >= valid_end;
+    if (__builtin_amdgcn_readfirstlane(wave_idle)) k_loop(std::true_type{});
+    else k_loop(std::false_type{});
   }
 
   // ---- epilogue through LDS. Lane holds, per 32x32 block and q in 0..3, rows 8q + 4*(lane/32) + 0..3 of column lane%32:
