@@ -30,11 +30,21 @@ PEAK_HBM_GBS = 8000.0  # MI355X HBM3E
 # this same command, FETCH_SIZE scaled x2.0 and WRITE_SIZE x1.0 against a 1 GiB device copy (known size);
 # summary and commands: profiles/grouped_gemm_c3_moe_fwd_bwd.md. Not measurable from inside this process.
 TRAFFIC_BYTES_PER_LAUNCH = {
-    # scatter: mean of the two launches (c_fc dX on the contraction-strided kernel, c_proj fwd on 256 x 384 tiles)
-    "grouped_gemm<scatter>": 2 * 0.5 * (8.130e6 + 3.316e6) * 1024 + 0.5 * (2.622e5 + 3.275e5) * 1024,
-    "grouped_gemm<dw>": 2 * 5.883e6 * 1024 + 1.376e6 * 1024,  # both weight gradients, row-major operands
-    "grouped_gemm<swiglu>": 2 * 8.886e6 * 1024 + 2.753e6 * 1024,
-    "grouped_gemm<grouped>": 2 * 3.811e6 * 1024 + 9.175e5 * 1024,  # c_proj dX, contraction-strided weights
+    "grouped_gemm_dw_rows": 2 * 5.883e6 * 1024 + 1.376e6 * 1024,  # both weight gradients, row-major operands
+    "grouped_gemm<swiglu>": 2 * 8.886e6 * 1024 + 2.753e6 * 1024,  # c_fc forward
+    "grouped_gemm_nn<scatter>": 2 * 8.130e6 * 1024 + 2.622e5 * 1024,  # c_fc dX, contraction-strided weights
+    "grouped_gemm_nn<grouped>": 2 * 3.811e6 * 1024 + 9.175e5 * 1024,  # c_proj dX, contraction-strided weights
+    "grouped_gemm<scatter>": 2 * 3.316e6 * 1024 + 3.275e5 * 1024,  # c_proj forward, 256 x 384 tiles
+}
+
+# the kernel instantiation each launch name runs at this workload, as rocprofv3's kernel trace spells it
+# (grouped_gemm_line_kernel<T, MODE, BN, BT>: MODE 0 grouped, 1 scatter, 2 swiglu, 4 dw)
+ROCPROF_KERNEL = {
+    "grouped_gemm_dw_rows": "grouped_gemm_line_kernel<bf16, 4, 256, true>",
+    "grouped_gemm<swiglu>": "grouped_gemm_line_kernel<bf16, 2, 256, false>",
+    "grouped_gemm_nn<scatter>": "grouped_gemm_line_kernel<bf16, 1, 256, true>",
+    "grouped_gemm_nn<grouped>": "grouped_gemm_line_kernel<bf16, 0, 256, true>",
+    "grouped_gemm<scatter>": "grouped_gemm_line_kernel<bf16, 1, 384, false>",
 }
 
 # workload: configs[2] of the baseline, the configuration its headline metric (MoE fwd+bwd TFLOP/s) is quoted on
@@ -397,6 +407,7 @@ def main() -> int:
     roofline = {
         "bound": "mfma",
         "kernel": dominant,
+        "rocprof_kernel": ROCPROF_KERNEL.get(dominant),
         "achieved": achieved,
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",

@@ -187,7 +187,10 @@ def _sort_by_expert_eager(expert_ids: torch.Tensor, num_experts: int, align: int
 # ---------------------------------------------------------------------------------------------------------------
 class LaunchTimer:
     """Optional per-launch timing of the grouped GEMMs with events on the launch stream (used by bench.py).
-    records: list of (kernel name, [N, K] or [M, N] of the launch, start event, end event)."""
+    records: list of (kernel name, [N, K] or [M, N] of the launch, start event, end event). Names follow the entry point
+    and epilogue, so that at the benchmark's shapes one name is one kernel instantiation: grouped_gemm<epilogue>
+    (ck_grouped_gemm), grouped_gemm_nn<epilogue> (ck_grouped_gemm_nn, weights read as stored), grouped_gemm<dw>
+    (ck_grouped_gemm_dw, transposed operands), grouped_gemm_dw_rows (ck_grouped_gemm_dw_rows, row-major operands)."""
 
     def __init__(self) -> None:
         self.records: list = []
@@ -264,7 +267,7 @@ def _gemm_dx(d_y, w, seg: ExpertSegments, epilogue, out):
         if launch_timer is None:
             launch()
         else:
-            launch_timer.time(_EPILOGUE_NAMES[epilogue], (n_in, n_out), launch)
+            launch_timer.time(_EPILOGUE_NAMES[epilogue].replace("grouped_gemm<", "grouped_gemm_nn<"), (n_in, n_out), launch)
         return
     _gemm(d_y, 0, _transpose_weights(w), seg, epilogue, out)
 
@@ -310,7 +313,7 @@ def _gemm_dw_rows(a, b, seg: ExpertSegments, dw):
     if launch_timer is None:
         launch()
     else:
-        launch_timer.time("grouped_gemm<dw>", (M, N), launch)
+        launch_timer.time("grouped_gemm_dw_rows", (M, N), launch)
 
 
 def _dw_from_rows(max_rows: int, num_experts: int, align: int, *shapes: tuple[int, int]) -> bool:
