@@ -340,6 +340,45 @@ def gemm_only(dev, launches: int):
                       "TFLOP/s": flops / ms / 1e9, "frac_mfma": flops / ms / 1e9 / PEAK_BF16_TFLOPS}))
 
 
+def library_gemm_yardstick(dev, iters: int = 10):
+    """What this box's chip sustains on dense bf16 products of the layer's per-expert shapes through torch.matmul
+    (the vendor GEMM library), on the same kind of data (activations N(0,1), weights N(0,0.02)) and on zeros: the
+    same-box yardstick for the grouped GEMM figures (clocks are power-managed and depend on the operand bits)."""
+    import torch
+
+    out = {}
+    shapes = {
+        "c_fc_largest_expert_10928x28672x4096": (10928, 2 * I, H),
+        "c_proj_largest_expert_10928x4096x14336": (10928, H, I),
+        "c_fc_all_rows_32768x28672x4096": (T * TOP_K, 2 * I, H),
+        "square_8192": (8192, 8192, 8192),
+    }
+    for name, (m, n, k) in shapes.items():
+        for data in ("normal", "zeros"):
+            if data == "normal":
+                a = torch.randn(m, k, device=dev, dtype=torch.bfloat16)
+                b = (torch.randn(n, k, device=dev) * 0.02).to(torch.bfloat16)
+            else:
+                a = torch.zeros(m, k, device=dev, dtype=torch.bfloat16)
+                b = torch.zeros(n, k, device=dev, dtype=torch.bfloat16)
+            c = torch.empty(m, n, device=dev, dtype=torch.bfloat16)
+            for _ in range(3):
+                torch.matmul(a, b.t(), out=c)
+            torch.cuda.synchronize()
+            s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            s.record()
+            for _ in range(iters):
+                torch.matmul(a, b.t(), out=c)
+            e.record()
+            torch.cuda.synchronize()
+            ms = s.elapsed_time(e) / iters
+            tf = 2.0 * m * n * k / ms / 1e9
+            out[f"{name}_{data}"] = {"ms": ms, "TFLOP/s": tf, "frac_mfma": tf / PEAK_BF16_TFLOPS}
+            del a, b, c
+    torch.cuda.empty_cache()
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -352,6 +391,8 @@ def main() -> int:
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device copy (outside the timed region): the known-size kernel that "
                     "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
+    ap.add_argument("--only-yardstick", action="store_true",
+                    help="run only torch.matmul on the layer's per-expert shapes (the same-box library yardstick)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this build uses no second GPU (no collectives, no sharding); run with --gpus 1",
@@ -366,6 +407,9 @@ def main() -> int:
     dev = torch.device("cuda:0")
     if args.only_gemm > 0:
         gemm_only(dev, args.only_gemm)
+        return 0
+    if args.only_yardstick:
+        print(json.dumps({"library_gemm_yardstick": library_gemm_yardstick(dev)}))
         return 0
     moe, x, grad_out, freq, zipf_c = build_layer(dev)
     x.requires_grad_()
@@ -457,6 +501,7 @@ def main() -> int:
         torch.cuda.empty_cache()
         # the secondary metric (count + scatter GB/s: the HBM-bound kernels on their own) and the other two GPU configs
         line["count_scatter"], line["other_configs"] = secondary_hbm_kernels(dev)
+        line["library_gemm_yardstick"] = library_gemm_yardstick(dev)
         moe = None
     if not args.skip_cpu_baseline:
         if moe is None:

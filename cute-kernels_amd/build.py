@@ -1,9 +1,15 @@
 """Ahead-of-time build of libck_mi355.so (HIP, gfx950 only) into the Python package directory.
 
-    python cute-kernels_amd/build.py [--jobs N] [--force]
+    python cute-kernels_amd/build.py [--jobs N] [--force] [--define NAME=VALUE ...] [--output FILE.so]
 
 Every translation unit under csrc/ is compiled with hipcc to an object file (in parallel) and linked into
 cute_kernels/libck_mi355.so. Nothing is compiled at import time: the package only ever dlopens the result.
+
+Measurement builds: `--define CK_ABLATE=2 --output libck_ablate2.so` compiles the same sources with the given
+preprocessor definitions into their own object directory and links a separately named library next to the product
+one (the product library is untouched). The package loads it instead when the environment variable CK_MI355_LIB names
+it (file name inside cute_kernels/, or a path); the switches are documented where they are used (CK_ABLATE, CK_STAMP
+in csrc/grouped_gemm_line.hip and csrc/grouped_gemm_fp8.hip).
 """
 
 from __future__ import annotations
@@ -36,13 +42,13 @@ def _newest_header_mtime() -> float:
     return max(os.path.getmtime(h) for h in headers)
 
 
-def _compile(src: str, force: bool) -> str:
-    obj = os.path.join(OBJ_DIR, src + ".o")
+def _compile(src: str, force: bool, defines: tuple[str, ...] = (), obj_dir: str = OBJ_DIR) -> str:
+    obj = os.path.join(obj_dir, src + ".o")
     src_path = os.path.join(CSRC, src)
     if not force and os.path.exists(obj):
         if os.path.getmtime(obj) >= max(os.path.getmtime(src_path), _newest_header_mtime()):
             return obj
-    cmd = [HIPCC, *COMMON_FLAGS]
+    cmd = [HIPCC, *COMMON_FLAGS, *(f"-D{d}" for d in defines)]
     if src.endswith(".hip"):
         cmd += DEVICE_FLAGS
     cmd += ["-c", src_path, "-o", obj]
@@ -52,21 +58,27 @@ def _compile(src: str, force: bool) -> str:
     return obj
 
 
-def build(jobs: int = 8, force: bool = False) -> str:
-    os.makedirs(OBJ_DIR, exist_ok=True)
+def build(jobs: int = 8, force: bool = False, defines: tuple[str, ...] = (), output: str | None = None) -> str:
+    if defines and not output:
+        raise ValueError("a build with --define needs its own --output name: the product library takes no definitions")
+    lib_path = LIB_PATH if not output else os.path.join(os.path.dirname(LIB_PATH), os.path.basename(output))
+    obj_dir = OBJ_DIR if not output else os.path.join(OBJ_DIR, os.path.splitext(os.path.basename(output))[0])
+    os.makedirs(obj_dir, exist_ok=True)
     with ThreadPoolExecutor(max_workers=max(1, jobs)) as pool:
-        objs = list(pool.map(lambda s: _compile(s, force), _sources()))
-    cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", LIB_PATH, *objs]
+        objs = list(pool.map(lambda s: _compile(s, force, tuple(defines), obj_dir), _sources()))
+    cmd = [HIPCC, "-shared", "-fPIC", "--offload-arch=gfx950", "-o", lib_path, *objs]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
         raise RuntimeError(f"link failed:\n{proc.stdout}\n{proc.stderr}")
-    return LIB_PATH
+    return lib_path
 
 
 if __name__ == "__main__":
     ap = argparse.ArgumentParser()
     ap.add_argument("--jobs", type=int, default=8)
     ap.add_argument("--force", action="store_true")
+    ap.add_argument("--define", action="append", default=[], metavar="NAME=VALUE")
+    ap.add_argument("--output", default=None, metavar="FILE.so")
     args = ap.parse_args()
-    print(build(args.jobs, args.force))
+    print(build(args.jobs, args.force, tuple(args.define), args.output))
     sys.exit(0)

@@ -15,6 +15,11 @@ import torch
 
 _LIB_NAME = "libck_mi355.so"
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), _LIB_NAME)
+# Measurement builds (build.py --define ... --output libck_<name>.so) are loaded instead of the product library when
+# CK_MI355_LIB names one: a file name inside this directory, or a path. Still no fallback: a missing file raises.
+if os.environ.get("CK_MI355_LIB"):
+    _alt = os.environ["CK_MI355_LIB"]
+    _LIB_PATH = _alt if os.path.sep in _alt else os.path.join(os.path.dirname(os.path.abspath(__file__)), _alt)
 
 CK_F32, CK_F16, CK_BF16 = 0, 1, 2
 CK_EPI_GROUPED, CK_EPI_SCATTER, CK_EPI_SWIGLU, CK_EPI_SWIGLU_BWD = 0, 1, 2, 3

@@ -16,11 +16,6 @@ import torch.nn as nn
 import torch.nn.functional as F
 
 
-def continuous_count_torch(x: torch.Tensor, size: int) -> torch.Tensor:
-    """cute_kernels/kernels/continuous_count/torch_implementation.py:8-10"""
-    return x.bincount(minlength=size).to(torch.uint32)
-
-
 def swiglu_torch(gate: torch.Tensor, up: torch.Tensor) -> torch.Tensor:
     """cute_kernels/kernels/swiglu/torch_implementation.py:9-18: fp32 math, one rounding."""
     dtype = gate.dtype
@@ -147,9 +142,11 @@ class MoEOracle(nn.Module):
 
 
 # ---------------------------------------------------------------------------------------------------------------
-# fp8 (e4m3) quantised-expert forward. The reference has NO fp8 code or tests: PARITY UNPINNED upstream. This is the
-# specification this build gives itself: the reference layer (torch_implementation.py:137-169) evaluated on
-# de-quantised operands, with the roundings a 16-bit tensor between the two expert linears implies.
+# fp8 (e4m3) quantised-expert forward. The reference has NO fp8 code or tests, so there is nothing upstream to compare
+# with; this is the specification this build gives itself: the reference layer (torch_implementation.py:137-169)
+# evaluated on de-quantised operands, with the roundings a 16-bit tensor between the two expert linears implies.
+# Both functions are pinned in tests/test_oracle.py against the OCP e4m3fn value table written out from the format
+# definition (brute-force nearest value, ties to even) and an fp64 dense per-token formulation built on that table.
 # ---------------------------------------------------------------------------------------------------------------
 E4M3_MAX = 448.0
 

@@ -284,3 +284,176 @@ def test_load_balancing_loss_closed_form_and_invariants():
     peaked = torch.full((16, E), -1e4)
     peaked[:, 3] = 0.0
     assert abs(float(mo.load_balancing_loss_torch(peaked, torch.full((16, k), 3))) - E * k) < 1e-4
+
+
+# ---- fp8 (e4m3fn) quantiser and quantised-expert forward ----------------------------------------------------------
+def _e4m3fn_table() -> np.ndarray:
+    """All 256 OCP e4m3fn values from the format definition (1 sign, 4 exponent bits with bias 7, 3 mantissa bits;
+    exponent 0 is subnormal; S.1111.111 is NaN; there is no infinity), written out without any library cast."""
+    vals = np.empty(256, dtype=np.float64)
+    for code in range(256):
+        sign = -1.0 if code & 0x80 else 1.0
+        exp, man = (code >> 3) & 0xF, code & 0x7
+        if exp == 0xF and man == 0x7:
+            vals[code] = np.nan
+        elif exp == 0:
+            vals[code] = sign * (man / 8.0) * 2.0**-6
+        else:
+            vals[code] = sign * (1.0 + man / 8.0) * 2.0 ** (exp - 7)
+    return vals
+
+
+def _nearest_e4m3fn_code(v: float, table: np.ndarray) -> int:
+    """Brute force: the finite code closest to v; on an exact tie the one with an even mantissa bit (even code)."""
+    best, best_d = None, None
+    for code in range(256):
+        if np.isnan(table[code]) or (table[code] == 0 and code == 0x80 and not np.signbit(v)):
+            continue
+        if table[code] == 0 and code == 0x00 and np.signbit(v):
+            continue
+        d = abs(table[code] - v)
+        if best is None or d < best_d or (d == best_d and code % 2 == 0 and best % 2 == 1):
+            best, best_d = code, d
+    return best
+
+
+def _quantize_rows_brute(x64: np.ndarray, table: np.ndarray):
+    """Independent per-row quantiser: scale = amax / 448 (1 for an all-zero row), q = nearest table value of
+    fp32(x * fp32(448 / amax))."""
+    codes = np.zeros(x64.shape, dtype=np.uint8)
+    scales = np.ones(x64.shape[0], dtype=np.float32)
+    for r in range(x64.shape[0]):
+        row = x64[r].astype(np.float32)
+        amax = np.float32(np.abs(row).max())
+        inv = np.float32(1.0)
+        if amax > 0:
+            scales[r] = amax / np.float32(448.0)
+            inv = np.float32(448.0) / amax
+        for c in range(row.size):
+            codes[r, c] = _nearest_e4m3fn_code(float(np.float32(row[c] * inv)), table)
+    return codes, scales
+
+
+def test_e4m3fn_table_facts():
+    t = _e4m3fn_table()
+    assert np.nanmax(t) == 448.0 and np.nanmin(t) == -448.0
+    assert t[0x7E] == 448.0 and np.isnan(t[0x7F]) and np.isnan(t[0xFF])
+    assert t[0x01] == 2.0**-9 and t[0x08] == 2.0**-6 and t[0x38] == 1.0  # smallest subnormal / normal, one
+    assert np.sum(np.isfinite(t)) == 254
+    # torch's cast decodes the same table (library routine against the format definition)
+    decoded = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).float().numpy()
+    np.testing.assert_array_equal(np.nan_to_num(decoded, nan=12345.0), np.nan_to_num(t, nan=12345.0).astype(np.float32))
+
+
+def test_quantize_rows_e4m3_against_brute_force_nearest_value():
+    table = _e4m3fn_table()
+    g = torch.Generator().manual_seed(21)
+    rows = [
+        torch.randn(24, generator=g),                                  # ordinary row, maximum somewhere inside
+        torch.zeros(24),                                               # all-zero row: scale 1, codes 0
+        torch.tensor([0.1, -3.0, 0.2] + [0.0] * 21),                    # negative maximum, not at index 0
+        torch.tensor([448.0] + [v for v in (17.0, 19.0, 21.0, 23.0, 25.0, 27.0, 29.0, 31.0)] + [0.0] * 15),  # ties: odd multiples of the half step in [16, 32)
+        torch.tensor([448.0, 2.0**-9, 2.0**-10, 1.5 * 2.0**-10, 3.0 * 2.0**-10, 2.0**-7 + 2.0**-10] + [0.0] * 18),  # subnormals and their ties
+        torch.tensor([1e-30, -1e-31] + [0.0] * 22),                     # tiny maximum: scale far below 1
+        torch.tensor([3e38, -1e38, 5.0] + [0.0] * 21),                  # huge maximum
+        torch.randn(24, generator=g) * 1e-3,
+    ]
+    x = torch.stack(rows)
+    q, scale = mo.quantize_rows_e4m3_torch(x)
+    assert q.dtype == torch.float8_e4m3fn and scale.dtype == torch.float32 and scale.shape == (len(rows),)
+    codes, scales = _quantize_rows_brute(x.double().numpy(), table)
+    got = q.view(torch.uint8).numpy()
+    # +0 and -0 decode to the same value: compare decoded values, then codes where the value is not zero
+    np.testing.assert_array_equal(table[got], table[codes])
+    nz = table[codes] != 0
+    np.testing.assert_array_equal(got[nz], codes[nz])
+    np.testing.assert_array_equal(scale.numpy(), scales)
+    # scale = amax / 448, and 1 for the all-zero row
+    amax = x.abs().amax(-1)
+    assert float(scale[1]) == 1.0 and not np.any(got[1] & 0x7F)
+    np.testing.assert_array_equal(scale[amax > 0].numpy(), (amax[amax > 0] / 448.0).numpy())
+    # the row maximum saturates exactly at +-448
+    for r in range(len(rows)):
+        if float(amax[r]) > 0:
+            i = int(x[r].abs().argmax())
+            assert table[got[r, i]] == (448.0 if float(x[r, i]) > 0 else -448.0)
+    # ties go to the even mantissa: 17 -> 16, 19 -> 20, 21 -> 20, 23 -> 24, ... (step 2 in [16, 32))
+    assert table[got[3, 1:9]].tolist() == [16.0, 20.0, 20.0, 24.0, 24.0, 28.0, 28.0, 32.0]
+    # subnormals (step 2^-9): 2^-9 exact, 2^-10 ties to 0, 1.5 * 2^-10 rounds up to 2^-9, 3 * 2^-10 ties to 2^-8
+    assert table[got[4, 1:5]].tolist() == [2.0**-9, 0.0, 2.0**-9, 2.0**-8]
+    # the error bound of round-to-nearest: |x - q * scale| <= half a step of the binade of the scaled value
+    deq = table[got] * scale.double().numpy()[:, None]
+    scaled = np.abs(x.double().numpy() / scale.double().numpy()[:, None])
+    step = np.where(scaled < 2.0**-6, 2.0**-9, 2.0 ** (np.floor(np.log2(np.maximum(scaled, 2.0**-6))) - 3))
+    assert np.all(np.abs(x.double().numpy() - deq) <= (0.5 * step * (1 + 1e-6)) * scale.double().numpy()[:, None])
+
+
+def test_quantize_rows_e4m3_scale_direction_and_dtypes():
+    """De-quantisation is q * scale (not q / scale), whatever the input dtype; a swapped direction is off by (amax/448)^2."""
+    table = _e4m3fn_table()
+    for dtype in (torch.float32, torch.bfloat16, torch.float16):
+        x = (torch.randn(5, 40, generator=torch.Generator().manual_seed(4)) * 7).to(dtype)
+        q, s = mo.quantize_rows_e4m3_torch(x)
+        deq = table[q.view(torch.uint8).numpy()] * s.double().numpy()[:, None]
+        rel = np.linalg.norm(deq - x.double().numpy()) / np.linalg.norm(x.double().numpy())
+        assert rel < 0.04  # 3 mantissa bits: about 2^-4 / sqrt(3) relative error per element
+
+
+def _bf16(v: np.ndarray) -> np.ndarray:
+    """fp64 -> nearest bfloat16 (ties to even) as fp64, through bit arithmetic on the fp32 pattern (no torch cast)."""
+    f = np.asarray(v, dtype=np.float64).astype(np.float32)
+    bits = f.view(np.uint32).astype(np.uint64)
+    rounded = ((bits + 0x7FFF + ((bits >> 16) & 1)) >> 16) << 16
+    return rounded.astype(np.uint32).view(np.float32).astype(np.float64)
+
+
+def _dense_e4m3_moe_fp64(moe, x, selected, gates, table):
+    """Independent formulation of the quantised-expert forward: brute-force quantiser, table de-quantisation, fp64
+    products per token and slot, 16-bit roundings where a 16-bit tensor sits (pre-activation, activation, expert
+    output, combined output). No call into oracle/."""
+    E, H = moe.num_experts, x.shape[1]
+    w1c, w1s = _quantize_rows_brute(moe.c_fc.weight.detach().double().flatten(0, 1).numpy(), table)
+    w2c, w2s = _quantize_rows_brute(moe.c_proj.weight.detach().double().flatten(0, 1).numpy(), table)
+    w1 = (table[w1c] * w1s.astype(np.float64)[:, None]).reshape(E, -1, H)
+    w2 = (table[w2c] * w2s.astype(np.float64)[:, None]).reshape(E, H, -1)
+    xc, xs = _quantize_rows_brute(x.double().numpy(), table)
+    xd = table[xc] * xs.astype(np.float64)[:, None]
+    I = w2.shape[2]
+    out = np.zeros(x.shape, dtype=np.float64)
+    for t in range(x.shape[0]):
+        for j in range(selected.shape[1]):
+            e = int(selected[t, j])
+            pre = _bf16(w1[e] @ xd[t])
+            up, gate = pre[:I], pre[I:]
+            act = _bf16(up * gate / (1.0 + np.exp(-gate)))
+            ac, a_s = _quantize_rows_brute(act[None], table)
+            y = _bf16(w2[e] @ (table[ac[0]] * float(a_s[0])))
+            out[t] += float(gates[t, j]) * y
+    return _bf16(out)
+
+
+def test_moe_e4m3_forward_oracle_matches_dense_fp64_formulation_on_table():
+    table = _e4m3fn_table()
+    torch.manual_seed(33)
+    E, k, H, I, T = 4, 2, 32, 48, 9
+    moe = mo.MoEOracle(E, k, H, I, mo.swiglu_packed_torch, True, False, 0.25).to(torch.bfloat16)
+    x = torch.randn(T, H).to(torch.bfloat16)
+    x[3] = 0  # an all-zero token: scale 1, output 0
+    sel = torch.stack([torch.randperm(E)[:k] for _ in range(T)])
+    gates = torch.softmax(torch.randn(T, k), -1).to(torch.bfloat16)
+    got = mo.moe_e4m3_forward_oracle(moe, x, sel, gates).double().numpy()
+    want = _dense_e4m3_moe_fp64(moe, x, sel.numpy(), gates.double().numpy(), table)
+    assert np.abs(want).mean() > 0.05  # an O(0.1 .. 1) signal, so that the tolerance below means something
+    assert not np.any(got[3]) and not np.any(want[3])
+    # fp32 against fp64 accumulation can move a value across a bf16 rounding boundary now and then, and such a flip
+    # can move an activation to the neighbouring e4m3 value: allow two bf16 steps, and require most elements bit-equal.
+    # A mistake in the specification (scale direction, the zero-row rule, a missing 16-bit rounding of the
+    # pre-activation or the activation, up/gate swapped, gates applied before the rounding of y) is far outside.
+    np.testing.assert_allclose(got, want, rtol=2.0**-6, atol=2.0**-9)
+    assert np.mean(got == want) > 0.9
+    # sensitivity: with the up and gate halves of c_fc exchanged the result is nowhere near
+    swapped = mo.MoEOracle(E, k, H, I, mo.swiglu_packed_torch, True, False, 0.25).to(torch.bfloat16)
+    swapped.load_state_dict(moe.state_dict())
+    with torch.no_grad():
+        swapped.c_fc.weight.copy_(torch.cat(moe.c_fc.weight.chunk(2, dim=1)[::-1], dim=1))
+    assert not np.allclose(mo.moe_e4m3_forward_oracle(swapped, x, sel, gates).double().numpy(), want, rtol=2.0**-6, atol=2.0**-9)
