@@ -369,15 +369,18 @@ extern "C" int64_t ck_count_workspace_words(int32_t num_bins) {
   return 1 + (int64_t)(num_bins > 0 ? num_bins : 0) * count_replicas(num_bins);
 }
 
-extern "C" int ck_count_offsets(const void* ids, int32_t ids_are_i64, int64_t n, int32_t num_bins, uint32_t* counts,
-                                uint32_t* ends, uint32_t* starts, uint32_t* workspace, void* stream) {
-  CK_REQUIRE(num_bins >= 1 && num_bins <= kMaxCountBins, "ck_count_offsets: num_bins=%d outside [1, %d]", num_bins,
-             kMaxCountBins);
-  CK_REQUIRE(n >= 0, "ck_count_offsets: n=%lld is negative", (long long)n);
-  CK_REQUIRE(counts != nullptr && workspace != nullptr, "ck_count_offsets: counts and workspace are required");
-  CK_REQUIRE(n == 0 || ids != nullptr, "ck_count_offsets: ids is NULL");
+namespace ck {
+namespace {
+
+// Validates the arguments and launches count_kernel on `workspace` (zero on entry, zero again on exit).
+int launch_count(const char* name, const void* ids, int32_t ids_are_i64, int64_t n, int32_t num_bins, uint32_t* counts,
+                 uint32_t* ends, uint32_t* starts, uint32_t* workspace, hipStream_t s) {
+  CK_REQUIRE(num_bins >= 1 && num_bins <= kMaxCountBins, "%s: num_bins=%d outside [1, %d]", name, num_bins, kMaxCountBins);
+  CK_REQUIRE(n >= 0, "%s: n=%lld is negative", name, (long long)n);
+  CK_REQUIRE(counts != nullptr && workspace != nullptr, "%s: counts and workspace are required", name);
+  CK_REQUIRE(n == 0 || ids != nullptr, "%s: ids is NULL", name);
   const size_t esz = ids_are_i64 ? 8 : 4;
-  CK_REQUIRE((reinterpret_cast<uintptr_t>(ids) & (esz - 1)) == 0, "ck_count_offsets: ids is not element-aligned");
+  CK_REQUIRE((reinterpret_cast<uintptr_t>(ids) & (esz - 1)) == 0, "%s: ids is not element-aligned", name);
 
   const int64_t vec = 16 / (int64_t)esz;
   // 4 vectors per thread per trip; one block for small inputs. Large inputs: 2 blocks per CU stream fastest with the LDS
@@ -395,7 +398,6 @@ extern "C" int ck_count_offsets(const void* ids, int32_t ids_are_i64, int64_t n,
   const int reg_bins = num_bins <= 8 ? 8 : 0;  // 16 register counters measured slower (3.3 TB/s) than LDS atomics (5.6)
   const int copies = reg_bins > 0 ? 1 : (num_bins <= 1024 ? kWavesPerBlock : 1);
   const size_t lds_bytes = ((size_t)copies * num_bins + kWavesPerBlock + 2) * sizeof(uint32_t);
-  hipStream_t s = static_cast<hipStream_t>(stream);
 #define CK_LAUNCH_COUNT(ID_T, RB)                                                                              \
   hipLaunchKernelGGL((count_kernel<ID_T, RB>), dim3((unsigned)blocks), dim3(kBlock), lds_bytes, s,            \
                      static_cast<const ID_T*>(ids), n, (int)num_bins, copies, count_replicas(num_bins), counts, ends,   \
@@ -408,8 +410,74 @@ extern "C" int ck_count_offsets(const void* ids, int32_t ids_are_i64, int64_t n,
     else CK_LAUNCH_COUNT(int32_t, 0);
   }
 #undef CK_LAUNCH_COUNT
-  CK_CHECK_LAUNCH("ck_count_offsets");
+  CK_CHECK_LAUNCH(name);
   return CK_OK;
+}
+
+// ---- the entry point that allocates nothing ---------------------------------------------------------------------
+// The count kernel's workspace (ticket + replicated global accumulators: at most 1 + 16384 words) lives in this
+// file-scope device array instead of a caller's buffer. Every GPU holds its own copy at its own address until the
+// process ends. In host code the array's name is only a handle for hipGetSymbolAddress: the address a kernel may use is
+// looked up once per device, with that device current, and kept in g_scratch_ptr.
+constexpr int kScratchWords = 1 + kMaxCountBins;
+static __device__ __align__(256) uint32_t scratch[kScratchWords];
+
+constexpr int kMaxScratchDevices = 64;
+uint32_t* g_scratch_ptr[kMaxScratchDevices] = {};
+
+int scratch_for_current_device(const char* name, uint32_t** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= kMaxScratchDevices) {
+    set_error("%s: cannot tell the current device (%s, device %d)", name, hipGetErrorString(e), dev);
+    return CK_ERR_LAUNCH;
+  }
+  uint32_t* p = __atomic_load_n(&g_scratch_ptr[dev], __ATOMIC_ACQUIRE);
+  if (p == nullptr) {  // first call on this device; a race between host threads only repeats the same lookup
+    void* sym = nullptr;
+    e = hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || sym == nullptr) {
+      set_error("%s: hipGetSymbolAddress(scratch) failed on device %d: %s", name, dev, hipGetErrorString(e));
+      return CK_ERR_LAUNCH;
+    }
+    p = static_cast<uint32_t*>(sym);
+    __atomic_store_n(&g_scratch_ptr[dev], p, __ATOMIC_RELEASE);
+  }
+  *out = p;
+  return CK_OK;
+}
+
+__global__ __launch_bounds__(kBlock) void zero_words_kernel(uint32_t* __restrict__ p, int words) {
+  const int i = blockIdx.x * kBlock + threadIdx.x;
+  if (i < words) p[i] = 0u;
+}
+
+}  // namespace
+}  // namespace ck
+
+extern "C" int ck_count_offsets(const void* ids, int32_t ids_are_i64, int64_t n, int32_t num_bins, uint32_t* counts,
+                                uint32_t* ends, uint32_t* starts, uint32_t* workspace, void* stream) {
+  return launch_count("ck_count_offsets", ids, ids_are_i64, n, num_bins, counts, ends, starts, workspace,
+                      static_cast<hipStream_t>(stream));
+}
+
+extern "C" int ck_count_offsets_static(const void* ids, int32_t ids_are_i64, int64_t n, int32_t num_bins, uint32_t* counts,
+                                       uint32_t* ends, uint32_t* starts, void* stream) {
+  const char* name = "ck_count_offsets_static";
+  CK_REQUIRE(num_bins >= 1 && num_bins <= kMaxCountBins,
+             "%s: num_bins=%d outside [1, %d] (the built-in workspace holds %d words)", name, num_bins, kMaxCountBins,
+             kScratchWords);
+  const int64_t words = ck_count_workspace_words(num_bins);
+  CK_REQUIRE(words <= kScratchWords, "%s: num_bins=%d needs %lld workspace words, the built-in workspace holds %d", name,
+             num_bins, (long long)words, kScratchWords);
+  uint32_t* ws = nullptr;
+  if (int rc = scratch_for_current_device(name, &ws)) return rc;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // The array keeps whatever the last call on this GPU left (zeros after a completed call, anything after one that was
+  // cut short): the words this call uses are cleared first, by a kernel, so that the sequence can be captured in a graph.
+  hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)ceil_div(words, kBlock)), dim3(kBlock), 0, s, ws, (int)words);
+  CK_CHECK_LAUNCH(name);
+  return launch_count(name, ids, ids_are_i64, n, num_bins, counts, ends, starts, ws, s);
 }
 
 extern "C" int64_t ck_sort_max_rows(int64_t R, int32_t E, int32_t align) {

@@ -47,6 +47,7 @@ _SIGNATURES = {
     "ck_abi_version": (c_int32, []),
     "ck_count_workspace_words": (c_int64, [c_int32]),
     "ck_count_offsets": (c_int32, [c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
+    "ck_count_offsets_static": (c_int32, [c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ck_route_topk_softmax": (c_int32, [c_void_p, c_int32, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ck_route_topk_softmax_bwd": (c_int32, [c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_void_p, c_int32, c_void_p]),
     "ck_sort_max_rows": (c_int64, [c_int64, c_int32, c_int32]),

@@ -51,6 +51,15 @@ int64_t ck_count_workspace_words(int32_t num_bins);
 int ck_count_offsets(const void* ids, int32_t ids_are_i64, int64_t n, int32_t num_bins, uint32_t* counts,
                      uint32_t* ends, uint32_t* starts, uint32_t* workspace, void* stream);
 
+/* ck_count_offsets for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc): no counterpart in the reference. Same arguments and results as ck_count_offsets without the
+ * workspace: the ticket and accumulators live in a 65,540-byte device array inside the library (one copy per GPU, held
+ * until the process ends), looked up once per device. The call clears the words it uses with a small kernel and then
+ * runs the same count kernel; it calls no hipMalloc / hipFree. num_bins above 16384 is rejected (CK_ERR_ARG).
+ * All calls on one GPU share that array: calls that overlap on one GPU (two streams, two host threads) race. */
+int ck_count_offsets_static(const void* ids, int32_t ids_are_i64, int64_t n, int32_t num_bins, uint32_t* counts,
+                            uint32_t* ends, uint32_t* starts, void* stream);
+
 /* ---------------------------------------------------------------------------------------------------------------
  * (b1) router: top-k over logits, softmax over the k selected logits
  * Replaces: MoE_Torch._get_topk + F.softmax(values.float()) --
