@@ -311,8 +311,10 @@ def secondary_hbm_kernels(dev):
     return out, configs
 
 
-def gemm_only(dev, launches: int):
-    """Just the c_fc-forward-shape grouped GEMM (grouped epilogue) at the C3 shape: the target of counter runs."""
+def gemm_only(dev, launches: int, stamps: bool = False):
+    """Just the c_fc-forward-shape grouped GEMM (grouped epilogue) at the C3 shape: the target of counter runs.
+    stamps: with a CK_STAMP measurement build (build.py --define CK_STAMP=1 --output libck_stamp.so, loaded through
+    CK_MI355_LIB), also print where a wave's cycles go: main loop, waiting for loads, waiting at the barrier, epilogue."""
     import numpy as np
     import torch
 
@@ -325,7 +327,14 @@ def gemm_only(dev, launches: int):
     seg = cute_kernels.sort_by_expert(ids.to(dev), E, 256)
     x = torch.randn(T, H, device=dev, dtype=torch.bfloat16)
     w = torch.randn(E, 2 * I, H, device=dev, dtype=torch.bfloat16) * 0.02
+    if os.environ.get("CK_BENCH_ZEROS") == "1":  # all-zero operands: the chip's clock under the same instruction stream
+        x.zero_()
+        w.zero_()
     y = torch.empty(seg.max_rows, 2 * I, device=dev, dtype=torch.bfloat16)
+    trace = None
+    if stamps:
+        trace = torch.zeros(8 * 8 * 20000, dtype=torch.int64, device=dev)
+        os.environ["CK_TRACE_PTR"] = hex(trace.data_ptr())  # read by the library at every call (stamp builds only)
     for _ in range(2):
         scattermoe._gemm(x, TOP_K, w, seg, _C.CK_EPI_GROUPED, y)
     s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -336,8 +345,23 @@ def gemm_only(dev, launches: int):
     torch.cuda.synchronize()
     ms = s.elapsed_time(e) / launches
     flops = 4.0 * R * H * I
-    print(json.dumps({"kernel": "grouped_gemm<grouped>", "shape": [R, 2 * I, H], "avg_launch_ms": ms,
-                      "TFLOP/s": flops / ms / 1e9, "frac_mfma": flops / ms / 1e9 / PEAK_BF16_TFLOPS}))
+    rec = {"kernel": "grouped_gemm<grouped>", "shape": [R, 2 * I, H], "avg_launch_ms": ms,
+           "TFLOP/s": flops / ms / 1e9, "frac_mfma": flops / ms / 1e9 / PEAK_BF16_TFLOPS}
+    if trace is not None:
+        t = trace.view(-1, 8).cpu().numpy().astype(np.float64)
+        t = t[t[:, 5] > 0]  # waves that ran a main loop
+        assert len(t) > 0, "no stamps: is CK_MI355_LIB a CK_STAMP build?"
+        tot = t[:, 0] + t[:, 1] + t[:, 4]
+        rec["stamps"] = {
+            "waves": int(len(t)), "k_steps": float(t[:, 5].mean()),
+            "cycles_per_wave": {"prologue": float(t[:, 0].mean()), "main_loop": float(t[:, 1].mean()),
+                                "load_wait": float(t[:, 2].mean()), "barrier_wait": float(t[:, 3].mean()),
+                                "epilogue": float(t[:, 4].mean())},
+            "share_of_tile": {"main_loop": float((t[:, 1] / tot).mean()), "load_wait": float((t[:, 2] / tot).mean()),
+                              "barrier_wait": float((t[:, 3] / tot).mean()), "epilogue": float((t[:, 4] / tot).mean())},
+            "main_loop_cycles_per_k_step": float((t[:, 1] / t[:, 5]).mean()),
+        }
+    print(json.dumps(rec))
 
 
 def library_gemm_yardstick(dev, iters: int = 10):
@@ -391,6 +415,8 @@ def main() -> int:
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device copy (outside the timed region): the known-size kernel that "
                     "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
+    ap.add_argument("--stamps", action="store_true",
+                    help="with --only-gemm and a CK_STAMP measurement build: print the per-wave cycle breakdown")
     ap.add_argument("--only-yardstick", action="store_true",
                     help="run only torch.matmul on the layer's per-expert shapes (the same-box library yardstick)")
     args = ap.parse_args()
@@ -406,7 +432,7 @@ def main() -> int:
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     if args.only_gemm > 0:
-        gemm_only(dev, args.only_gemm)
+        gemm_only(dev, args.only_gemm, args.stamps)
         return 0
     if args.only_yardstick:
         print(json.dumps({"library_gemm_yardstick": library_gemm_yardstick(dev)}))

@@ -39,6 +39,8 @@ struct GemmParams {
   const float* w_scale;  // fp8 only: per-output-channel scale of w, [E, N]
   int act_kind;          // kSwiglu epilogue: CK_ACT_SWIGLU (up * gate * sigmoid(gate)) or CK_ACT_GLU (up * sigmoid(gate))
   void* trace;           // measurement builds only: per-workgroup phase timestamps (8 x uint64 each), else NULL
+  int stagger_xcd;       // experiment: start delay of the first workgroup on each CU, in 10 ns units per XCD index ...
+  int stagger_cu;        // ... and per CU index within the XCD
 };
 
 // The 16-bit kernel with 128-byte LDS rows (grouped_gemm_line.hip): 256 x bn tiles, bn = 256 or 384, contraction length a
@@ -84,6 +86,40 @@ struct Mfma<f16_t> {
     return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
   }
 };
+
+// v_mfma_f32_16x16x32: A lane l holds row l % 16, contraction values 8 (l / 16) .. + 7; B likewise for column l % 16; the
+// result register s of lane l is row 4 (l / 16) + s, column l % 16. On N(0,1) operands a register-only loop of this
+// shape sustains about 2.0 PFLOP/s where the 32x32x16 shape sustains 1.7 (the clock is power-managed), hence its use in
+// the 128-byte-row kernel.
+template <typename T>
+struct Mfma16;
+// run_acc: the same instruction with the accumulator pinned to the accumulation registers (AGPRs) and updated in place.
+// With one wave per SIMD a kernel has 256 of them next to its 256 vector registers; left to choose, the register
+// allocator spreads 256 accumulator values over both files and shuffles them at every loop boundary. The instruction is
+// opaque to the compiler's hazard checks: a caller that reads the accumulators with vector instructions afterwards
+// waits out the MFMA write latency itself (mfma_drain).
+template <>
+struct Mfma16<bf16_t> {
+  typedef bf16x8 frag;
+  __device__ static inline f32x4 run(const frag& a, const frag& b, const f32x4& c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+  __device__ static inline void run_acc(const frag& a, const frag& b, f32x4& c) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+};
+template <>
+struct Mfma16<f16_t> {
+  typedef f16x8 frag;
+  __device__ static inline f32x4 run(const frag& a, const frag& b, const f32x4& c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
+  }
+  __device__ static inline void run_acc(const frag& a, const frag& b, f32x4& c) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+};
+// after the last run_acc, before anything else reads the accumulators: longer than any MFMA's result latency
+__device__ inline void mfma_drain() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
 
 // f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant expression
 template <int N, typename F>

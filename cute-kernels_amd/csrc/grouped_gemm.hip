@@ -39,28 +39,13 @@ const bool g_eight_waves = [] {
   return !(env != nullptr && env[0] == '4');
 }();
 
-// CK_GEMM_LINE=0 in the environment keeps every launch on the kernels of this file (A/B measurements); CK_GEMM_TILE=256 /
-// 384 forces the width of the 128-byte-row kernel's tile. Both are read per call, so tests can switch them in-process.
+// CK_GEMM_LINE=0 in the environment keeps every launch on the kernels of this file (A/B measurements); read per call, so
+// tests can switch it in-process.
 inline bool line_kernel_enabled() {
   const char* env = getenv("CK_GEMM_LINE");
   return !(env != nullptr && env[0] == '0');
 }
-inline int forced_tile() {
-  const char* env = getenv("CK_GEMM_TILE");
-  return env == nullptr ? 0 : atoi(env);
-}
 
-// 256 x 384 tiles carry 20 % more FLOPs per byte loaded from L2 but pay more for the ragged column edge and for their
-// (longer) epilogue: they serve long contractions, when the padded column count does not eat the gain.
-// `cols` output columns, `narrow` / `wide` columns per tile, `contraction`: (average) K.
-inline int line_tile_width(int64_t cols, int narrow, int wide, int64_t contraction) {
-  if (forced_tile() == 256) return 256;
-  if (forced_tile() == 384) return 384;
-  if (contraction < 2048) return 256;  // short contractions are dominated by the per-tile epilogue: more, smaller tiles
-  const double util_narrow = (double)cols / (double)(ceil_div(cols, narrow) * narrow);
-  const double util_wide = (double)cols / (double)(ceil_div(cols, wide) * wide);
-  return util_wide * 1.05 > util_narrow ? 384 : 256;
-}
 
 // PIPE 0: K step 64, global -> registers -> padded LDS, two stages (any K % 8 == 0).
 // PIPE 1: K step 32, global -> LDS directly (no register staging), four XOR-swizzled stages, loads three steps ahead
@@ -817,7 +802,7 @@ extern "C" int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* 
   prm.ld_t = ld_t;
   prm.aux = aux;
   prm.aux_in = aux_in;
-#if (CK_ABLATE & 256)
+#if (CK_ABLATE & 256) || defined(CK_STAMP)
   if (const char* t = getenv("CK_TRACE_PTR")) prm.trace = reinterpret_cast<void*>(strtoull(t, nullptr, 16));
 #endif
   int out_cols = N;  // columns that tile along the grid
@@ -838,8 +823,7 @@ extern "C" int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* 
              "(align = 256, K %% 64 == 0)", name);
   if (line_kernel) {
     const bool swiglu = epilogue == CK_EPI_SWIGLU;
-    const int bn = epilogue == CK_EPI_SCATTER ? line_tile_width(out_cols, 256, 384, K >= 8192 ? K : 0)
-                                              : (forced_tile() == 384 ? 384 : 256);
+    const int bn = 256;
     prm.n_tiles = (int)ceil_div(out_cols, swiglu ? bn / 2 : bn);
     const int64_t line_blocks = m_tiles * prm.n_tiles;
     CK_REQUIRE(line_blocks < (int64_t)0x7fffffff, "%s: grid too large", name);
@@ -950,14 +934,14 @@ extern "C" int ck_grouped_gemm_dw(const void* a_t, const void* b_t, int64_t ld_t
   prm.tile_expert = seg->tile_expert;
   prm.row_slot = seg->row_slot;
   prm.y = dw;
-#if (CK_ABLATE & 256)
+#if (CK_ABLATE & 256) || defined(CK_STAMP)
   if (const char* t = getenv("CK_TRACE_PTR")) prm.trace = reinterpret_cast<void*>(strtoull(t, nullptr, 16));
 #endif
   hipStream_t s = static_cast<hipStream_t>(stream);
   // tile size follows the problem, not the segment alignment: small weight matrices get 128x128 tiles
   const bool big = (M >= 1024 && N >= 1024);
   if (big && !g_force_pipe0 && line_kernel_enabled()) {
-    const int bn = line_tile_width(N, 256, 384, seg->max_rows / seg->num_experts);
+    const int bn = 256;
     prm.m_tiles = (int)ceil_div(M, kLineBM);
     prm.n_tiles = (int)ceil_div(N, bn);
     const int64_t line_blocks = (int64_t)prm.m_tiles * prm.n_tiles * seg->num_experts;

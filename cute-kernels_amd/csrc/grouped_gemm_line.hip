@@ -1,5 +1,5 @@
 // Scattered grouped GEMM with 128-byte LDS rows: 256 x BN block tiles (BN = 256 or 384), bf16 / f16 inputs, fp32
-// accumulation.
+// accumulation on v_mfma_f32_16x16x32.
 //
 // Why 128-byte rows: the grouped GEMMs are bound by L2 -> LDS load throughput, and that throughput depends on how many
 // contiguous bytes a tile row fetches per request: measured chip-wide on L2-resident panels, global_load_lds_dwordx4
@@ -7,64 +7,87 @@
 // elements = one 128-byte line per tile row. A stage is then 64 KiB (BN = 256) or 80 KiB (BN = 384), and two stages fill
 // the LDS: step kt multiplies out of one stage while the loads of step kt + 1 fill the other.
 //
-// Workgroup = 8 waves (two per SIMD) in a 4 x 2 grid, wave tile 64 x BN/2 = 2 x (BN/64) v_mfma_f32_32x32x16 blocks.
-// Fragments rotate through the four 16-wide slices of a step. BN = 384 has registers for one fragment set: a register is
-// reloaded for the next slice as soon as the last MFMA that reads it has issued. BN = 256 keeps two sets and reads the
-// next slice's fragments a whole slice ahead. One barrier per step, in front of the last slice: by then
-// every wave has read the whole current stage (its last-slice fragments are in registers) and the next stage has landed,
-// so the loads of step kt + 2 go out under the last slice's MFMAs, as do the fragment reads of step kt + 1.
+// Why 16x16x32 blocks: the chip's clock is power-managed and the 16x16x32 instruction costs less energy per FLOP on
+// random operands than 32x32x16 (register-only loops on N(0,1) data: 2.04 against 1.70 PFLOP/s).
+//
+// Workgroup = WGM x 2 waves: 4 x 2 (eight waves, two per SIMD, wave tile 64 x BN/2) or 2 x 2 (four waves, one per SIMD,
+// wave tile 128 x 128 with the accumulators in AGPRs: a third less LDS fragment traffic per FLOP). A K step is two
+// 32-wide slices; a slice is MI x NI MFMAs on MI + NI 16-byte fragments. One barrier per step, in front of the last
+// slice: by then every wave has read the whole current stage (its last-slice fragments are in registers) and the next
+// stage has landed, so the loads of step kt + 2 go out under the last slice's MFMAs (spread over the slice), as do the
+// fragment reads of step kt + 1.
 // BN = 384 carries 20 % more FLOPs per loaded byte (153.6 against 128) and is used where the contraction is long.
 #include <stdlib.h>
 
 #include "gemm_common.h"
 
 #ifndef CK_ABLATE
-#define CK_ABLATE 0  // measurement builds only: 1 no barrier, 2 no loads in the loop, 4 no fragment reads, 8 no wait for the loads, 16 every step loads the first two K steps again (L2 hits), 32 no epilogue, 64 no MFMA, 128 no row-major output stores, 512 single fragment set at BN = 256
+#define CK_ABLATE 0  // measurement builds only (build.py --define CK_ABLATE=n --output ...): 1 no barrier, 2 no loads in the loop, 4 no fragment reads, 8 no wait for the loads, 16 every step loads the first two K steps again (L2 hits), 32 no epilogue, 64 no MFMA, 128 no row-major output stores
+#endif
+
+#ifndef CK_LOAD_GAP
+#define CK_LOAD_GAP 0  // measurement builds only: MFMAs between two loads of the next-but-one K step (0: spread over the whole last slice)
+#endif
+#ifndef CK_READ_GAP
+#define CK_READ_GAP 0  // measurement builds only: MFMAs between two fragment reads of the two-set schedule (default 1: the reads go out behind the first MI + NI MFMAs)
+#endif
+#ifndef CK_STAMP
+#define CK_STAMP 0  // measurement builds only: 1 = every wave adds up the cycles it spends waiting for the loads and at the barrier of each K step and writes them, with its main-loop and epilogue cycles, to GemmParams::trace
 #endif
 
 namespace ck {
 namespace {
 
 constexpr int BM = 256;
-constexpr int WGM = 4;                     // waves along M (always 2 along N)
-constexpr int NW = 2 * WGM, NT = 64 * NW;
-constexpr int WM = BM / WGM, MI = WM / 32;  // 64-row wave tile: 2 row blocks
-constexpr int BK = 64, KS = BK / 16, NSTAGE = 2;
+constexpr int BK = 64, KS = BK / 32, NSTAGE = 2;
 constexpr int kRowBytes = BK * 2;  // 128: one cache line per tile row and K step
-constexpr int A_LD = BM * kRowBytes / (1024 * NW);  // 1 KiB wave-loads per wave and K step
-static_assert(MI == 2, "the slice schedule below is written for two A row blocks per wave");
+static_assert(KS == 2, "a K step is two 32-wide slices");
 
 // 16-byte chunk c of row r sits in slot c ^ swz128(r): 16 lanes reading one chunk index of 16 consecutive rows (one phase
 // of a ds_read_b128) then touch all 64 banks once -- even rows cover banks 0-31 with 8 distinct slots, odd rows 32-63.
 __device__ inline int swz128(int row) { return (row >> 1) & 7; }
 
-template <int BN>
+template <int BN, int WGM>
 struct Tile {
-  static constexpr int WN = BN / 2, NI = WN / 32;
+  static constexpr int NW = 2 * WGM, NT = 64 * NW;   // waves: WGM along M, 2 along N
+  static constexpr int WM = BM / WGM, MI = WM / 16;  // wave tile rows: 64 (4 row blocks) or 128 (8)
+  static constexpr int WN = BN / 2, NI = WN / 16;
   static constexpr int kStageBytes = (BM + BN) * kRowBytes;
+  static constexpr int A_LD = BM * kRowBytes / (1024 * NW);  // 1 KiB wave-loads per wave and K step
   static constexpr int B_LD = BN * kRowBytes / (1024 * NW);
   static constexpr int kLoadsPerStep = A_LD + B_LD;
   static constexpr size_t kLdsBytes = (size_t)NSTAGE * kStageBytes;
-  // epilogue: slab of half the tile's columns (half of each wave's column blocks), kept transposed S[col][row]
-  static constexpr int kSlabBlocks = NI / 2, kSlabCols = 2 * kSlabBlocks * 32, kSlabLd = BM + 4;
-  static constexpr int kMetaOffset = kSlabCols * kSlabLd * 2;  // after the slab: output row of every tile row (scatter)
+  // two fragment sets (the next slice is read a whole slice ahead) where the registers allow: 512 per lane with one
+  // wave per SIMD, 256 with two
+  static constexpr bool kDouble = WGM == 2;  // (contraction-strided operands: see the kernel)
   static_assert(kLdsBytes <= 160 * 1024, "two stages fit the LDS of a CU");
-  static_assert(kMetaOffset % 16 == 0 && kMetaOffset + BM * 4 <= (int)kLdsBytes, "slab and row table fit in the dead stages");
-  static_assert(kLoadsPerStep <= 2 * NI, "every load of a step has an MFMA of the last slice to hide behind");
+  static_assert(kLoadsPerStep <= MI * NI, "every load of a step has an MFMA of the last slice to hide behind");
+  static_assert(NI % 4 == 0, "whole column-block pairs in each half of a wave's columns");
+  static_assert(NT >= BM, "one thread per tile row");
 };
 
 // BT ("B as stored by its owner"): the weight operand is [contraction, columns] row-major, i.e. contraction-strided --
 // the input-gradient GEMMs read W[e] [out, in] this way instead of a transposed copy. Its stage holds 64 contraction rows
 // of BN columns, and fragments come out of LDS through ds_read_b64_tr_b16 (see read_b).
-template <typename T, int MODE, int BN, bool BT>
-__global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams prm) {
-  typedef Tile<BN> TL;
+// EXTRA: the launch has a bias operand or a transposed side output (y_t); the instantiations without them carry none of
+// that code (it cost the common launches spills, and every spill reload waits for the output stores in flight).
+template <typename T, int MODE, int BN, bool BT, int WGM, bool EXTRA>
+__global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const GemmParams prm) {
+  typedef Tile<BN, WGM> TL;
+  constexpr int NW = TL::NW, NT = TL::NT, WM = TL::WM, MI = TL::MI, A_LD = TL::A_LD;
   constexpr int WN = TL::WN, NI = TL::NI, B_LD = TL::B_LD, kLoadsPerStep = TL::kLoadsPerStep, kStageBytes = TL::kStageBytes;
-  constexpr int kSlabBlocks = TL::kSlabBlocks, kSlabCols = TL::kSlabCols, kSlabLd = TL::kSlabLd, kMetaOffset = TL::kMetaOffset;
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   char* lds_c = reinterpret_cast<char*>(lds_raw);
-  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int tid = threadIdx.x, lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);  // uniform: everything derived from it stays in scalar registers
   const int wm = wave >> 1, wn = wave & 1;
+  if ((prm.stagger_xcd | prm.stagger_cu) != 0 && blockIdx.x < 256) {  // experiment: phase-shift the CUs' tile loops
+    const uint64_t t0 = wall_clock64();
+    const uint64_t wait = (uint64_t)(blockIdx.x % kXcds) * prm.stagger_xcd + (uint64_t)(blockIdx.x / kXcds) * prm.stagger_cu;
+    while (wall_clock64() - t0 < wait) __builtin_amdgcn_s_sleep(8);
+  }
+  [[maybe_unused]] uint64_t st_begin = 0, st_loop = 0, st_end = 0, st_vm = 0, st_bar = 0;
+  if constexpr (CK_STAMP != 0) st_begin = clock64();
 
   // ---- which tile (same XCD-aware orders as the 256 x 256 kernel)
   int mt, nt, expert;
@@ -108,15 +131,14 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
   if constexpr (MODE == kScatter) {
     if (tid < BM && m0 + tid < valid_end) scatter_row = prm.row_slot[m0 + tid];
   }
-  static_assert(NT >= BM, "one thread per tile row");
 
-  f32x16 acc[MI][NI];
+  f32x4 acc[MI][NI];
 #pragma unroll
   for (int i = 0; i < MI; ++i)
 #pragma unroll
     for (int j = 0; j < NI; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 
   // ---- global -> LDS addressing: lane l of a wave-load fills slot l (16 bytes) of 64 consecutive slots = 8 rows of 128 B;
   // the lane fetches the chunk that belongs in its slot, so the 8 lanes of a row read one whole line of global memory
@@ -136,13 +158,16 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
   }
   constexpr int kAtRowBytes = BM * 2;
   auto swap02 = [](int w) { return (w & ~5) | ((w & 1) << 2) | ((w >> 2) & 1); };
+  // contraction-strided stages (64 contraction rows of 256 columns): 32-byte window q (16 columns) of row n sits at
+  // window position swap02(q) ^ tr_swz(n) of the row
+  auto tr_swz = [](int n) { return (n & 3) | (((n >> 3) & 1) << 2); };
   uint32_t a_off[A_LD], b_off[B_LD];
 #pragma unroll
   for (int t = 0; t < A_LD; ++t) {
     if constexpr (AT) {
       const int pos = (wave * A_LD + t) * 1024 + lane * 16;  // byte position of this lane's slot in the A stage
       const int n = pos / kAtRowBytes, slot16 = (pos % kAtRowBytes) / 16;
-      const int q = swap02((slot16 >> 1) ^ (n & 3));
+      const int q = swap02((slot16 >> 1) ^ tr_swz(n));
       int64_t col = m0 + (2 * q + (slot16 & 1)) * 8;
       if (col >= prm.M) col = m0;  // ragged edge: re-read a valid chunk, never stored
       a_off[t] = (uint32_t)(((int64_t)n * prm.lda + col) * 2);
@@ -162,16 +187,17 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
       a_off[t] = (uint32_t)((row * prm.lda + k_begin) * 2 + c * 16);
     }
   }
-  // BT: 32-byte window q of contraction row n sits at window position swap02(q) ^ (n & 3) of the row (swap02 exchanges
-  // bits 0 and 2 of the window index): the 4 rows x 32 bytes one 16-lane group of a transposing read touches fill one
-  // 128-byte block, and the neighbouring group (next 16 columns) falls into the other half of the banks.
+  // BT: 32-byte window q of contraction row n sits at window position swap02(q) ^ tr_swz(n) of the row (swap02 exchanges
+  // bits 0 and 2 of the window index, tr_swz(n) = bits 0-1 of n and bit 3 of n moved to bit 2): the 4 rows x 32 bytes one
+  // 16-lane group of a transposing read touches fill one 128-byte block, and the neighbouring group (the same columns 8
+  // contraction rows further down) falls into the other half of the banks.
   constexpr int kBtRowBytes = BN * 2, kBtWindows = kBtRowBytes / 32;
 #pragma unroll
   for (int t = 0; t < B_LD; ++t) {
     if constexpr (BT) {
       const int pos = (wave * B_LD + t) * 1024 + lane * 16;  // byte position of this lane's slot in the B stage
       const int n = pos / kBtRowBytes, slot16 = (pos % kBtRowBytes) / 16;
-      const int q = swap02((slot16 >> 1) ^ (n & 3));           // the window that belongs at this position
+      const int q = swap02((slot16 >> 1) ^ tr_swz(n));         // the window that belongs at this position
       int64_t col = (int64_t)nt * BN + (2 * q + (slot16 & 1)) * 8;
       if (col >= prm.N) col = (int64_t)nt * BN;                // ragged edge: re-read a valid chunk, never stored
       b_off[t] = (uint32_t)(((int64_t)n * prm.ldw + col) * 2);
@@ -192,9 +218,18 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
   static_assert(!BT || kBtWindows % 8 == 0 || kBtWindows == 24, "window swizzle works on groups of 8 windows");
   const int nk = k_len / BK;
 
-  auto dma16 = [&](const char* src, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(src) : "m0");
+  // One 1 KiB wave-load: scalar base (the operand at this K step, uniform over the wave) + the lane's 32-bit byte offset,
+  // so that a load costs no vector arithmetic (a 64-bit vector add per load delayed the MFMA behind it)
+  auto dma16 = [&](const char* base, uint32_t off, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(off), "s"(base) : "m0");
   };
+  auto uniform_ptr = [](const char* p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
+  };
+  const char* a_base_u = uniform_ptr(a_base);
+  const char* b_base_u = uniform_ptr(b_base);
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds_c;
   const uint32_t wave_a = __builtin_amdgcn_readfirstlane(lds_base + wave * A_LD * 1024);
   const uint32_t wave_b = __builtin_amdgcn_readfirstlane(lds_base + BM * kRowBytes + wave * B_LD * 1024);
@@ -203,74 +238,74 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
     const int64_t kb_b = BT ? (int64_t)((CK_ABLATE & 16) ? (step & 1) : step) * BK * prm.ldw * 2 : kb;  // BT: 64 contraction rows further down
     const int64_t kb_a = AT ? (int64_t)step * BK * prm.lda * 2 : kb;
     const uint32_t st = (uint32_t)((step & (NSTAGE - 1)) * kStageBytes);
-    if (g < A_LD) dma16(a_base + kb_a + a_off[g], wave_a + st + g * 1024);
-    else dma16(b_base + kb_b + b_off[g - A_LD], wave_b + st + (g - A_LD) * 1024);
+    if (g < A_LD) dma16(a_base_u + kb_a, a_off[g], wave_a + st + g * 1024);
+    else dma16(b_base_u + kb_b, b_off[g - A_LD], wave_b + st + (g - A_LD) * 1024);
   };
   auto issue = [&](int step) {
 #pragma unroll
     for (int g = 0; g < kLoadsPerStep; ++g) issue_one(step, g);
   };
 
-  // ---- fragments: slice sl of a row is its 16-byte chunks 2 sl (lanes 0-31) and 2 sl + 1 (lanes 32-63)
-  typedef typename Mfma<T>::frag frag_t;
-  const int fsw = swz128(lane & 31), fh = lane >> 5;
+  // ---- fragments: slice sl of a row is its 16-byte chunks 4 sl + lane / 16 (the lane's 8 contraction values)
+  typedef typename Mfma16<T>::frag frag_t;
+  const int fsw = swz128(lane & 15), fq = lane >> 4;
   int slice_off[KS];
 #pragma unroll
-  for (int sl = 0; sl < KS; ++sl) slice_off[sl] = ((2 * sl + fh) ^ fsw) * 16;
-  const int fa_row = (wm * WM + (lane & 31)) * kRowBytes;
-  const int fb_row = BM * kRowBytes + (wn * WN + (lane & 31)) * kRowBytes;
-  // 256-wide tiles have the registers for two fragment sets: the reads for the next slice then go out a whole slice ahead
-  constexpr bool kDouble = BN == 256 && (CK_ABLATE & 512) == 0;  // (measured: 2.5 to 3.5 % faster launches)
+  for (int sl = 0; sl < KS; ++sl) slice_off[sl] = ((4 * sl + fq) ^ fsw) * 16;
+  const int fa_row = (wm * WM + (lane & 15)) * kRowBytes;
+  const int fb_row = BM * kRowBytes + (wn * WN + (lane & 15)) * kRowBytes;
+  constexpr bool kDouble = TL::kDouble;
   constexpr int kSets = kDouble ? 2 : 1;
   frag_t fa[kSets][MI], fb[kSets][NI];
   typedef __attribute__((__vector_size__(4 * sizeof(short)))) short tr16x4;
+  // Contraction-strided stages. Lane l = 16 g + i of a transposing read points at 4 consecutive columns (4 (i % 4) ..) of
+  // contraction row i / 4 of a 4-row x 16-column patch and receives the 4 rows of column i; two reads (rows +0..3,
+  // +4..7 of the lane group's 8 rows 8 g ..) make the 8 contraction values 8 g .. 8 g + 7 of column i -- the MFMA's layout.
+  // Rows 8 g + (i / 4) (+ 4): tr_swz = (i / 4) ^ 4 (g % 2) for both reads' rows up to the +4, which leaves bits 0-1 and 3.
   int at_off[MI];
-  if constexpr (AT) {  // as bt_off below, on the A stage
+  if constexpr (AT) {
     const int g = lane >> 4, i = lane & 15, n_low = i >> 2;
 #pragma unroll
     for (int b = 0; b < MI; ++b) {
-      const int q = (wm * WM + b * 32) / 16 + (g & 1);
-      at_off[b] = (8 * (g >> 1) + n_low) * kAtRowBytes + (swap02(q) ^ n_low) * 32 + 8 * (i & 3);
+      const int q = (wm * WM + b * 16) / 16;
+      at_off[b] = (8 * g + n_low) * kAtRowBytes + (swap02(q) ^ (n_low | ((g & 1) << 2))) * 32 + 8 * (i & 3);
     }
   }
-  auto read_a = [&](int stage, int sl, int i) {
+  auto read_a = [&](int set, int stage, int sl, int i) {
     if constexpr (AT) {
-      const char* p = lds_c + stage * kStageBytes + at_off[i] + 16 * sl * kAtRowBytes;
+      const char* p = lds_c + stage * kStageBytes + at_off[i] + 32 * sl * kAtRowBytes;
       union {
         tr16x4 h[2];
         frag_t f;
       } u;
       u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr16x4 __attribute__((address_space(3)))*)(p));
       u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr16x4 __attribute__((address_space(3)))*)(p + 4 * kAtRowBytes));
-      fa[kDouble ? (sl & 1) : 0][i] = u.f;
+      fa[set][i] = u.f;
     } else {
-      fa[kDouble ? (sl & 1) : 0][i] = *reinterpret_cast<const frag_t*>(lds_c + stage * kStageBytes + slice_off[sl] + fa_row + i * 32 * kRowBytes);
+      fa[set][i] = *reinterpret_cast<const frag_t*>(lds_c + stage * kStageBytes + slice_off[sl] + fa_row + i * 16 * kRowBytes);
     }
   };
-  // BT: lane l = 16 g + i of a transposing read points at 4 consecutive columns (4 (i % 4) ..) of contraction row i / 4
-  // of a 4-row x 16-column patch and receives the 4 rows of column i; two reads (rows +0..3, +4..7) make the 8 contraction
-  // values of column 16 (g % 2) + i for k-half g / 2 -- the MFMA's B layout.
   int bt_off[NI];
   if constexpr (BT) {
     const int g = lane >> 4, i = lane & 15, n_low = i >> 2;
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
-      const int q = (wn * WN + j * 32) / 16 + (g & 1);
-      bt_off[j] = BM * kRowBytes + (8 * (g >> 1) + n_low) * kBtRowBytes + (swap02(q) ^ n_low) * 32 + 8 * (i & 3);
+      const int q = (wn * WN + j * 16) / 16;
+      bt_off[j] = BM * kRowBytes + (8 * g + n_low) * kBtRowBytes + (swap02(q) ^ (n_low | ((g & 1) << 2))) * 32 + 8 * (i & 3);
     }
   }
-  auto read_b = [&](int stage, int sl, int j) {
+  auto read_b = [&](int set, int stage, int sl, int j) {
     if constexpr (BT) {
-      const char* p = lds_c + stage * kStageBytes + bt_off[j] + 16 * sl * kBtRowBytes;
+      const char* p = lds_c + stage * kStageBytes + bt_off[j] + 32 * sl * kBtRowBytes;
       union {
         tr16x4 h[2];
         frag_t f;
       } u;
       u.h[0] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr16x4 __attribute__((address_space(3)))*)(p));
       u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr16x4 __attribute__((address_space(3)))*)(p + 4 * kBtRowBytes));
-      fb[kDouble ? (sl & 1) : 0][j] = u.f;
+      fb[set][j] = u.f;
     } else {
-      fb[kDouble ? (sl & 1) : 0][j] = *reinterpret_cast<const frag_t*>(lds_c + stage * kStageBytes + slice_off[sl] + fb_row + j * 32 * kRowBytes);
+      fb[set][j] = *reinterpret_cast<const frag_t*>(lds_c + stage * kStageBytes + slice_off[sl] + fb_row + j * 16 * kRowBytes);
     }
   };
   auto mfma = [&](int set, int i, int j) {
@@ -278,7 +313,9 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
       asm volatile("" ::"v"(fa[set][i]), "v"(fb[set][j]));
       return;
     }
-    acc[i][j] = Mfma<T>::run(fa[set][i], fb[set][j], acc[i][j]);
+    // weight fragment first: a lane gets 4 consecutive output columns of one row
+    if constexpr (WGM == 2) Mfma16<T>::run_acc(fb[set][j], fa[set][i], acc[i][j]);
+    else acc[i][j] = Mfma16<T>::run(fb[set][j], fa[set][i], acc[i][j]);
   };
 
   // AT: contraction rows past the expert's count (the ragged end of its last K step) hold whatever the buffers hold.
@@ -302,6 +339,7 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
     }
   };
 
+  if constexpr (CK_STAMP != 0) st_loop = clock64();
   if (nk > 0) {
     issue(0);
     if (nk > 1) {
@@ -313,19 +351,22 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
       asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }
 #pragma unroll
-    for (int i = 0; i < MI; ++i) read_a(0, 0, i);
+    for (int i = 0; i < MI; ++i) read_a(0, 0, 0, i);
 #pragma unroll
-    for (int j = 0; j < NI; ++j) read_b(0, 0, j);
+    for (int j = 0; j < NI; ++j) read_b(0, 0, 0, j);
 
-    // One 16-wide slice: 2 * NI MFMAs, A row block 0 then 1, and the reloads for the slice after it (ns, nsl): fa[0] once
-    // row block 0 is done, fb[j] after the MFMA (1, j), fa[1] at the end.
-    // Slices 0 .. 2 of a step: the next slice is in the same stage.
-    // Slice 3: the next slice is slice 0 of step kt + 1 in the other stage. Phase 0 / 1: wait for that stage
-    //   (the only loads in flight) and for this wave's own fragment reads, then meet the other waves -- the whole current
-    //   stage has been read by everyone, so in phase 0 the loads of step kt + 2 overwrite it under this slice's MFMAs.
-    //   Phase 1 is step nk - 2 (nothing left to fetch), phase 2 the last step (nothing to wait for, nothing to reload).
+    // One 32-wide slice: MI x NI MFMAs, row block by row block, and the fragment reads for the slice after it (ns, nsl).
+    // Two fragment sets: the reads go out one after each of the first MI + NI MFMAs, in the order the next slice needs
+    // them. One set: fa[i] is reloaded once row block i is done, fb[j] after the MFMA (MI - 1, j).
+    // Slice 0 of a step: the next slice is in the same stage.
+    // Slice 1: the next slice is slice 0 of step kt + 1 in the other stage. Phase 0 / 1: wait for that stage (the only
+    //   loads in flight) and for this wave's own fragment reads, then meet the other waves -- the whole current stage has
+    //   been read by everyone, so in phase 0 the loads of step kt + 2 overwrite it under this slice's MFMAs, one load
+    //   every kLoadGap MFMAs. Phase 1 is step nk - 2 (nothing left to fetch), phase 2 the last step (nothing to wait
+    //   for, nothing to reload).
+    constexpr int kLoadGap = CK_LOAD_GAP > 0 ? CK_LOAD_GAP : (MI * NI) / kLoadsPerStep;
     auto slice = [&](int kt, auto sl, auto phase, auto idle) {
-      constexpr bool kIdle = decltype(idle)::value;  // this wave's 64 rows are all pad rows: no fragments, no MFMAs
+      constexpr bool kIdle = decltype(idle)::value;  // this wave's rows are all pad rows: no fragments, no MFMAs
       constexpr bool kLast = decltype(sl)::value == KS - 1;
       constexpr int kPhase = decltype(phase)::value;
       const int ns = kLast ? (kt + 1) & (NSTAGE - 1) : kt & (NSTAGE - 1);
@@ -338,47 +379,40 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
           asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
           zero_pad_slots(kt + 1);
           asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        } else if constexpr (CK_STAMP != 0) {
+          asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+          const uint64_t t0 = clock64();
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          const uint64_t t1 = clock64();
+          asm volatile("s_barrier" ::: "memory");
+          const uint64_t t2 = clock64();
+          st_vm += t1 - t0;
+          st_bar += t2 - t1;
         } else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       }
       constexpr int cur = kDouble ? (decltype(sl)::value & 1) : 0;
-      if constexpr (kDouble) {
-        // reads for the next slice in the order it needs them, one after each of the first MI + NI MFMAs
-        auto reload = [&](int n) {
-          if (n == 0) read_a(ns, nsl, 0);
-          else if (n <= NI) read_b(ns, nsl, n - 1);
-          else read_a(ns, nsl, 1);
-        };
+      constexpr int nxt = kDouble ? (cur ^ 1) : 0;
 #pragma unroll
-        for (int n = 0; n < 2 * NI; ++n) {
-          if constexpr (!kIdle) mfma(cur, n / NI, n % NI);
-          if constexpr (kLast && kPhase == 0 && !(CK_ABLATE & 2)) {
-            if (n < kLoadsPerStep) issue_one(kt + 2, n);
-          }
-          __builtin_amdgcn_sched_barrier(0);
-          if constexpr (kReload) {
-            if (n < MI + NI) reload(n);
+      for (int n = 0; n < MI * NI; ++n) {
+        const int i = n / NI, j = n % NI;
+        if constexpr (!kIdle) mfma(cur, i, j);
+        if constexpr (kLast && kPhase == 0 && !(CK_ABLATE & 2)) {
+          if (n % kLoadGap == 0 && n / kLoadGap < kLoadsPerStep) issue_one(kt + 2, n / kLoadGap);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        if constexpr (kReload) {
+          if constexpr (kDouble) {  // one read every kReadGap MFMAs, in the order the next slice needs them
+            constexpr int kReadGap = CK_READ_GAP > 0 ? CK_READ_GAP : 1;
+            if (n % kReadGap == 0 && n / kReadGap < MI + NI) {
+              const int r = n / kReadGap;
+              if (r < MI) read_a(nxt, ns, nsl, r);
+              else read_b(nxt, ns, nsl, r - MI);
+            }
+          } else {
+            if (j == NI - 1) read_a(0, ns, nsl, i);
+            if (i == MI - 1) read_b(0, ns, nsl, j);
           }
         }
-      } else {
-#pragma unroll
-        for (int j = 0; j < NI; ++j) {
-          if constexpr (!kIdle) mfma(0, 0, j);
-          if constexpr (kLast && kPhase == 0 && !(CK_ABLATE & 2)) {
-            if (j < kLoadsPerStep) issue_one(kt + 2, j);
-          }
-          __builtin_amdgcn_sched_barrier(0);
-        }
-        if constexpr (kReload) read_a(ns, nsl, 0);
-#pragma unroll
-        for (int j = 0; j < NI; ++j) {
-          if constexpr (!kIdle) mfma(0, 1, j);
-          if constexpr (kLast && kPhase == 0 && !(CK_ABLATE & 2)) {
-            if (NI + j < kLoadsPerStep) issue_one(kt + 2, NI + j);
-          }
-          __builtin_amdgcn_sched_barrier(0);
-          if constexpr (kReload) read_b(ns, nsl, j);
-        }
-        if constexpr (kReload) read_a(ns, nsl, 1);
       }
       __builtin_amdgcn_sched_barrier(0);
     };
@@ -389,240 +423,242 @@ __global__ __launch_bounds__(NT) void grouped_gemm_line_kernel(const GemmParams 
       if (kt + 2 == nk) k_step(kt++, std::integral_constant<int, 1>{});
       k_step(kt, std::integral_constant<int, 2>{});
     };
-    // A wave whose 64 tile rows all lie past the expert's last row (the tile is the ragged end of a segment) still
-    // issues its share of the loads and meets every barrier, but multiplies nothing: the wave it shares a SIMD with
-    // then has the matrix pipe to itself. Its accumulators stay zero and its rows are never stored.
+    // A wave whose tile rows all lie past the expert's last row (the tile is the ragged end of a segment) still issues
+    // its share of the loads and meets every barrier, but multiplies nothing: the wave it shares a SIMD with then has
+    // the matrix pipe to itself. Its accumulators stay zero and its rows are never stored.
     bool wave_idle = false;
     if constexpr (MODE != kDw) wave_idle = m0 + wm * WM >= valid_end;
     if (__builtin_amdgcn_readfirstlane(wave_idle)) k_loop(std::true_type{});
     else k_loop(std::false_type{});
   }
 
-  // ---- epilogue through LDS. Lane holds, per 32x32 block and q in 0..3, rows 8q + 4*(lane/32) + 0..3 of column lane%32:
-  // 8-byte writes into the transposed slab; ds_read_b64_tr_b16 brings row-major 16-byte pieces back out (a lane ends up
-  // with 8 consecutive columns of one row); transposed outputs leave with plain 16-byte reads.
-  typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4;
-  T* slab = reinterpret_cast<T*>(lds_raw);
-  int* scatter_rows = reinterpret_cast<int*>(lds_c + kMetaOffset);
-  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave is done with the stages
-  if constexpr (MODE == kScatter) {
-    if (tid < BM) scatter_rows[tid] = scatter_row;  // first read after the first slab barrier below
-  }
-  const int col_in_block = lane & 31;
-  const int row_quad = (lane >> 5) * 4;
-  const T kZero = Elem<T>::down(0.f);
-  // most tiles have no pad rows: then nothing is tested per element (the test is a 64-bit compare and a branch each)
-  const bool tile_full = MODE == kDw || m0 + BM <= valid_end;
+  // ---- epilogue, straight from the accumulators. The weight fragment is the MFMA's first operand, so a lane holds, per
+  // 16x16 block (i, j), the 4 consecutive output columns j * 16 + 4 (lane / 16) + 0..3 of tile row i * 16 + lane % 16:
+  // two packed registers. v_permlane16_swap exchanges them between neighbouring 16-lane rows for a pair of column blocks
+  // (j, j + 1): an even lane group ends up with 8 consecutive columns of block j, an odd one with 8 of block j + 1, so
+  // every lane stores 16 bytes and a store instruction writes 64 contiguous bytes of each of 16 output rows. No LDS
+  // round trip and no barrier (a slab in LDS took 16 k of the 196 k cycles of a K = 4096 tile on one wave per SIMD).
+  // Plain (cached) stores: L2 merges the two 64-byte halves of an output line before it leaves for memory (measured
+  // against non-temporal stores: 3 % faster launches at K = 4096).
+  if constexpr (WGM == 2) mfma_drain();
+  if constexpr (CK_STAMP != 0) st_end = clock64();
   if constexpr ((CK_ABLATE & 32) != 0) {
     float keep = 0.f;
-    static_for<MI>([&](auto i) { static_for<NI>([&](auto j) { keep += acc[i][j][0]; }); });
+    static_for<MI>([&](auto i) { static_for<NI>([&](auto j) { keep += acc[i][j][0] + acc[i][j][1] + acc[i][j][2] + acc[i][j][3]; }); });
     if (keep == 123.456f) static_cast<float*>(prm.y)[0] = keep;
     return;
   }
+  auto store_out = [](void* p, const vec16& v) {
+    if constexpr ((CK_ABLATE & 256) != 0) store16_nt(p, v);  // measurement: non-temporal output stores
+    else store16(p, v);
+  };
+  const int lrow = lane & 15, lg = lane >> 4;
+  const bool odd_group = (lg & 1) != 0;
+  const T kZero = Elem<T>::down(0.f);
+  auto pack2 = [](T a, T b) { return (uint32_t)bits16(a) | ((uint32_t)bits16(b) << 16); };
+  // 8 consecutive columns for this lane out of the column blocks j (values p) and j + 1 (values q) of one row block
+  auto gather8 = [&](const T (&p)[4], const T (&q)[4]) {
+    const uint32_t p0 = pack2(p[0], p[1]), p1 = pack2(p[2], p[3]), q0 = pack2(q[0], q[1]), q1 = pack2(q[2], q[3]);
+    const auto s0 = __builtin_amdgcn_permlane16_swap(p0, q0, false, false);  // odd rows of p <-> even rows of q
+    const auto s1 = __builtin_amdgcn_permlane16_swap(p1, q1, false, false);
+    vec16 v;  // even group: own p, then the p of the group above; odd group: the q of the group below, then own q
+    v.w[0] = s0[0];
+    v.w[1] = s1[0];
+    v.w[2] = s0[1];
+    v.w[3] = s1[1];
+    return v;
+  };
+  // column (relative to the wave's first column) of the 8 values gather8 leaves in this lane for the block pair (j, j + 1)
+  auto pair_col = [&](int j) { return (j + (odd_group ? 1 : 0)) * 16 + 4 * (lg & ~1); };
+  const int64_t tile_row0 = m0 + wm * WM;  // first row of this wave's tile rows (padded row / dW row)
 
-  auto stage_blocks = [&](auto&& value /* (i, jj, q, s) -> T */) {
-    static_for<MI>([&](auto i) {
-      static_for<kSlabBlocks>([&](auto jj) {
-        static_for<4>([&](auto q) {
-          const int r = wm * WM + i * 32 + 8 * q + row_quad;
-          const int c = wn * (kSlabBlocks * 32) + jj * 32 + col_in_block;
-          store4(slab + c * kSlabLd + r, value(i, jj, q, std::integral_constant<int, 0>{}),
-                 value(i, jj, q, std::integral_constant<int, 1>{}), value(i, jj, q, std::integral_constant<int, 2>{}),
-                 value(i, jj, q, std::integral_constant<int, 3>{}));
-        });
-      });
-    });
-  };
-  // slab column -> column of the block tile, for pass `pass` (which half of each wave's column blocks is staged)
-  auto tile_col = [&](int sc, int pass) {
-    return (sc / (kSlabBlocks * 32)) * WN + pass * (kSlabBlocks * 32) + sc % (kSlabBlocks * 32);
-  };
-  // Row-major drain. 16 lanes take a 4-row x 32-column block (what one transposing read pair delivers); the four lane
-  // groups of a wave take two adjacent column blocks of two adjacent row blocks, so that a store instruction writes whole
-  // 128-byte lines. The stores are non-temporal: outputs are written once and read by a later launch, and as plain
-  // stores they displace the operand panels that neighbouring tiles re-read from L2 (measured on 256 x 256 tiles with
-  // K = 2048: 7 to 13 % of the launch). Rows and column pairs are walked in unrolled loops: every address is a per-lane base plus a compile-time offset. row_ptr(tile row) -> address of the
-  // output row at the tile's first column (nullptr: pad row), block_col(cb) -> output column of slab column block cb
-  // relative to that, cols_left = valid columns from there on, tile_cols = columns the tile spans.
-  auto drain_rows = [&](auto&& row_ptr, auto&& block_col, int64_t cols_left, int tile_cols) {
-    const int l16 = tid & 15, csel = (tid >> 4) & 1, rsel = (tid >> 5) & 1;
-    const int tq = l16 & 3, tj = l16 >> 2;  // as a source lane: which slab column this lane points at
-    const int oq = l16 >> 2, oe = l16 & 3;  // as a destination lane: 8 columns oq of row oe of the 4 x 32 block
-    constexpr int kColPairs = kSlabCols / 64, kRowIters = (BM / 4) / (2 * NT / kWave);
-    static_assert(kSlabCols % 64 == 0 && (BM / 4) % (2 * NT / kWave) == 0, "whole column pairs and row iterations");
-    const bool cols_full = cols_left >= tile_cols;
-    auto body = [&](auto checked) {
-      static_for<kRowIters>([&](auto it) {
-        const int rb = (it * (NT / kWave) + wave) * 2 + rsel;
-        T* dst_row = row_ptr(rb * 4 + oe);
-        if (dst_row != nullptr) dst_row += 8 * oq;
-        const T* src_row = slab + (csel * 32 + 8 * tq + tj) * kSlabLd + rb * 4;
-        static_for<kColPairs>([&](auto cp) {
-          const T* src = src_row + cp * 64 * kSlabLd;
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(src));
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(src + 4 * kSlabLd));
-          const int col = csel ? block_col(std::integral_constant<int, 2 * decltype(cp)::value + 1>{}) : block_col(std::integral_constant<int, 2 * decltype(cp)::value>{});
-          if (dst_row != nullptr && (!checked || col + 8 * oq < cols_left) && (!(CK_ABLATE & 128) || lo[0] == 12345)) {
-            vec16 v;
-            v.w[0] = (uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
-            v.w[1] = (uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
-            v.w[2] = (uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
-            v.w[3] = (uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16);
-            store16_nt(dst_row + col, v);
-          }
-        });
-      });
-    };
-    if (cols_full) body(std::false_type{});
-    else body(std::true_type{});
-  };
-  auto drain_cols = [&](auto&& out_ptr /* (slab column, tile row) -> address of 8 rows of that column, or nullptr */) {
-    constexpr int kChunks = kSlabCols * (BM / 8);
-#pragma unroll 4
-    for (int ch = tid; ch < kChunks; ch += NT) {
-      const int c = ch / (BM / 8), r = (ch % (BM / 8)) * 8;
-      T* dst = out_ptr(c, r);
-      if (dst != nullptr) store16_nt(dst, load16(slab + c * kSlabLd + r));
-    }
-  };
+  if constexpr (MODE == kScatter) {  // output row of every tile row, through LDS (the stages are dead)
+    int* scatter_rows = reinterpret_cast<int*>(lds_c);
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave is done with the stages
+    if (tid < BM) scatter_rows[tid] = scatter_row;
+    __syncthreads();
+  }
 
+  // Addresses: a uniform 64-bit base (the wave's first output element) plus 32-bit byte offsets per lane, so that a store
+  // costs one 32-bit add at most (rows of one tile are less than 4 GiB apart; scattered rows get their own 64-bit base).
+  auto convert4 = [&](const f32x4& v, T (&o)[4]) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s) o[s] = Elem<T>::down(v[s]);
+  };
   if constexpr (MODE == kDw) {
-    T* dw = static_cast<T*>(prm.y) + (int64_t)expert * prm.M * prm.N;
-    static_for<2>([&](auto pass) {
-      stage_blocks([&](auto i, auto jj, auto q, auto s) {
-        return Elem<T>::down(acc[i][pass * kSlabBlocks + jj][4 * q + s]);
+    const int64_t col0 = (int64_t)nt * BN + wn * WN;
+    char* base = reinterpret_cast<char*>(static_cast<T*>(prm.y) + (int64_t)expert * prm.M * prm.N + tile_row0 * prm.N + col0);
+    const uint32_t row_pitch = (uint32_t)prm.N * 2u;
+    const int rows_left = (int)min((int64_t)WM, (int64_t)prm.M - tile_row0);   // rows of this wave that exist
+    const int cols_left = (int)min((int64_t)WN, (int64_t)prm.N - col0);        // columns of this wave that exist
+    static_for<MI>([&](auto i) {
+      const int r = i * 16 + lrow;
+      const uint32_t row_off = (uint32_t)r * row_pitch;
+      static_for<NI / 2>([&](auto jp) {
+        T p[4], q[4];
+        convert4(acc[i][2 * jp], p);
+        convert4(acc[i][2 * jp + 1], q);
+        const vec16 v = gather8(p, q);
+        const int c = pair_col(2 * jp);
+        if (r < rows_left && c < cols_left && !(CK_ABLATE & 128)) store_out(base + row_off + (uint32_t)c * 2u, v);
       });
-      __syncthreads();
-      drain_rows(
-          [&](int r) -> T* {
-            const int64_t m = m0 + r;
-            return m < prm.M ? dw + m * prm.N + (int64_t)nt * BN : nullptr;
-          },
-          [&](auto cb) { return tile_col(cb * 32, pass); }, prm.N - (int64_t)nt * BN, BN);
-      __syncthreads();
     });
   } else if constexpr (MODE == kGrouped || MODE == kScatter) {
     T* y = static_cast<T*>(prm.y);
     T* y_t = static_cast<T*>(prm.y_t);
+    const int64_t col0 = (int64_t)nt * BN + wn * WN;
+    const int cols_left = (int)min((int64_t)WN, (int64_t)prm.N - col0);
+    const int rows_left = (int)min((int64_t)WM, valid_end - tile_row0);  // valid (non-pad) rows of this wave; may be <= 0
     // optional per-expert bias row (aux_in = bias [E, N]): added to the fp32 accumulators, so that the output is rounded
-    // once, like F.linear with a bias. A lane's accumulators of one column block all belong to one output column.
-    if constexpr (!BT) {
+    // once, like F.linear with a bias
+    if constexpr (!BT && EXTRA) {
       if (prm.aux_in != nullptr) {
         const T* bias = static_cast<const T*>(prm.aux_in) + (int64_t)expert * prm.N;
 #pragma unroll
         for (int j = 0; j < NI; ++j) {
-          const int64_t n = (int64_t)nt * BN + wn * WN + j * 32 + col_in_block;
-          const float b = n < prm.N ? Elem<T>::up(bias[n]) : 0.f;
 #pragma unroll
-          for (int i = 0; i < MI; ++i)
+          for (int s = 0; s < 4; ++s) {
+            const int64_t n = col0 + j * 16 + 4 * lg + s;
+            const float b = n < prm.N ? Elem<T>::up(bias[n]) : 0.f;
 #pragma unroll
-            for (int r = 0; r < 16; ++r) acc[i][j][r] += b;
+            for (int i = 0; i < MI; ++i) acc[i][j][s] += b;
+          }
         }
       }
     }
-    static_for<2>([&](auto pass) {
-      // pad rows are staged as zeros: the transposed copy must hold zeros there
-      if (tile_full) {
-        stage_blocks([&](auto i, auto jj, auto q, auto s) { return Elem<T>::down(acc[i][pass * kSlabBlocks + jj][4 * q + s]); });
+    if constexpr (MODE == kGrouped && EXTRA) if (y_t != nullptr) {
+      // transposed copy [N, ld_t] with zeros in pad rows: a side output for the transposed-operand weight-gradient form
+      // (matrices narrower than 256); 2-byte stores, off the benchmark shapes' path
+      static_for<MI>([&](auto i) {
+        const int r = i * 16 + lrow;
+        const int64_t prow = tile_row0 + r;
+        static_for<NI>([&](auto j) {
+#pragma unroll
+          for (int s = 0; s < 4; ++s) {
+            const int64_t n = col0 + j * 16 + 4 * lg + s;
+            if (n < prm.N) y_t[n * prm.ld_t + prow] = r < rows_left ? Elem<T>::down(acc[i][j][s]) : kZero;
+          }
+        });
+      });
+    }
+    char* base = reinterpret_cast<char*>(y + tile_row0 * prm.N + col0);
+    const uint32_t row_pitch = (uint32_t)prm.N * 2u;
+    static_for<MI>([&](auto i) {
+      const int r = i * 16 + lrow;
+      char* row_ptr;
+      if constexpr (MODE == kScatter) {
+        const int64_t out_row = reinterpret_cast<const int*>(lds_c)[wm * WM + r];
+        row_ptr = reinterpret_cast<char*>(y + out_row * prm.N + col0);
       } else {
-        stage_blocks([&](auto i, auto jj, auto q, auto s) {
-          const int64_t p = m0 + wm * WM + i * 32 + 8 * q + row_quad + s;
-          return p < valid_end ? Elem<T>::down(acc[i][pass * kSlabBlocks + jj][4 * q + s]) : kZero;
-        });
+        row_ptr = base + (uint32_t)r * row_pitch;
       }
-      __syncthreads();
-      drain_rows(
-          [&](int r) -> T* {
-            const int64_t p = m0 + r;
-            if (!tile_full && p >= valid_end) return nullptr;
-            const int64_t row = (MODE == kScatter) ? (int64_t)scatter_rows[r] : p;
-            return y + row * prm.N + (int64_t)nt * BN;
-          },
-          [&](auto cb) { return tile_col(cb * 32, pass); }, prm.N - (int64_t)nt * BN, BN);
-      if (MODE == kGrouped && y_t != nullptr) {
-        drain_cols([&](int sc, int r) -> T* {
-          const int64_t n = (int64_t)nt * BN + tile_col(sc, pass);
-          return n < prm.N ? y_t + n * prm.ld_t + m0 + r : nullptr;
-        });
-      }
-      __syncthreads();
+      static_for<NI / 2>([&](auto jp) {
+        T p[4], q[4];
+        convert4(acc[i][2 * jp], p);
+        convert4(acc[i][2 * jp + 1], q);
+        const vec16 v = gather8(p, q);
+        const int c = pair_col(2 * jp);
+        if (r < rows_left && c < cols_left && !(CK_ABLATE & 128)) store_out(row_ptr + (uint32_t)c * 2u, v);
+      });
     });
-  } else {  // kSwiglu: column blocks 0 .. 2 of a wave are up, 3 .. 5 the gate of the same activation columns
+  } else {  // kSwiglu: the first half of a wave's column blocks are up, the second half the gate of the same activation columns
     T* pre = static_cast<T*>(prm.y);
     T* act = static_cast<T*>(prm.aux);
     T* act_t = static_cast<T*>(prm.y_t);
     const int64_t two_i = 2 * (int64_t)prm.I;
-    auto act_col = [&](int sc) {
-      return (int64_t)nt * (BN / 2) + (sc / (kSlabBlocks * 32)) * (WN / 2) + sc % (kSlabBlocks * 32);
-    };
-    static_for<3>([&](auto pass) {  // 0: up half of the pre-activation, 1: gate half, 2: activation
-      auto value = [&](auto i, auto jj, auto q, auto s, bool valid) {
-        const T up = Elem<T>::down(acc[i][jj][4 * q + s]);
-        const T gate = Elem<T>::down(acc[i][jj + kSlabBlocks][4 * q + s]);
-        if (pass == 0) return up;
-        if (pass == 1) return gate;
-        const float gf = Elem<T>::up(gate);  // from the rounded pre-activation, like the unfused path
-        const float sg = sigmoid_fast(gf);
-        const T a = Elem<T>::down(prm.act_kind == CK_ACT_GLU ? Elem<T>::up(up) * sg : Elem<T>::up(up) * gf * sg);  // same association as swiglu_fwd_kernel
-        return valid ? a : kZero;
-      };
-      if (tile_full) {
-        stage_blocks([&](auto i, auto jj, auto q, auto s) { return value(i, jj, q, s, true); });
-      } else {
-        stage_blocks([&](auto i, auto jj, auto q, auto s) {
-          return value(i, jj, q, s, m0 + wm * WM + i * 32 + 8 * q + row_quad + s < valid_end);
-        });
-      }
-      __syncthreads();
-      const int64_t col0 = (int64_t)nt * (BN / 2);  // the tile's first activation column
-      drain_rows(
-          [&](int r) -> T* {
-            const int64_t p = m0 + r;
-            if (!tile_full && p >= valid_end) return nullptr;
-            if (pass == 0) return pre + p * two_i + col0;
-            if (pass == 1) return pre + p * two_i + prm.I + col0;
-            return act + p * prm.I + col0;
-          },
-          [&](auto cb) { return (int)(act_col(cb * 32) - col0); }, prm.I - col0, BN / 2);
-      if (pass == 2 && act_t != nullptr) {
-        drain_cols([&](int sc, int r) -> T* {
-          const int64_t col = act_col(sc);
-          return col < prm.I ? act_t + col * prm.ld_t + m0 + r : nullptr;
-        });
-      }
-      __syncthreads();
+    const int64_t col0 = (int64_t)nt * (BN / 2) + wn * (WN / 2);  // the wave's first activation column
+    const int cols_left = (int)min((int64_t)(WN / 2), (int64_t)prm.I - col0);
+    const int rows_left = (int)min((int64_t)WM, valid_end - tile_row0);
+    constexpr int NH = NI / 2;  // column blocks per half
+    static_assert(NH % 2 == 0, "whole block pairs in each half");
+    char* pre_base = reinterpret_cast<char*>(pre + tile_row0 * two_i + col0);
+    char* act_base = reinterpret_cast<char*>(act + tile_row0 * prm.I + col0);
+    const uint32_t pre_pitch = (uint32_t)two_i * 2u, act_pitch = (uint32_t)prm.I * 2u, gate_off = (uint32_t)prm.I * 2u;
+    static_for<MI>([&](auto i) {
+      const int r = i * 16 + lrow;
+      const bool valid = r < rows_left;
+      const uint32_t pre_off = (uint32_t)r * pre_pitch, act_off = (uint32_t)r * act_pitch;
+      static_for<NH / 2>([&](auto jp) {
+        T up[2][4], gate[2][4], a[2][4];
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          convert4(acc[i][2 * jp + b], up[b]);
+          convert4(acc[i][2 * jp + b + NH], gate[b]);
+#pragma unroll
+          for (int s = 0; s < 4; ++s) {
+            const float gf = Elem<T>::up(gate[b][s]);  // from the rounded pre-activation, like the unfused path
+            const float sg = sigmoid_fast(gf);
+            a[b][s] = Elem<T>::down(prm.act_kind == CK_ACT_GLU ? Elem<T>::up(up[b][s]) * sg : Elem<T>::up(up[b][s]) * gf * sg);  // same association as swiglu_fwd_kernel
+          }
+        }
+        if constexpr (EXTRA) if (act_t != nullptr) {  // transposed activation [I, ld_t], zeros in pad rows (side output, 2-byte stores)
+#pragma unroll
+          for (int b = 0; b < 2; ++b) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+              const int64_t n = col0 + (2 * jp + b) * 16 + 4 * lg + s;
+              if (n < prm.I) act_t[n * prm.ld_t + tile_row0 + r] = valid ? a[b][s] : kZero;
+            }
+          }
+        }
+        const vec16 vu = gather8(up[0], up[1]), vg = gather8(gate[0], gate[1]), va = gather8(a[0], a[1]);
+        const int c = pair_col(2 * jp);
+        if (valid && c < cols_left && !(CK_ABLATE & 128)) {
+          store_out(pre_base + pre_off + (uint32_t)c * 2u, vu);
+          store_out(pre_base + pre_off + gate_off + (uint32_t)c * 2u, vg);
+          store_out(act_base + act_off + (uint32_t)c * 2u, va);
+        }
+      });
     });
+  }
+  if constexpr (CK_STAMP != 0) {  // per wave: prologue, main loop, of which load wait and barrier wait, epilogue (cycles)
+    if (prm.trace != nullptr && lane == 0) {
+      uint64_t* t = static_cast<uint64_t*>(prm.trace) + ((size_t)blockIdx.x * NW + wave) * 8;
+      t[0] = st_loop - st_begin;
+      t[1] = st_end - st_loop;
+      t[2] = st_vm;
+      t[3] = st_bar;
+      t[4] = clock64() - st_end;
+      t[5] = (uint64_t)nk;
+    }
   }
 }
 
-template <typename T, int MODE, int BN, bool BT>
-int launch_mode(const GemmParams& prm, unsigned blocks, hipStream_t s, const char* name) {
-  auto kernel = grouped_gemm_line_kernel<T, MODE, BN, BT>;
-  constexpr size_t kLds = Tile<BN>::kLdsBytes;
+template <typename T, int MODE, int BN, bool BT, int WGM, bool EXTRA>
+int launch_extra(const GemmParams& prm, unsigned blocks, hipStream_t s, const char* name) {
+  auto kernel = grouped_gemm_line_kernel<T, MODE, BN, BT, WGM, EXTRA>;
+  constexpr size_t kLds = Tile<BN, WGM>::kLdsBytes;
   static bool lds_reserved[kMaxDevices] = {};
   if (int rc = reserve_lds(reinterpret_cast<const void*>(kernel), kLds, lds_reserved, name)) return rc;
-  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(NT), kLds, s, prm);
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(Tile<BN, WGM>::NT), kLds, s, prm);
   CK_CHECK_LAUNCH(name);
   return CK_OK;
 }
 
-template <typename T, int BN>
+template <typename T, int MODE, int BN, bool BT, int WGM>
+int launch_mode(const GemmParams& prm, unsigned blocks, hipStream_t s, const char* name) {
+  if constexpr (!BT && MODE != kDw) {
+    if (prm.aux_in != nullptr || prm.y_t != nullptr) return launch_extra<T, MODE, BN, BT, WGM, true>(prm, blocks, s, name);
+  }
+  return launch_extra<T, MODE, BN, BT, WGM, false>(prm, blocks, s, name);
+}
+
+template <typename T, int BN, int WGM>
 int launch_bn(const GemmParams& prm, int mode, bool bt, unsigned blocks, hipStream_t stream, const char* name) {
-  if (bt) {  // the input-gradient GEMMs: grouped or scatter epilogue, 256-wide tiles (the 384-wide tile has no registers
-             // left for the transposing reads' addresses)
+  if (bt) {  // the input-gradient GEMMs: grouped or scatter epilogue, 256-wide tiles
     if constexpr (BN == 256) {
-      if (mode == kGrouped) return launch_mode<T, kGrouped, BN, true>(prm, blocks, stream, name);
-      if (mode == kScatter) return launch_mode<T, kScatter, BN, true>(prm, blocks, stream, name);
-      if (mode == kDw) return launch_mode<T, kDw, BN, true>(prm, blocks, stream, name);  // both operands row-major
+      if (mode == kGrouped) return launch_mode<T, kGrouped, BN, true, WGM>(prm, blocks, stream, name);
+      if (mode == kScatter) return launch_mode<T, kScatter, BN, true, WGM>(prm, blocks, stream, name);
+      if (mode == kDw) return launch_mode<T, kDw, BN, true, WGM>(prm, blocks, stream, name);  // both operands row-major
     }
     set_error("%s: contraction-strided operands go with 256-wide tiles and the grouped / scatter / dW epilogues", name);
     return CK_ERR_ARG;
   }
   switch (mode) {
-    case kGrouped: return launch_mode<T, kGrouped, BN, false>(prm, blocks, stream, name);
-    case kScatter: return launch_mode<T, kScatter, BN, false>(prm, blocks, stream, name);
-    case kSwiglu: return launch_mode<T, kSwiglu, BN, false>(prm, blocks, stream, name);
-    case kDw: return launch_mode<T, kDw, BN, false>(prm, blocks, stream, name);
+    case kGrouped: return launch_mode<T, kGrouped, BN, false, WGM>(prm, blocks, stream, name);
+    case kScatter: return launch_mode<T, kScatter, BN, false, WGM>(prm, blocks, stream, name);
+    case kSwiglu: return launch_mode<T, kSwiglu, BN, false, WGM>(prm, blocks, stream, name);
+    case kDw: return launch_mode<T, kDw, BN, false, WGM>(prm, blocks, stream, name);
     default: break;
   }
   set_error("%s: the 128-byte-row kernel has no epilogue %d", name, mode);
@@ -631,12 +667,12 @@ int launch_bn(const GemmParams& prm, int mode, bool bt, unsigned blocks, hipStre
 
 }  // namespace
 
-int launch_line(const GemmParams& prm, int mode, int bn, bool bt, int dtype, unsigned blocks, hipStream_t stream,
+int launch_line(const GemmParams& prm_in, int mode, int bn, bool bt, int dtype, unsigned blocks, hipStream_t stream,
                 const char* name) {
-  CK_DISPATCH_HALF(dtype, name, {
-    if (bn == 384) return launch_bn<scalar_t, 384>(prm, mode, bt, blocks, stream, name);
-    return launch_bn<scalar_t, 256>(prm, mode, bt, blocks, stream, name);
-  });
+  GemmParams prm = prm_in;
+  if (const char* env = getenv("CK_STAGGER_XCD")) prm.stagger_xcd = atoi(env);
+  if (const char* env = getenv("CK_STAGGER_CU")) prm.stagger_cu = atoi(env);
+  CK_DISPATCH_HALF(dtype, name, { return launch_bn<scalar_t, 256, 2>(prm, mode, bt, blocks, stream, name); });
   return CK_ERR_ARG;
 }
 

@@ -37,12 +37,12 @@ def _expected_grouped(a_rows_fn, w, seg, N):
     return out
 
 
-@pytest.fixture(params=["default", "384"])
+@pytest.fixture(params=["default", "general"])
 def gemm_tile(request, monkeypatch):
-    """Which block tile the 16-bit GEMMs use: the library's own choice, or the 256 x 384 variant wherever it applies
-    (align 256 and K % 32 == 0; the library reads CK_GEMM_TILE on every call)."""
+    """Which kernel the 16-bit GEMMs run on: the library's own choice (the 128-byte-row kernel wherever it applies: align
+    256 and K % 64 == 0), or the general kernel for every case (the library reads CK_GEMM_LINE on every call)."""
     if request.param != "default":
-        monkeypatch.setenv("CK_GEMM_TILE", request.param)
+        monkeypatch.setenv("CK_GEMM_LINE", "0")
     return request.param
 
 
