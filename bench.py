@@ -356,7 +356,8 @@ def gemm_only(dev, launches: int, stamps: bool = False):
             "waves": int(len(t)), "k_steps": float(t[:, 5].mean()),
             "cycles_per_wave": {"prologue": float(t[:, 0].mean()), "main_loop": float(t[:, 1].mean()),
                                 "load_wait": float(t[:, 2].mean()), "barrier_wait": float(t[:, 3].mean()),
-                                "epilogue": float(t[:, 4].mean())},
+                                "epilogue": float(t[:, 4].mean()), "slice0_per_step": float((t[:, 6] / (t[:, 5] - 1)).mean()),
+                                "slice1_per_step": float((t[:, 7] / (t[:, 5] - 1)).mean())},
             "share_of_tile": {"main_loop": float((t[:, 1] / tot).mean()), "load_wait": float((t[:, 2] / tot).mean()),
                               "barrier_wait": float((t[:, 3] / tot).mean()), "epilogue": float((t[:, 4] / tot).mean())},
             "main_loop_cycles_per_k_step": float((t[:, 1] / t[:, 5]).mean()),

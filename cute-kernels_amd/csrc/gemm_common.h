@@ -39,8 +39,6 @@ struct GemmParams {
   const float* w_scale;  // fp8 only: per-output-channel scale of w, [E, N]
   int act_kind;          // kSwiglu epilogue: CK_ACT_SWIGLU (up * gate * sigmoid(gate)) or CK_ACT_GLU (up * sigmoid(gate))
   void* trace;           // measurement builds only: per-workgroup phase timestamps (8 x uint64 each), else NULL
-  int stagger_xcd;       // experiment: start delay of the first workgroup on each CU, in 10 ns units per XCD index ...
-  int stagger_cu;        // ... and per CU index within the XCD
 };
 
 // The 16-bit kernel with 128-byte LDS rows (grouped_gemm_line.hip): 256 x bn tiles, bn = 256 or 384, contraction length a
@@ -137,6 +135,33 @@ __device__ inline uint16_t bits16(T v) {
     uint16_t u;
   } c;
   c.t = v;
+  return c.u;
+}
+
+// two fp32 values rounded (to nearest even) and packed into one register: one v_cvt_pk instruction
+typedef __attribute__((__vector_size__(2 * sizeof(float)))) float f32x2_t;
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+typedef __attribute__((__vector_size__(2 * sizeof(_Float16)))) _Float16 f16x2_t;
+template <typename T>
+__device__ inline uint32_t pack_pair(float a, float b);
+template <>
+__device__ inline uint32_t pack_pair<bf16_t>(float a, float b) {
+  const f32x2_t v = {a, b};
+  union {
+    bf16x2_t h;
+    uint32_t u;
+  } c;
+  c.h = __builtin_convertvector(v, bf16x2_t);
+  return c.u;
+}
+template <>
+__device__ inline uint32_t pack_pair<f16_t>(float a, float b) {
+  const f32x2_t v = {a, b};
+  union {
+    f16x2_t h;
+    uint32_t u;
+  } c;
+  c.h = __builtin_convertvector(v, f16x2_t);
   return c.u;
 }
 

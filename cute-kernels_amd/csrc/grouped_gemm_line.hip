@@ -28,9 +28,6 @@
 #ifndef CK_LOAD_GAP
 #define CK_LOAD_GAP 0  // measurement builds only: MFMAs between two loads of the next-but-one K step (0: spread over the whole last slice)
 #endif
-#ifndef CK_READ_GAP
-#define CK_READ_GAP 0  // measurement builds only: MFMAs between two fragment reads of the two-set schedule (default 1: the reads go out behind the first MI + NI MFMAs)
-#endif
 #ifndef CK_STAMP
 #define CK_STAMP 0  // measurement builds only: 1 = every wave adds up the cycles it spends waiting for the loads and at the barrier of each K step and writes them, with its main-loop and epilogue cycles, to GemmParams::trace
 #endif
@@ -81,12 +78,7 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   const int tid = threadIdx.x, lane = tid & (kWave - 1);
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);  // uniform: everything derived from it stays in scalar registers
   const int wm = wave >> 1, wn = wave & 1;
-  if ((prm.stagger_xcd | prm.stagger_cu) != 0 && blockIdx.x < 256) {  // experiment: phase-shift the CUs' tile loops
-    const uint64_t t0 = wall_clock64();
-    const uint64_t wait = (uint64_t)(blockIdx.x % kXcds) * prm.stagger_xcd + (uint64_t)(blockIdx.x / kXcds) * prm.stagger_cu;
-    while (wall_clock64() - t0 < wait) __builtin_amdgcn_s_sleep(8);
-  }
-  [[maybe_unused]] uint64_t st_begin = 0, st_loop = 0, st_end = 0, st_vm = 0, st_bar = 0;
+  [[maybe_unused]] uint64_t st_begin = 0, st_loop = 0, st_end = 0, st_vm = 0, st_bar = 0, st_s0 = 0, st_s1 = 0, st_mark = 0;
   if constexpr (CK_STAMP != 0) st_begin = clock64();
 
   // ---- which tile (same XCD-aware orders as the 256 x 256 kernel)
@@ -354,6 +346,13 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
     for (int i = 0; i < MI; ++i) read_a(0, 0, 0, i);
 #pragma unroll
     for (int j = 0; j < NI; ++j) read_b(0, 0, 0, j);
+    if constexpr ((CK_ABLATE & 4) != 0 && kDouble) {  // no fragment reads in the loop: both sets hold the first slice
+#pragma unroll
+      for (int i = 0; i < MI; ++i) fa[1][i] = fa[0][i];
+#pragma unroll
+      for (int j = 0; j < NI; ++j) fb[1][j] = fb[0][j];
+    }
+    if constexpr (CK_STAMP != 0) st_mark = clock64();
 
     // One 32-wide slice: MI x NI MFMAs, row block by row block, and the fragment reads for the slice after it (ns, nsl).
     // Two fragment sets: the reads go out one after each of the first MI + NI MFMAs, in the order the next slice needs
@@ -388,6 +387,8 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
           const uint64_t t2 = clock64();
           st_vm += t1 - t0;
           st_bar += t2 - t1;
+          st_s0 += t0 - st_mark;  // slice 0 of this step (the slice in front of the wait)
+          st_mark = t2;
         } else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       }
       constexpr int cur = kDouble ? (decltype(sl)::value & 1) : 0;
@@ -401,13 +402,10 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
         }
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (kReload) {
-          if constexpr (kDouble) {  // one read every kReadGap MFMAs, in the order the next slice needs them
-            constexpr int kReadGap = CK_READ_GAP > 0 ? CK_READ_GAP : 1;
-            if (n % kReadGap == 0 && n / kReadGap < MI + NI) {
-              const int r = n / kReadGap;
-              if (r < MI) read_a(nxt, ns, nsl, r);
-              else read_b(nxt, ns, nsl, r - MI);
-            }
+          if constexpr (kDouble) {  // behind the first MI + NI MFMAs, in the order the next slice needs them (spreading
+                                    // them over the whole slice measured the same)
+            if (n < MI) read_a(nxt, ns, nsl, n);
+            else if (n < MI + NI) read_b(nxt, ns, nsl, n - MI);
           } else {
             if (j == NI - 1) read_a(0, ns, nsl, i);
             if (i == MI - 1) read_b(0, ns, nsl, j);
@@ -415,6 +413,11 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
         }
       }
       __builtin_amdgcn_sched_barrier(0);
+      if constexpr (CK_STAMP != 0 && kLast && kPhase < 2) {
+        const uint64_t t3 = clock64();
+        st_s1 += t3 - st_mark;  // slice 1: from the barrier to the end of the step
+        st_mark = t3;
+      }
     };
     auto k_loop = [&](auto idle) {
       auto k_step = [&](int kt, auto phase) { static_for<KS>([&](auto sl) { slice(kt, sl, phase, idle); }); };
@@ -437,7 +440,8 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   // two packed registers. v_permlane16_swap exchanges them between neighbouring 16-lane rows for a pair of column blocks
   // (j, j + 1): an even lane group ends up with 8 consecutive columns of block j, an odd one with 8 of block j + 1, so
   // every lane stores 16 bytes and a store instruction writes 64 contiguous bytes of each of 16 output rows. No LDS
-  // round trip and no barrier (a slab in LDS took 16 k of the 196 k cycles of a K = 4096 tile on one wave per SIMD).
+  // round trip and no barrier (a slab in LDS took 16 k of the 196 k cycles of a K = 4096 tile on one wave per SIMD; this
+  // form 9 k, of which 5 k are the register reads, conversions and swaps and 4 k the stores).
   // Plain (cached) stores: L2 merges the two 64-byte halves of an output line before it leaves for memory (measured
   // against non-temporal stores: 3 % faster launches at K = 4096).
   if constexpr (WGM == 2) mfma_drain();
@@ -455,10 +459,8 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   const int lrow = lane & 15, lg = lane >> 4;
   const bool odd_group = (lg & 1) != 0;
   const T kZero = Elem<T>::down(0.f);
-  auto pack2 = [](T a, T b) { return (uint32_t)bits16(a) | ((uint32_t)bits16(b) << 16); };
-  // 8 consecutive columns for this lane out of the column blocks j (values p) and j + 1 (values q) of one row block
-  auto gather8 = [&](const T (&p)[4], const T (&q)[4]) {
-    const uint32_t p0 = pack2(p[0], p[1]), p1 = pack2(p[2], p[3]), q0 = pack2(q[0], q[1]), q1 = pack2(q[2], q[3]);
+  // 8 consecutive columns for this lane out of the column blocks j (packed pairs p0, p1) and j + 1 (q0, q1) of one row block
+  auto gather8 = [&](uint32_t p0, uint32_t p1, uint32_t q0, uint32_t q1) {
     const auto s0 = __builtin_amdgcn_permlane16_swap(p0, q0, false, false);  // odd rows of p <-> even rows of q
     const auto s1 = __builtin_amdgcn_permlane16_swap(p1, q1, false, false);
     vec16 v;  // even group: own p, then the p of the group above; odd group: the q of the group below, then own q
@@ -468,8 +470,20 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
     v.w[3] = s1[1];
     return v;
   };
+  auto gather8_acc = [&](const f32x4& p, const f32x4& q) {
+    return gather8(pack_pair<T>(p[0], p[1]), pack_pair<T>(p[2], p[3]), pack_pair<T>(q[0], q[1]), pack_pair<T>(q[2], q[3]));
+  };
   // column (relative to the wave's first column) of the 8 values gather8 leaves in this lane for the block pair (j, j + 1)
   auto pair_col = [&](int j) { return (j + (odd_group ? 1 : 0)) * 16 + 4 * (lg & ~1); };
+  // store_lines(v1, v2, j, ptr_of_row, row_ok, col_ok): the block quad j .. j + 3 of one row block, two 16-byte pieces per
+  // lane (v1: blocks j, j + 1; v2: blocks j + 2, j + 3); ptr_of_row(r) -> address of the wave's first column in row r
+  // (0 .. 15) of the row block; row_ok(r), col_ok(c) -> inside the matrix. (Regrouping the pieces so that every store
+  // writes whole 128-byte lines -- a rotation by 8 inside the 16-lane rows -- measured the same and is not done.)
+  auto store_lines = [&](const vec16& v1, const vec16& v2, int j, auto&& ptr_of_row, auto&& row_ok, auto&& col_ok) {
+    const int c1 = pair_col(j), c2 = pair_col(j + 2);
+    if (row_ok(lrow) && col_ok(c1) && (!(CK_ABLATE & 128) || prm.K == -12345)) store_out(ptr_of_row(lrow) + (uint32_t)c1 * 2u, v1);
+    if (row_ok(lrow) && col_ok(c2) && (!(CK_ABLATE & 128) || prm.K == -12345)) store_out(ptr_of_row(lrow) + (uint32_t)c2 * 2u, v2);
+  };
   const int64_t tile_row0 = m0 + wm * WM;  // first row of this wave's tile rows (padded row / dW row)
 
   if constexpr (MODE == kScatter) {  // output row of every tile row, through LDS (the stages are dead)
@@ -492,16 +506,12 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
     const int rows_left = (int)min((int64_t)WM, (int64_t)prm.M - tile_row0);   // rows of this wave that exist
     const int cols_left = (int)min((int64_t)WN, (int64_t)prm.N - col0);        // columns of this wave that exist
     static_for<MI>([&](auto i) {
-      const int r = i * 16 + lrow;
-      const uint32_t row_off = (uint32_t)r * row_pitch;
-      static_for<NI / 2>([&](auto jp) {
-        T p[4], q[4];
-        convert4(acc[i][2 * jp], p);
-        convert4(acc[i][2 * jp + 1], q);
-        const vec16 v = gather8(p, q);
-        const int c = pair_col(2 * jp);
-        if (r < rows_left && c < cols_left && !(CK_ABLATE & 128)) store_out(base + row_off + (uint32_t)c * 2u, v);
+      static_for<NI / 4>([&](auto jq) {
+        const vec16 v1 = gather8_acc(acc[i][4 * jq], acc[i][4 * jq + 1]), v2 = gather8_acc(acc[i][4 * jq + 2], acc[i][4 * jq + 3]);
+        store_lines(v1, v2, 4 * jq, [&](int r) { return base + (uint32_t)(i * 16 + r) * row_pitch; },
+                    [&](int r) { return i * 16 + r < rows_left; }, [&](int c) { return c < cols_left; });
       });
+      __builtin_amdgcn_sched_barrier(0);  // row block by row block: the stores of one drain under the conversions of the next
     });
   } else if constexpr (MODE == kGrouped || MODE == kScatter) {
     T* y = static_cast<T*>(prm.y);
@@ -544,22 +554,21 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
     char* base = reinterpret_cast<char*>(y + tile_row0 * prm.N + col0);
     const uint32_t row_pitch = (uint32_t)prm.N * 2u;
     static_for<MI>([&](auto i) {
-      const int r = i * 16 + lrow;
-      char* row_ptr;
+      char* row_a = nullptr;  // scatter: the output row this lane writes in this row block
       if constexpr (MODE == kScatter) {
-        const int64_t out_row = reinterpret_cast<const int*>(lds_c)[wm * WM + r];
-        row_ptr = reinterpret_cast<char*>(y + out_row * prm.N + col0);
-      } else {
-        row_ptr = base + (uint32_t)r * row_pitch;
+        const int* rows = reinterpret_cast<const int*>(lds_c) + wm * WM + i * 16;
+        row_a = reinterpret_cast<char*>(y + (int64_t)rows[lrow] * prm.N + col0);
       }
-      static_for<NI / 2>([&](auto jp) {
-        T p[4], q[4];
-        convert4(acc[i][2 * jp], p);
-        convert4(acc[i][2 * jp + 1], q);
-        const vec16 v = gather8(p, q);
-        const int c = pair_col(2 * jp);
-        if (r < rows_left && c < cols_left && !(CK_ABLATE & 128)) store_out(row_ptr + (uint32_t)c * 2u, v);
+      static_for<NI / 4>([&](auto jq) {
+        const vec16 v1 = gather8_acc(acc[i][4 * jq], acc[i][4 * jq + 1]), v2 = gather8_acc(acc[i][4 * jq + 2], acc[i][4 * jq + 3]);
+        store_lines(v1, v2, 4 * jq,
+                    [&](int r) {
+                      if constexpr (MODE == kScatter) return row_a;
+                      else return base + (uint32_t)(i * 16 + r) * row_pitch;
+                    },
+                    [&](int r) { return i * 16 + r < rows_left; }, [&](int c) { return c < cols_left; });
       });
+      __builtin_amdgcn_sched_barrier(0);
     });
   } else {  // kSwiglu: the first half of a wave's column blocks are up, the second half the gate of the same activation columns
     T* pre = static_cast<T*>(prm.y);
@@ -577,7 +586,8 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
     static_for<MI>([&](auto i) {
       const int r = i * 16 + lrow;
       const bool valid = r < rows_left;
-      const uint32_t pre_off = (uint32_t)r * pre_pitch, act_off = (uint32_t)r * act_pitch;
+      static_assert(NH == 4, "one quad of column blocks per half");
+      vec16 vu_[2], vg_[2], va_[2];
       static_for<NH / 2>([&](auto jp) {
         T up[2][4], gate[2][4], a[2][4];
 #pragma unroll
@@ -601,14 +611,20 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
             }
           }
         }
-        const vec16 vu = gather8(up[0], up[1]), vg = gather8(gate[0], gate[1]), va = gather8(a[0], a[1]);
-        const int c = pair_col(2 * jp);
-        if (valid && c < cols_left && !(CK_ABLATE & 128)) {
-          store_out(pre_base + pre_off + (uint32_t)c * 2u, vu);
-          store_out(pre_base + pre_off + gate_off + (uint32_t)c * 2u, vg);
-          store_out(act_base + act_off + (uint32_t)c * 2u, va);
-        }
+        auto pk = [&](const T (&v)[4], int h) { return (uint32_t)bits16(v[2 * h]) | ((uint32_t)bits16(v[2 * h + 1]) << 16); };
+        const vec16 vu = gather8(pk(up[0], 0), pk(up[0], 1), pk(up[1], 0), pk(up[1], 1));
+        const vec16 vg = gather8(pk(gate[0], 0), pk(gate[0], 1), pk(gate[1], 0), pk(gate[1], 1));
+        const vec16 va = gather8(pk(a[0], 0), pk(a[0], 1), pk(a[1], 0), pk(a[1], 1));
+        vu_[jp] = vu;
+        vg_[jp] = vg;
+        va_[jp] = va;
       });
+      auto rows_ok = [&](int r) { return i * 16 + r < rows_left; };
+      auto cols_ok = [&](int c) { return c < cols_left; };
+      store_lines(vu_[0], vu_[1], 0, [&](int r) { return pre_base + (uint32_t)(i * 16 + r) * pre_pitch; }, rows_ok, cols_ok);
+      store_lines(vg_[0], vg_[1], 0, [&](int r) { return pre_base + (uint32_t)(i * 16 + r) * pre_pitch + gate_off; }, rows_ok, cols_ok);
+      store_lines(va_[0], va_[1], 0, [&](int r) { return act_base + (uint32_t)(i * 16 + r) * act_pitch; }, rows_ok, cols_ok);
+      __builtin_amdgcn_sched_barrier(0);
     });
   }
   if constexpr (CK_STAMP != 0) {  // per wave: prologue, main loop, of which load wait and barrier wait, epilogue (cycles)
@@ -620,6 +636,8 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
       t[3] = st_bar;
       t[4] = clock64() - st_end;
       t[5] = (uint64_t)nk;
+      t[6] = st_s0;
+      t[7] = st_s1;
     }
   }
 }
@@ -669,9 +687,7 @@ int launch_bn(const GemmParams& prm, int mode, bool bt, unsigned blocks, hipStre
 
 int launch_line(const GemmParams& prm_in, int mode, int bn, bool bt, int dtype, unsigned blocks, hipStream_t stream,
                 const char* name) {
-  GemmParams prm = prm_in;
-  if (const char* env = getenv("CK_STAGGER_XCD")) prm.stagger_xcd = atoi(env);
-  if (const char* env = getenv("CK_STAGGER_CU")) prm.stagger_cu = atoi(env);
+  const GemmParams& prm = prm_in;
   CK_DISPATCH_HALF(dtype, name, { return launch_bn<scalar_t, 256, 2>(prm, mode, bt, blocks, stream, name); });
   return CK_ERR_ARG;
 }
