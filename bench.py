@@ -484,6 +484,7 @@ def main() -> int:
         "unit": "TFLOP/s",
         "frac": achieved / PEAK_BF16_TFLOPS,
         "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(dominant),
+        "traffic_source": "static: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, see profiles/ (not measured in this run)",
         "avg_launch_ms": d["ms"] / d["launches"],
         "flops_per_launch": d["flops"] / d["launches"],
     }

@@ -447,6 +447,22 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
   // static_for keeps every accumulator index a compile-time constant (the accumulators live in AGPRs).
   const int col_in_block = lane & 31;
   const int row_quad = (lane >> 5) * 4;
+  // optional per-expert bias row (aux_in = bias [E, N], grouped / scatter epilogues): added to the fp32 accumulators, so
+  // that the output is rounded once, like F.linear with a bias. A lane's accumulators of one column block all belong to
+  // one output column.
+  if constexpr (MODE == kGrouped || MODE == kScatter) {
+    if (prm.aux_in != nullptr) {
+      const T* bias = static_cast<const T*>(prm.aux_in) + (int64_t)expert * prm.N;
+      static_for<NI>([&](auto j) {
+        const int64_t n = (int64_t)nt * BN + wn * WN + j * 32 + col_in_block;
+        const float b = n < prm.N ? Elem<T>::up(bias[n]) : 0.f;
+        static_for<MI>([&](auto i) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[i][j][r] += b;
+        });
+      });
+    }
+  }
   if constexpr ((CK_ABLATE & 32) != 0) {  // measurement builds: no epilogue (keep the accumulators alive)
     float keep = 0.f;
 #pragma unroll
@@ -818,9 +834,8 @@ extern "C" int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* 
   hipStream_t s = static_cast<hipStream_t>(stream);
   // kSwiglu tiles cover BN/2 activation columns each
   auto n_tiles_for = [&](int bn) { return (int)ceil_div(out_cols, epilogue == CK_EPI_SWIGLU ? bn / 2 : bn); };
-  CK_REQUIRE(aux_in == nullptr || epilogue == CK_EPI_SWIGLU_BWD || (line_kernel && epilogue != CK_EPI_SWIGLU),
-             "%s: the bias operand (aux_in) goes with the grouped / scatter epilogues of the 256-row-tile kernel "
-             "(align = 256, K %% 64 == 0)", name);
+  CK_REQUIRE(aux_in == nullptr || epilogue != CK_EPI_SWIGLU,
+             "%s: the bias operand (aux_in) goes with the grouped / scatter epilogues", name);
   if (line_kernel) {
     const bool swiglu = epilogue == CK_EPI_SWIGLU;
     const int bn = 256;

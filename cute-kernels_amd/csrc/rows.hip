@@ -68,10 +68,10 @@ __global__ __launch_bounds__(kBlock) void combine_rows_kernel(const T* __restric
 }
 
 // d_gates[t, j] = <expanded[t, j, :], grad_out[t, :]>, one wave per (t, j)
-template <typename T>
+template <typename T, typename OUT>
 __global__ __launch_bounds__(kBlock) void gate_grad_kernel(const T* __restrict__ expanded, const T* __restrict__ grad_out,
                                                             int64_t pairs, int k, int chunks_per_row,
-                                                            T* __restrict__ d_gates) {
+                                                            OUT* __restrict__ d_gates) {
   constexpr int P = Elem<T>::per16;
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t pair = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
@@ -86,7 +86,7 @@ __global__ __launch_bounds__(kBlock) void gate_grad_kernel(const T* __restrict__
     for (int i = 0; i < P; ++i) acc += Elem<T>::up(a.e[i]) * Elem<T>::up(b.e[i]);
   }
   acc = wave_sum(acc);
-  if (lane == 0) d_gates[pair] = Elem<T>::down(acc);
+  if (lane == 0) d_gates[pair] = Elem<OUT>::down(acc);
 }
 
 // ---- 64x64 tiles of 16-bit elements through LDS ---------------------------------------------------------------
@@ -419,12 +419,31 @@ extern "C" int ck_combine_rows(const void* expanded, const void* gates, int64_t 
     }
     if (d_gates_out != nullptr) {
       const int64_t pairs = T * k;
-      hipLaunchKernelGGL((gate_grad_kernel<scalar_t>), dim3((unsigned)ceil_div(pairs, kBlock / kWave)), dim3(kBlock),
+      hipLaunchKernelGGL((gate_grad_kernel<scalar_t, scalar_t>), dim3((unsigned)ceil_div(pairs, kBlock / kWave)), dim3(kBlock),
                          0, s, static_cast<const scalar_t*>(expanded), static_cast<const scalar_t*>(grad_out), pairs,
                          (int)k, cpr, static_cast<scalar_t*>(d_gates_out));
     }
   });
   CK_CHECK_LAUNCH("ck_combine_rows");
+  return CK_OK;
+}
+
+extern "C" int ck_gate_grad_f32(const void* expanded, const void* grad_out, int64_t T, int32_t k, int32_t H,
+                                float* d_gates, int32_t dtype, void* stream) {
+  CK_REQUIRE(T >= 0 && k >= 1 && H >= 1, "ck_gate_grad_f32: bad sizes T=%lld k=%d H=%d", (long long)T, k, H);
+  if (T == 0) return CK_OK;
+  CK_REQUIRE(expanded && grad_out && d_gates, "ck_gate_grad_f32: NULL argument");
+  CK_REQUIRE(aligned16(expanded) && aligned16(grad_out), "ck_gate_grad_f32: expanded / grad_out must be 16-byte aligned");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  CK_DISPATCH_FLOAT(dtype, "ck_gate_grad_f32", {
+    constexpr int P = Elem<scalar_t>::per16;
+    CK_REQUIRE(H % P == 0, "ck_gate_grad_f32: H=%d is not a multiple of %d", H, P);
+    const int64_t pairs = T * k;
+    hipLaunchKernelGGL((gate_grad_kernel<scalar_t, float>), dim3((unsigned)ceil_div(pairs, kBlock / kWave)), dim3(kBlock), 0,
+                       s, static_cast<const scalar_t*>(expanded), static_cast<const scalar_t*>(grad_out), pairs, (int)k,
+                       H / P, d_gates);
+  });
+  CK_CHECK_LAUNCH("ck_gate_grad_f32");
   return CK_OK;
 }
 

@@ -55,6 +55,7 @@ _SIGNATURES = {
     "ck_sort_by_expert": (c_int32, [c_void_p, c_int32, c_int64, c_int32, c_int32] + [c_void_p] * 10),
     "ck_gather_rows": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_int32, c_void_p]),
     "ck_combine_rows": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int32, c_void_p]),
+    "ck_gate_grad_f32": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_int32, c_void_p, c_int32, c_void_p]),
     "ck_group_rows_padded": (
         c_int32,
         [c_void_p, c_void_p, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_void_p, c_void_p, c_int64, c_int32, c_void_p],

@@ -34,6 +34,7 @@ class _Ctx:
     def __init__(self, needs_input_grad=()) -> None:
         self.needs_input_grad = tuple(needs_input_grad)
         self.saved_tensors = ()
+        self.gate_slot = self.slot = None  # traced graphs pass d_gates in the gates' dtype (no fp32 side channel)
 
     def save_for_backward(self, *tensors) -> None:
         self.saved_tensors = tensors
@@ -414,7 +415,7 @@ def swiglu_experts_backward(
     ctx.saved_tensors = (
         x.contiguous(), w_fc.contiguous(), w_proj.contiguous(), gates.contiguous(), pre, act_t if need_proj else None, expanded,
     )
-    d_x, d_w_fc, d_w_proj, d_gates, _, _ = _moe._SwigluExperts.backward(ctx, grad_out)
+    d_x, d_w_fc, d_w_proj, d_gates = _moe._SwigluExperts.backward(ctx, grad_out)[:4]
     return _or_empty(d_x, x), _or_empty(d_w_fc, x), _or_empty(d_w_proj, x), _or_empty(d_gates, x)
 
 
@@ -525,7 +526,7 @@ def experts_down_backward(
     ctx = _Ctx((need_h, need_w, need_gates, False, need_bias))
     ctx.seg = _segments(seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, align)
     ctx.saved_tensors = (h.contiguous(), w.contiguous(), gates.contiguous(), expanded)
-    d_h, d_w, d_gates, _, d_bias, _ = _moe._ExpertsDown.backward(ctx, grad_out)
+    d_h, d_w, d_gates, _, d_bias = _moe._ExpertsDown.backward(ctx, grad_out)[:5]
     return _or_empty(d_h, h), _or_empty(d_w, h), _or_empty(d_gates, h), _or_empty(d_bias, h)
 
 

@@ -48,6 +48,8 @@ def quantize_expert_weights_e4m3(weight: torch.Tensor) -> tuple[torch.Tensor, to
 def _gemm_fp8(a8, a_scale, gather_div, w8, w_scale, seg: ExpertSegments, epilogue, y, aux, out_dtype):
     E, N, K = w8.shape
     cs = seg.c_struct()
+    if gather_div > 0:  # gathered rows are addressed with 32-bit byte offsets from the start of the token-order tensor
+        assert a8.numel() < 2**32, "the token-order fp8 input of a grouped GEMM must stay below 4 GiB"
 
     def launch():
         with torch.cuda.device(w8.device):

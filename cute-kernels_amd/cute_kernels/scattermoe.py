@@ -23,11 +23,27 @@ _ops = None  # cute_kernels.compile_ops, set by the package once it is imported 
 # ---------------------------------------------------------------------------------------------------------------
 # routing
 # ---------------------------------------------------------------------------------------------------------------
+class _GateGradSlot:
+    """Side channel between the expert block's backward and the router's backward. Autograd hands a 16-bit gates tensor
+    a 16-bit gradient; the softmax backward then subtracts nearly equal rounded numbers and gate.weight.grad loses
+    digits. The expert block leaves its unrounded fp32 d_gates here, and the router's backward uses it when the gradient
+    it receives is exactly that tensor rounded (i.e. nothing else contributed to the gates' gradient)."""
+
+    __slots__ = ("d_gates_f32",)
+
+    def __init__(self):
+        self.d_gates_f32 = None
+
+
+def _gate_slot(gates: torch.Tensor):
+    return getattr(gates, "_ck_gate_slot", None)
+
+
 class _RouteTopKSoftmax(torch.autograd.Function):
     """logits [T, E] -> gates [T, k] (softmax over the k largest logits, in logits.dtype), selected [T, k] int64."""
 
     @staticmethod
-    def forward(ctx, logits: torch.Tensor, k: int, long_indices: bool = True):
+    def forward(ctx, logits: torch.Tensor, k: int, long_indices: bool = True, slot: _GateGradSlot | None = None):
         _C.require_gpu(logits)
         logits = logits.contiguous()
         T, E = logits.shape
@@ -43,6 +59,7 @@ class _RouteTopKSoftmax(torch.autograd.Function):
         ctx.save_for_backward(gates, selected)
         ctx.E = E
         ctx.dtype = logits.dtype
+        ctx.slot = slot
         selected_out = selected.long() if long_indices else selected
         ctx.mark_non_differentiable(selected_out)
         return gates.to(logits.dtype), selected_out
@@ -51,6 +68,12 @@ class _RouteTopKSoftmax(torch.autograd.Function):
     def backward(ctx, d_gates: torch.Tensor, _d_selected):
         gates, selected = ctx.saved_tensors
         T, k = gates.shape
+        exact = ctx.slot.d_gates_f32 if ctx.slot is not None else None
+        if exact is not None and exact.shape == d_gates.shape and d_gates.dtype != torch.float32:
+            # the unrounded gradient, if what arrived is that tensor rounded (decided on the device: no host sync)
+            same = (exact.to(d_gates.dtype) == d_gates).all()
+            d_gates = torch.where(same, exact, d_gates.float())
+            ctx.slot.d_gates_f32 = None
         d_gates = d_gates.float().contiguous()
         d_logits = torch.empty(T, ctx.E, dtype=ctx.dtype, device=gates.device)
         lib = _C.lib()
@@ -61,7 +84,7 @@ class _RouteTopKSoftmax(torch.autograd.Function):
                     _C.dtype_code(ctx.dtype), _C.stream(),
                 )
             )
-        return d_logits, None, None
+        return d_logits, None, None, None
 
 
 def route_topk_softmax(logits: torch.Tensor, k: int, long_indices: bool = True) -> tuple[torch.Tensor, torch.Tensor]:
@@ -71,7 +94,10 @@ def route_topk_softmax(logits: torch.Tensor, k: int, long_indices: bool = True) 
     if is_tracing():
         gates, selected = _ops.route_topk_softmax(logits, k)
         return gates.to(logits.dtype), (selected.long() if long_indices else selected)
-    return _RouteTopKSoftmax.apply(logits, k, long_indices)
+    slot = _GateGradSlot()
+    gates, selected = _RouteTopKSoftmax.apply(logits, k, long_indices, slot)
+    gates._ck_gate_slot = slot  # found again by the expert block that consumes these gates (see _GateGradSlot)
+    return gates, selected
 
 
 @torch.no_grad()
@@ -138,14 +164,29 @@ def choose_align(num_rows: int, num_experts: int) -> int:
 
 
 @torch.no_grad()
-def sort_by_expert(expert_ids: torch.Tensor, num_experts: int, align: int | None = None) -> ExpertSegments:
-    """Stable sort of the flat (token, slot) expert ids, with counts / offsets and the tile-aligned segment tables."""
+def sort_by_expert(
+    expert_ids: torch.Tensor, num_experts: int, align: int | None = None, validate: bool = False
+) -> ExpertSegments:
+    """Stable sort of the flat (token, slot) expert ids, with counts / offsets and the tile-aligned segment tables.
+
+    Contract: every id lies in [0, num_experts) -- what a top-k over num_experts logits produces. An id outside that
+    range is dropped, not sorted (the reference's argsort / bincount path would keep it or raise): the counts exclude it,
+    ends[-1] falls short of the number of ids, and the last entries of sorted_expert_idxs / sorted_scattered_idxs and
+    the row_slot entries nobody owns stay unwritten. validate=True checks ends[-1] against the number of ids and raises
+    on a mismatch; it costs a device-to-host read, so the layer does not ask for it."""
     assert expert_ids.dtype in (torch.int32, torch.long)
     if align is None:
         align = choose_align(expert_ids.numel(), num_experts)
     if is_tracing():
         return _ops.sort_by_expert_segments(expert_ids, num_experts, align)
-    return _sort_by_expert_eager(expert_ids, num_experts, align)
+    seg = _sort_by_expert_eager(expert_ids, num_experts, align)
+    if validate and expert_ids.numel() > 0:
+        placed = int(seg.ends[-1])
+        if placed != expert_ids.numel():
+            raise ValueError(
+                f"sort_by_expert: {expert_ids.numel() - placed} of {expert_ids.numel()} expert ids lie outside [0, {num_experts})"
+            )
+    return seg
 
 
 def _sort_by_expert_eager(expert_ids: torch.Tensor, num_experts: int, align: int) -> ExpertSegments:
@@ -236,15 +277,12 @@ def _gemm(a, gather_div, w, seg: ExpertSegments, epilogue, y, y_t=None, aux=None
 
 
 def _bias_in_epilogue(seg: ExpertSegments, K: int) -> bool:
-    """Whether ck_grouped_gemm takes the per-expert bias as an operand of its grouped / scatter epilogue (the
-    256-row-tile kernel: the bias joins the fp32 accumulators and the output is rounded once, like F.linear); otherwise
-    the bias is added by its own kernel after the GEMM."""
+    """Whether ck_grouped_gemm takes the per-expert bias as an operand of its grouped / scatter epilogue (the bias joins
+    the fp32 accumulators and the output is rounded once, like F.linear). CK_GEMM_BIAS_FUSED=0 in the environment adds it
+    with its own kernel after the GEMM instead (two roundings; kept for comparison)."""
     import os
 
-    return (
-        seg.align == 256 and K % 64 == 0 and os.environ.get("CK_GEMM_LINE", "1") != "0"
-        and os.environ.get("CK_GEMM_PIPE", "1") != "0" and os.environ.get("CK_GEMM_BIAS_FUSED", "1") != "0"
-    )
+    return os.environ.get("CK_GEMM_BIAS_FUSED", "1") != "0"
 
 
 def _gemm_dx(d_y, w, seg: ExpertSegments, epilogue, out):
@@ -365,6 +403,20 @@ def _combine(expanded, gates, T, k, H, grad_out=None, want_out=True, want_d_gate
     return out, d_gates
 
 
+def _gate_grad(expanded, grad_out, T, k, H, gates_dtype, slot):
+    """d_gates in fp32 (kept in `slot` for the router's backward) and rounded to the gates' dtype for autograd."""
+    d32 = torch.empty(T, k, dtype=torch.float32, device=expanded.device)
+    with torch.cuda.device(expanded.device):
+        _C.check(
+            _C.lib().ck_gate_grad_f32(
+                _C.ptr(expanded), _C.ptr(grad_out), T, k, H, _C.ptr(d32), _C.dtype_code(expanded.dtype), _C.stream()
+            )
+        )
+    if slot is not None:
+        slot.d_gates_f32 = d32
+    return d32.to(gates_dtype)
+
+
 def gather_rows(src: torch.Tensor, idx: torch.Tensor, coeff: torch.Tensor | None = None, fan_out: int = 1) -> torch.Tensor:
     """out[n] = src[idx[n] // fan_out] * coeff[idx[n]] -- the reference's `group` (ops.py:108-140)."""
     _C.require_gpu(src, idx)
@@ -472,7 +524,8 @@ class _ExpertsDown(torch.autograd.Function):
     """h [max_rows, I] (padded grouped), gates [T, k] -> out [T, H]: the reference's c_proj with grouped_in=True."""
 
     @staticmethod
-    def forward(ctx, h, w, gates, seg: ExpertSegments, bias=None, slot_expert=None):
+    def forward(ctx, h, w, gates, seg: ExpertSegments, bias=None, slot_expert=None, gate_slot=None):
+        ctx.gate_slot = gate_slot
         h = h.contiguous()
         w = w.contiguous()
         gates = gates.contiguous()
@@ -497,7 +550,7 @@ class _ExpertsDown(torch.autograd.Function):
         grad_out = grad_out.contiguous()
         d_h = d_w = d_gates = d_bias = None
         if ctx.needs_input_grad[2]:
-            _, d_gates = _combine(expanded, None, T, k, N, grad_out=grad_out, want_out=False, want_d_gates=True)
+            d_gates = _gate_grad(expanded, grad_out, T, k, N, gates.dtype, ctx.gate_slot)
         need_w = ctx.needs_input_grad[1]
         rows_form = _dw_from_rows(seg.max_rows, seg.num_experts, seg.align, (N, K))
         d_y, d_y_t = _group_rows(grad_out, gates, k, seg, True, need_w and not rows_form)
@@ -513,7 +566,7 @@ class _ExpertsDown(torch.autograd.Function):
         if ctx.needs_input_grad[0]:
             d_h = torch.zeros(seg.max_rows, K, dtype=h.dtype, device=h.device)
             _gemm_dx(d_y, w, seg, _C.CK_EPI_GROUPED, d_h)
-        return d_h, d_w, d_gates, None, d_bias, None
+        return d_h, d_w, d_gates, None, d_bias, None, None
 
 
 def experts_up(
@@ -544,7 +597,7 @@ def experts_down(
             seg.max_rows, seg.num_experts, seg.align,
         )[0]
     _C.require_gpu(h, weight, gates, bias)
-    return _ExpertsDown.apply(h, weight, gates.to(h.dtype), seg, bias)
+    return _ExpertsDown.apply(h, weight, gates.to(h.dtype), seg, bias, None, _gate_slot(gates))
 
 
 # ---------------------------------------------------------------------------------------------------------------
@@ -555,7 +608,8 @@ class _SwigluExperts(torch.autograd.Function):
     epilogue and the SwiGLU backward fused into the epilogue of the c_proj input-gradient GEMM."""
 
     @staticmethod
-    def forward(ctx, x, w_fc, w_proj, gates, seg: ExpertSegments, act_kind: int = _C.CK_ACT_SWIGLU):
+    def forward(ctx, x, w_fc, w_proj, gates, seg: ExpertSegments, act_kind: int = _C.CK_ACT_SWIGLU, gate_slot=None):
+        ctx.gate_slot = gate_slot
         x = x.contiguous()
         w_fc = w_fc.contiguous()
         w_proj = w_proj.contiguous()
@@ -599,7 +653,7 @@ class _SwigluExperts(torch.autograd.Function):
         rows_form = _dw_from_rows(seg.max_rows, seg.num_experts, seg.align, (H, I), (two_i, H))  # as in forward
 
         if need_gates:
-            _, d_gates = _combine(expanded, None, T, k, H, grad_out=grad_out, want_out=False, want_d_gates=True)
+            d_gates = _gate_grad(expanded, grad_out, T, k, H, gates.dtype, ctx.gate_slot)
 
         # gate-scaled grad_out rows in padded grouped order (+ transpose for d_w_proj unless it reads rows)
         d_y, d_y_t = _group_rows(grad_out, gates, k, seg, True, need_proj and not rows_form)
@@ -643,7 +697,7 @@ class _SwigluExperts(torch.autograd.Function):
                 d_expanded = torch.empty(T * k, H, dtype=dt, device=dev)
                 _gemm_dx(d_pre, w_fc, seg, _C.CK_EPI_SCATTER, d_expanded)
                 d_x = d_expanded if k == 1 else _combine(d_expanded, None, T, k, H)[0]
-        return d_x, d_w_fc, d_w_proj, d_gates, None, None
+        return d_x, d_w_fc, d_w_proj, d_gates, None, None, None
 
 
 def swiglu_experts(
@@ -662,4 +716,4 @@ def swiglu_experts(
             grad and w_proj.requires_grad, grad and gates.requires_grad, act_kind,
         )[0]
     _C.require_gpu(x, w_fc, w_proj, gates)
-    return _SwigluExperts.apply(x, w_fc, w_proj, gates.to(x.dtype), seg, act_kind)
+    return _SwigluExperts.apply(x, w_fc, w_proj, gates.to(x.dtype), seg, act_kind, _gate_slot(gates))

@@ -81,7 +81,8 @@ int ck_route_topk_softmax_bwd(const float* gates, const float* d_gates, const in
  * Replaces: selected_experts.flatten().sort() and bincount(...).cumsum(-1) --
  *           cute_kernels/kernels/scattermoe/triton_implementation/__init__.py:82-83; the argsort / bincount of
  *           torch_implementation.py:171-193.
- * expert_ids: R = T*k flat ids (int32 or int64), all in [0, E). E <= 4096.
+ * expert_ids: R = T*k flat ids (int32 or int64), all in [0, E). E <= 4096. An id outside [0, E) is dropped: counts
+ *             exclude it, ends[E - 1] < R tells, and the tails of sorted_* stay unwritten (the caller's check).
  * Outputs (all int32 unless noted):
  *   sorted_expert_idxs[R], sorted_scattered_idxs[R]  -- the stable sort and its permutation
  *   counts[E], ends[E], starts[E] (uint32)            -- histogram, inclusive and exclusive prefix sums
@@ -115,6 +116,13 @@ int ck_gather_rows(const void* src, const int32_t* idx, const void* coeff, int32
  * may be NULL. gates / d_gates_out have the dtype of expanded. */
 int ck_combine_rows(const void* expanded, const void* gates, int64_t T, int32_t k, int32_t H, void* out,
                     const void* grad_out, void* d_gates_out, int32_t dtype, void* stream);
+
+/* d_gates[t, j] = <expanded[t, j, :], grad_out[t, :]> in fp32, whatever the dtype of the rows: the d_gates of
+ * cute_kernels/kernels/scattermoe/triton_implementation/ops.py:214 (a bmm in the activation dtype there) kept unrounded,
+ * so that the softmax backward of the router (ck_route_topk_softmax_bwd, fp32 d_gates) does not subtract rounded
+ * numbers. expanded [T * k, H], grad_out [T, H], d_gates [T, k]. */
+int ck_gate_grad_f32(const void* expanded, const void* grad_out, int64_t T, int32_t k, int32_t H, float* d_gates,
+                     int32_t dtype, void* stream);
 /* Padded grouped copy of token rows and (optionally) its transpose, for the grouped GEMMs below:
  *   row p valid : grouped[p, :] = src[row_slot[p] / fan_out, :] * (coeff ? coeff[row_slot[p]] : 1)
  *   row p pad   : zeros
@@ -163,8 +171,7 @@ typedef struct ck_segments {
  *                           zeros in pad rows, optional (NULL to skip)
  *   CK_EPI_SCATTER        : y [R, N]: valid row p is written to row row_slot[p] (back to (token, slot) order)
  *                           both: aux_in, if not NULL, is a bias [E, N] whose row e joins the fp32 accumulators of expert
- *                           e's rows before the one rounding (F.linear with a bias, torch_implementation.py:42); needs
- *                           seg->align == 256 and K % 64 == 0 (ck_add_expert_bias covers the other cases)
+ *                           e's rows before the one rounding (F.linear with a bias, torch_implementation.py:42)
  *   CK_EPI_SWIGLU         : N = 2*I packed [up | gate] (cute_kernels/kernels/swiglu/__init__.py:121): writes the
  *                           pre-activation to y [max_rows, 2I], act = up*silu(gate) (computed from the rounded
  *                           pre-activation, as the unfused path would) to aux [max_rows, I], and act^T to

@@ -77,9 +77,15 @@ def test_moe_layer_compiled(device, act, is_glu, add_bias):
     yc, logits_c = compiled(xc)
     yc.float().square().sum().backward()
     assert torch.equal(y, yc) and torch.equal(logits, logits_c)
-    assert torch.equal(xe.grad, xc.grad)
+    # Everything that does not pass through d_gates is bit-identical. The eager layer hands d_gates from the expert
+    # block to the router in fp32 (a side channel next to autograd); a traced graph carries it in the gates' dtype, as
+    # the reference does (ops.py:214). So the router's share of x.grad and gate.weight.grad differ by that one rounding.
     for n, p in moe.named_parameters():
-        assert torch.equal(eager_grads[n], p.grad), n
+        if n == "gate.weight":
+            torch.testing.assert_close(eager_grads[n].float(), p.grad.float(), rtol=2e-2, atol=2e-2 * float(p.grad.float().abs().max()))
+        else:
+            assert torch.equal(eager_grads[n], p.grad), n
+    torch.testing.assert_close(xe.grad.float(), xc.grad.float(), rtol=2e-2, atol=2e-2 * float(xc.grad.float().abs().max()))
     # inference: nothing is saved, nothing breaks
     with torch.no_grad():
         assert torch.equal(compiled(x)[0], moe(x)[0])

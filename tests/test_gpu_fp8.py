@@ -106,25 +106,35 @@ def test_moe_e4m3_layer_forward(device, dtype, T, E, k, H, I):
 
 
 def test_moe_e4m3_layer_at_c5_shape(device):
-    """The C5 benchmark shape (T = 65,536, H = 4,096, E = 128, top-8, I = 1,536) against the e4m3 oracle restated per
-    expert with torch's library routines on the device (quantise exactly as moe_oracle does, dequantise to fp32, F.linear
-    per expert segment, round where a 16-bit tensor sits). Stated fp8 tolerance rtol 5e-2 / atol 5e-2; parity of this
-    path is unpinned by the reference (it has no fp8 code)."""
+    """The C5 benchmark workload as bench.py runs it: T = 65,536, H = 4,096, E = 128, top-8, I = 1,536, behind an RMSNorm
+    prologue (eps 1e-6, weight ~ N(1, 0.02)) and with the rank-dependent router bias that gives a Zipf(0.8) expert load.
+    Checked against the e4m3 oracle restated per expert with torch's library routines on the device (quantise exactly
+    as moe_oracle does, dequantise to fp32, F.linear per expert segment, round where a 16-bit tensor sits). Stated fp8
+    tolerance rtol 5e-2 / atol 5e-2; the reference has no fp8 code, so this path has no upstream counterpart (the
+    oracle itself is pinned on the CPU against the e4m3 value table)."""
     torch.manual_seed(3)
     T, E, k, H, I = 65536, 128, 8, 4096, 1536
     dt = torch.bfloat16
     moe = cute_kernels.MoE(E, k, H, I, cute_kernels.swiglu_packed_cute, True, False, 0.02).to(dt).to(device)
-    q = cute_kernels.MoE_E4M3(moe)
     x = torch.randn(T, H, generator=torch.Generator().manual_seed(4)).to(dt).to(device)
+    w_norm = (1 + 0.02 * torch.randn(H, generator=torch.Generator().manual_seed(5))).to(dt).to(device)
+    ranks = torch.arange(1, E + 1, dtype=torch.float32, device=device)
+    bias = (-0.25 * torch.log(ranks)).to(dt)  # the scale bench.py's calibration finds for Zipf(0.8) at this shape
+    moe.gate.register_forward_hook(lambda mod, inp, out: out + bias)
+    q = cute_kernels.MoE_E4M3(moe)
     with torch.no_grad():
-        y, logits = q(x)
+        xn = cute_kernels.rmsnorm_cute(x, w_norm, 1e-6)
+        torch.testing.assert_close(xn.float(), mo.rmsnorm_torch(x, w_norm, 1e-6).float(), rtol=1e-2, atol=1e-2)
+        y, logits = q(xn)
         sel = cute_kernels.route_topk_softmax_raw(logits, k)[0].long()
+        load = torch.bincount(sel.flatten(), minlength=E).float()
+        assert float(load[:8].mean()) > 2.0 * float(load[-8:].mean())  # the skewed load really is exercised
         gates = torch.softmax(logits.gather(-1, sel).float(), dim=-1).to(dt)
         w1q, w1s = mo.quantize_rows_e4m3_torch(moe.c_fc.weight.flatten(0, 1))
         w2q, w2s = mo.quantize_rows_e4m3_torch(moe.c_proj.weight.flatten(0, 1))
         w1 = (w1q.float() * w1s[:, None]).view(E, 2 * I, H)
         w2 = (w2q.float() * w2s[:, None]).view(E, H, I)
-        xq, xs = mo.quantize_rows_e4m3_torch(x)
+        xq, xs = mo.quantize_rows_e4m3_torch(xn)
         xd = xq.float() * xs[:, None]
         expect = torch.zeros(T, H, dtype=torch.float32, device=device)
         for e in range(E):

@@ -289,14 +289,29 @@ class _OracleWithSelection(mo.MoEOracle):
 
 
 def _close_via_truth(ours, oracle, truth, what, rtol=RTOL, atol=ATOL):
-    ours, oracle, truth = ours.float().cpu(), oracle.float(), truth.float()
-    direct = (ours - oracle).abs() <= atol + rtol * oracle.abs()
-    via = (ours - truth).abs() <= (oracle - truth).abs() + atol + rtol * truth.abs()
+    """Per element: within atol * s + rtol * |x| of the oracle, or no further from the fp32 truth than the oracle is plus
+    that margin, where s is the RMS of the tensor (the absolute tolerance is stated in units of the tensor's typical
+    magnitude, so that it cannot exceed the signal it checks). Over the whole tensor: our RMS distance to the truth is at
+    most 1.1 x the oracle's -- an all-zero, mis-scaled or permuted result fails this whatever the tolerances."""
+    ours, oracle, truth = ours.detach().float().cpu(), oracle.detach().float().cpu(), truth.detach().float().cpu()
+    nonzero = int((truth != 0).sum())  # weight gradients of experts that received no token are exact zeros: leave them out of the scale
+    if nonzero == 0:  # e.g. gate.weight.grad with top-1 routing (a softmax over one logit is constant)
+        assert float(ours.abs().max()) <= 1e-3 and float(oracle.abs().max()) <= 1e-3, f"{what}: should vanish"
+        return
+    scale = float((truth.square().sum() / nonzero).sqrt())
+    direct = (ours - oracle).abs() <= atol * scale + rtol * oracle.abs()
+    via = (ours - truth).abs() <= (oracle - truth).abs() + atol * scale + rtol * truth.abs()
     bad = ~(direct | via)
-    assert not bad.any(), (
+    worst_ours, worst_oracle = float((ours - truth).abs().max()), float((oracle - truth).abs().max())
+    # one element per million may miss the per-element bound (a gate-weighted sum of rounded rows that cancel), but none
+    # may be further from the truth than 1.25 x the oracle's own worst element
+    assert int(bad.sum()) <= bad.numel() // 1_000_000 and worst_ours <= 1.25 * worst_oracle + atol * scale, (
         f"{what}: {int(bad.sum())}/{bad.numel()} elements off; worst |ours-oracle|={float((ours - oracle).abs().max()):.4g}, "
-        f"|ours-truth|={float((ours - truth).abs().max()):.4g}, |oracle-truth|={float((oracle - truth).abs().max()):.4g}"
+        f"|ours-truth|={worst_ours:.4g}, |oracle-truth|={worst_oracle:.4g}, rms={scale:.4g}"
     )
+    err_ours = float(((ours - truth).square().sum() / nonzero).sqrt())
+    err_oracle = float(((oracle - truth).square().sum() / nonzero).sqrt())
+    assert err_ours <= 1.1 * err_oracle + 2e-3 * scale, f"{what}: RMS error {err_ours:.4g} against the oracle's {err_oracle:.4g} (rms {scale:.4g})"
 
 
 def _acts(name):
@@ -310,14 +325,17 @@ def _acts(name):
 def _run_layer_case(device, dtype, T, E, k, H, I, act_name, x_shape=None, seed=42, add_bias=False):
     torch.manual_seed(seed)
     act_gpu, act_cpu, is_glu = _acts(act_name)
-    moe = cute_kernels.MoE(E, k, H, I, act_gpu, is_glu, add_bias, 0.02).to(dtype)
+    # weights ~ N(0, 1 / fan_in-ish): pre-activations, outputs and gradients are O(1), so the tolerances below (stated
+    # relative to each tensor's RMS) check real digits
+    std = 1.0 / (H ** 0.5)
+    moe = cute_kernels.MoE(E, k, H, I, act_gpu, is_glu, add_bias, std).to(dtype)
     if add_bias:  # the constructor zeroes biases (torch_implementation.py:56-60); give them values
         with torch.no_grad():
             moe.c_fc.bias.normal_(0, 0.1)
             moe.c_proj.bias.normal_(0, 0.1)
-    oracle = _OracleWithSelection(E, k, H, I, act_cpu, is_glu, add_bias, 0.02).to(dtype)
+    oracle = _OracleWithSelection(E, k, H, I, act_cpu, is_glu, add_bias, std).to(dtype)
     oracle.load_state_dict(moe.state_dict())  # same state_dict keys as the reference (scattermoe_test.py:83-94)
-    truth = _OracleWithSelection(E, k, H, I, act_cpu, is_glu, add_bias, 0.02).float()
+    truth = _OracleWithSelection(E, k, H, I, act_cpu, is_glu, add_bias, std).float()
     truth.load_state_dict({n: v.float() for n, v in moe.state_dict().items()})
     moe = moe.to(device)
 
@@ -361,14 +379,9 @@ def _run_layer_case(device, dtype, T, E, k, H, I, act_name, x_shape=None, seed=4
                 getattr(moe, name).bias.grad, getattr(oracle, name).bias.grad, getattr(truth, name).bias.grad,
                 f"{name}.bias.grad", atol=3e-2,
             )
-    # d_gates is rounded to the activation dtype by the reference's accelerated path (ops.py:214), by its torch path and
-    # by ours; the softmax backward then subtracts nearly equal numbers, so that one rounding -- not the kernels -- is
-    # the error floor of gate.weight.grad: about eps * max|d_gates| * max|x| per element.
-    eps = 2.0**-8 if dtype == torch.bfloat16 else 2.0**-11
-    floor = 2 * eps * float(truth.last_router_weights.grad.abs().max()) * float(x.float().abs().max())
-    _close_via_truth(
-        moe.gate.weight.grad, oracle.gate.weight.grad, truth.gate.weight.grad, "gate.weight.grad", atol=3e-2 + floor
-    )
+    # d_gates stays in fp32 between the expert block's backward and the router's (the reference rounds it to the
+    # activation dtype, ops.py:214, and so does the oracle): same tolerance as the other weight gradients
+    _close_via_truth(moe.gate.weight.grad, oracle.gate.weight.grad, truth.gate.weight.grad, "gate.weight.grad", atol=3e-2)
     return moe, oracle
 
 
@@ -459,13 +472,15 @@ def _close_via_truth_on_device(ours, oracle, truth, what, rtol=RTOL, atol=ATOL):
 
 
 @pytest.mark.parametrize(
-    "name,T,E,k,H,I,skew",
-    [("C3", 16384, 8, 2, 4096, 14336, 0.5), ("C4", 8192, 64, 8, 2048, 1408, 0.0)],
+    "name,T,E,k,H,I,skew,norm",
+    [("C3", 16384, 8, 2, 4096, 14336, 0.5, False), ("C4", 8192, 64, 8, 2048, 1408, 0.0, True)],
 )
-def test_moe_layer_at_full_baseline_shapes(device, name, T, E, k, H, I, skew):
-    """The benchmark's own shapes, forward and every gradient, against the oracle layer evaluated by torch's library
+def test_moe_layer_at_full_baseline_shapes(device, name, T, E, k, H, I, skew, norm):
+    """The benchmark's own workloads, forward and every gradient, against the oracle layer evaluated by torch's library
     routines on the same device (bf16, and fp32 as the truth that arbitrates rounding): same tolerances as the small
-    cases. `skew` > 0 adds the benchmark's rank-dependent router bias so that expert loads are ragged (Zipf-like)."""
+    cases. `skew` > 0 adds the benchmark's rank-dependent router bias so that expert loads are ragged (Zipf-like);
+    `norm` puts the RMSNorm prologue (eps 1e-6, weight ~ N(1, 0.02)) in front of the layer as bench.py does for C4:
+    rmsnorm_cute on our side, F.rms_norm in the oracle, gradients taken through it."""
     torch.manual_seed(7)
     dtype = torch.bfloat16
     moe = cute_kernels.MoE(E, k, H, I, cute_kernels.swiglu_packed_cute, True, False, 0.02).to(dtype)
@@ -481,6 +496,13 @@ def test_moe_layer_at_full_baseline_shapes(device, name, T, E, k, H, I, skew):
     x = torch.randn(T, H, generator=torch.Generator().manual_seed(1)).to(dtype).to(device)
     r = torch.randn(T, H, generator=torch.Generator().manual_seed(2)).to(dtype).to(device)
     xg, xo, xt = x.clone().requires_grad_(), x.clone().requires_grad_(), x.clone().float().requires_grad_()
+    hg, ho, ht = xg, xo, xt  # what the layer sees
+    if norm:
+        w_n = (1 + 0.02 * torch.randn(H, generator=torch.Generator().manual_seed(3))).to(dtype).to(device)
+        wg, wo, wt = w_n.clone().requires_grad_(), w_n.clone().requires_grad_(), w_n.clone().float().requires_grad_()
+        hg = cute_kernels.rmsnorm_cute(xg, wg, 1e-6)
+        ho = mo.rmsnorm_torch(xo, wo, 1e-6)
+        ht = mo.rmsnorm_torch(xt, wt, 1e-6)
 
     captured = {}
     orig = moe._compute_routing_weights
@@ -491,13 +513,13 @@ def test_moe_layer_at_full_baseline_shapes(device, name, T, E, k, H, I, skew):
         return out
 
     moe._compute_routing_weights = spy
-    y, logits = moe(xg)
+    y, logits = moe(hg)
     oracle.forced_selection = truth.forced_selection = captured["sel"]
     load = torch.bincount(captured["sel"].flatten(), minlength=E).float() / (T * k)
     if skew > 0:
         assert float(load.max()) > 2.5 * float(load.min())  # ragged segments really are exercised
-    yo, logits_o = oracle(xo)
-    yt, _ = truth(xt)
+    yo, logits_o = oracle(ho)
+    yt, _ = truth(ht)
     torch.testing.assert_close(logits.float(), logits_o.float(), rtol=RTOL, atol=ATOL)
     _close_via_truth_on_device(y, yo.detach(), yt.detach(), f"{name} output")
 
@@ -505,15 +527,15 @@ def test_moe_layer_at_full_baseline_shapes(device, name, T, E, k, H, I, skew):
     (yo * r).sum().backward()
     (yt * r.float()).sum().backward()
     _close_via_truth_on_device(xg.grad, xo.grad, xt.grad, f"{name} x.grad", atol=2e-2)
+    if norm:
+        _close_via_truth_on_device(wg.grad, wo.grad, wt.grad, f"{name} rmsnorm weight.grad", atol=3e-2)
     for pname in ["c_fc", "c_proj"]:
         _close_via_truth_on_device(
             getattr(moe, pname).weight.grad, getattr(oracle, pname).weight.grad, getattr(truth, pname).weight.grad,
             f"{name} {pname}.weight.grad", atol=3e-2,
         )
-    eps = 2.0**-8
-    floor = 2 * eps * float(truth.last_router_weights.grad.abs().max()) * float(x.float().abs().max())
     _close_via_truth_on_device(
-        moe.gate.weight.grad, oracle.gate.weight.grad, truth.gate.weight.grad, f"{name} gate.weight.grad", atol=3e-2 + floor
+        moe.gate.weight.grad, oracle.gate.weight.grad, truth.gate.weight.grad, f"{name} gate.weight.grad", atol=3e-2
     )
 
 

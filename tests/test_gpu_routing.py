@@ -194,3 +194,22 @@ def test_load_balancing_loss_matches_oracle(device, dtype, T, E, k):
     torch.testing.assert_close(lg.grad.float().cpu(), lo.grad, **gtol)
     f, P = cute_kernels.load_balancing_stats(lg.detach(), sel.to(device))
     assert abs(float(f.sum()) - k) < 1e-5 and abs(float(P.sum()) - 1.0) < 1e-2
+
+
+def test_sort_by_expert_out_of_range_ids_are_dropped_and_can_be_detected(device):
+    """The contract for ids outside [0, E): dropped from counts and offsets (ends[-1] < R), the rest sorted as if they
+    were not there; validate=True turns that into an error."""
+    ids = torch.tensor([3, 0, 7, 2, 2, -1, 1, 0, 9, 3], dtype=torch.int32)
+    E = 4
+    seg = cute_kernels.sort_by_expert(ids.to(device), E, 128)
+    keep = (ids >= 0) & (ids < E)
+    want_counts = torch.bincount(ids[keep].long(), minlength=E)
+    assert seg.counts.cpu().long().tolist() == want_counts.tolist()
+    placed = int(seg.ends[-1])
+    assert placed == int(keep.sum()) < ids.numel()
+    order = [i for e in range(E) for i in range(ids.numel()) if int(ids[i]) == e]  # stable sort of the valid ids
+    assert seg.sorted_scattered_idxs[:placed].cpu().tolist() == order
+    assert seg.sorted_expert_idxs[:placed].cpu().tolist() == sorted(ids[keep].tolist())
+    with pytest.raises(ValueError, match="outside"):
+        cute_kernels.sort_by_expert(ids.to(device), E, 128, validate=True)
+    cute_kernels.sort_by_expert(ids[keep].to(device), E, 128, validate=True)  # all in range: no error
