@@ -484,6 +484,32 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
     if (row_ok(lrow) && col_ok(c1) && (!(CK_ABLATE & 128) || prm.K == -12345)) store_out(ptr_of_row(lrow) + (uint32_t)c1 * 2u, v1);
     if (row_ok(lrow) && col_ok(c2) && (!(CK_ABLATE & 128) || prm.K == -12345)) store_out(ptr_of_row(lrow) + (uint32_t)c2 * 2u, v2);
   };
+  // The same for outputs whose rows are `pitch` bytes apart from a uniform base (every epilogue but the scatter one): the
+  // store takes the base in scalar registers and the lane's 32-bit byte offset (row_off: lane row * pitch, advanced by
+  // 16 rows per row block, + column bytes), so that it costs one or two 32-bit vector instructions and no 64-bit vector
+  // arithmetic; `inside`: the wave's whole tile lies inside the matrix and nothing is tested per store.
+  auto store_at = [&](char* base_u, uint32_t off, const vec16& v) {
+    const u32x4_t d = {v.w[0], v.w[1], v.w[2], v.w[3]};
+    if constexpr ((CK_ABLATE & 256) != 0) asm volatile("global_store_dwordx4 %0, %1, %2 nt" ::"v"(off), "v"(d), "s"(base_u) : "memory");
+    else asm volatile("global_store_dwordx4 %0, %1, %2" ::"v"(off), "v"(d), "s"(base_u) : "memory");
+  };
+  auto store_lines_at = [&](const vec16& v1, const vec16& v2, int j, char* base_u, uint32_t row_off, bool inside, bool row_in,
+                            int cols_left) {
+    const uint32_t o1 = row_off + (uint32_t)pair_col(j) * 2u, o2 = row_off + (uint32_t)pair_col(j + 2) * 2u;
+    if ((CK_ABLATE & 128) && prm.K != -12345) return;
+    if (inside) {
+      store_at(base_u, o1, v1);
+      store_at(base_u, o2, v2);
+    } else {
+      if (row_in && pair_col(j) < cols_left) store_at(base_u, o1, v1);
+      if (row_in && pair_col(j + 2) < cols_left) store_at(base_u, o2, v2);
+    }
+  };
+  auto uniform_out = [](char* p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<char*>(((uint64_t)hi << 32) | lo);
+  };
   const int64_t tile_row0 = m0 + wm * WM;  // first row of this wave's tile rows (padded row / dW row)
 
   if constexpr (MODE == kScatter) {  // output row of every tile row, through LDS (the stages are dead)
@@ -501,16 +527,18 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   };
   if constexpr (MODE == kDw) {
     const int64_t col0 = (int64_t)nt * BN + wn * WN;
-    char* base = reinterpret_cast<char*>(static_cast<T*>(prm.y) + (int64_t)expert * prm.M * prm.N + tile_row0 * prm.N + col0);
+    char* base = uniform_out(reinterpret_cast<char*>(static_cast<T*>(prm.y) + (int64_t)expert * prm.M * prm.N + tile_row0 * prm.N + col0));
     const uint32_t row_pitch = (uint32_t)prm.N * 2u;
     const int rows_left = (int)min((int64_t)WM, (int64_t)prm.M - tile_row0);   // rows of this wave that exist
     const int cols_left = (int)min((int64_t)WN, (int64_t)prm.N - col0);        // columns of this wave that exist
+    const bool inside = rows_left >= WM && cols_left >= WN;
+    uint32_t row_off = (uint32_t)lrow * row_pitch;
     static_for<MI>([&](auto i) {
       static_for<NI / 4>([&](auto jq) {
         const vec16 v1 = gather8_acc(acc[i][4 * jq], acc[i][4 * jq + 1]), v2 = gather8_acc(acc[i][4 * jq + 2], acc[i][4 * jq + 3]);
-        store_lines(v1, v2, 4 * jq, [&](int r) { return base + (uint32_t)(i * 16 + r) * row_pitch; },
-                    [&](int r) { return i * 16 + r < rows_left; }, [&](int c) { return c < cols_left; });
+        store_lines_at(v1, v2, 4 * jq, base, row_off, inside, i * 16 + lrow < rows_left, cols_left);
       });
+      row_off += 16u * row_pitch;
       __builtin_amdgcn_sched_barrier(0);  // row block by row block: the stores of one drain under the conversions of the next
     });
   } else if constexpr (MODE == kGrouped || MODE == kScatter) {
@@ -551,8 +579,10 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
         });
       });
     }
-    char* base = reinterpret_cast<char*>(y + tile_row0 * prm.N + col0);
+    char* base = uniform_out(reinterpret_cast<char*>(y + tile_row0 * prm.N + col0));
     const uint32_t row_pitch = (uint32_t)prm.N * 2u;
+    const bool inside = rows_left >= WM && cols_left >= WN;
+    uint32_t row_off = (uint32_t)lrow * row_pitch;
     static_for<MI>([&](auto i) {
       char* row_a = nullptr;  // scatter: the output row this lane writes in this row block
       if constexpr (MODE == kScatter) {
@@ -561,13 +591,14 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
       }
       static_for<NI / 4>([&](auto jq) {
         const vec16 v1 = gather8_acc(acc[i][4 * jq], acc[i][4 * jq + 1]), v2 = gather8_acc(acc[i][4 * jq + 2], acc[i][4 * jq + 3]);
-        store_lines(v1, v2, 4 * jq,
-                    [&](int r) {
-                      if constexpr (MODE == kScatter) return row_a;
-                      else return base + (uint32_t)(i * 16 + r) * row_pitch;
-                    },
-                    [&](int r) { return i * 16 + r < rows_left; }, [&](int c) { return c < cols_left; });
+        if constexpr (MODE == kScatter) {
+          store_lines(v1, v2, 4 * jq, [&](int) { return row_a; }, [&](int r) { return i * 16 + r < rows_left; },
+                      [&](int c) { return c < cols_left; });
+        } else {
+          store_lines_at(v1, v2, 4 * jq, base, row_off, inside, i * 16 + lrow < rows_left, cols_left);
+        }
       });
+      row_off += 16u * row_pitch;
       __builtin_amdgcn_sched_barrier(0);
     });
   } else {  // kSwiglu: the first half of a wave's column blocks are up, the second half the gate of the same activation columns
@@ -580,9 +611,11 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
     const int rows_left = (int)min((int64_t)WM, valid_end - tile_row0);
     constexpr int NH = NI / 2;  // column blocks per half
     static_assert(NH % 2 == 0, "whole block pairs in each half");
-    char* pre_base = reinterpret_cast<char*>(pre + tile_row0 * two_i + col0);
-    char* act_base = reinterpret_cast<char*>(act + tile_row0 * prm.I + col0);
+    char* pre_base = uniform_out(reinterpret_cast<char*>(pre + tile_row0 * two_i + col0));
+    char* act_base = uniform_out(reinterpret_cast<char*>(act + tile_row0 * prm.I + col0));
     const uint32_t pre_pitch = (uint32_t)two_i * 2u, act_pitch = (uint32_t)prm.I * 2u, gate_off = (uint32_t)prm.I * 2u;
+    const bool inside = rows_left >= WM && cols_left >= WN / 2;
+    uint32_t pre_off = (uint32_t)lrow * pre_pitch, act_off = (uint32_t)lrow * act_pitch;
     static_for<MI>([&](auto i) {
       const int r = i * 16 + lrow;
       const bool valid = r < rows_left;
@@ -619,11 +652,11 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
         vg_[jp] = vg;
         va_[jp] = va;
       });
-      auto rows_ok = [&](int r) { return i * 16 + r < rows_left; };
-      auto cols_ok = [&](int c) { return c < cols_left; };
-      store_lines(vu_[0], vu_[1], 0, [&](int r) { return pre_base + (uint32_t)(i * 16 + r) * pre_pitch; }, rows_ok, cols_ok);
-      store_lines(vg_[0], vg_[1], 0, [&](int r) { return pre_base + (uint32_t)(i * 16 + r) * pre_pitch + gate_off; }, rows_ok, cols_ok);
-      store_lines(va_[0], va_[1], 0, [&](int r) { return act_base + (uint32_t)(i * 16 + r) * act_pitch; }, rows_ok, cols_ok);
+      store_lines_at(vu_[0], vu_[1], 0, pre_base, pre_off, inside, valid, cols_left);
+      store_lines_at(vg_[0], vg_[1], 0, pre_base, pre_off + gate_off, inside, valid, cols_left);
+      store_lines_at(va_[0], va_[1], 0, act_base, act_off, inside, valid, cols_left);
+      pre_off += 16u * pre_pitch;
+      act_off += 16u * act_pitch;
       __builtin_amdgcn_sched_barrier(0);
     });
   }
