@@ -2,27 +2,32 @@
 // Forward (inference) only: Y = (A_e * diag(a_scale)) (W[e] * diag(w_scale[e]))^T, the two scale vectors applied to the
 // fp32 accumulators in the epilogue.
 //
-// Same machinery as the 16-bit kernel with 128-byte LDS rows (tile-aligned expert segments, 256x256 tile, 8 waves,
-// global -> LDS direct loads of whole cache lines, two XOR-swizzled stages, hand-ordered load / fragment-read / MFMA
-// stream, LDS-staged epilogue), with one byte per element: a K step is 128 elements = two v_mfma_f32_32x32x64_f8f6f4 per
-// 32 x 32 block (twice the rate of the 16-bit MFMA), fragments are 32 bytes per lane, and every byte fetched from L2
-// carries twice the FLOPs.
+// Same machinery as the 16-bit kernel with 128-byte LDS rows (grouped_gemm_line.hip): tile-aligned expert segments,
+// 256 x 256 tile, four waves (one per SIMD) with 128 x 128 wave tiles and the accumulators pinned to AGPRs, global -> LDS
+// direct loads of whole cache lines from a scalar base, two XOR-swizzled stages, and an epilogue straight from the
+// accumulators. One byte per element: a K step is 128 elements = one v_mfma_f32_16x16x128_f8f6f4 per 16 x 16 block
+// (twice the rate of the 16-bit MFMA; on random e4m3 operands a register-only loop of this shape sustains 4.3 PFLOP/s,
+// the 32x32x64 shape 3.9), fragments are 32 bytes per lane, and every byte fetched from L2 carries twice the FLOPs.
+// A step is a single slice, so there is one fragment set and it rotates: the registers of A row block i are reloaded
+// from the next stage as soon as row block i has been multiplied, those of B block j behind the last row block. The
+// barrier therefore sits at the start of a step (the next stage must have landed before the first reload), and the loads
+// of step kt + 2 go out in the first half of step kt so that the last of them still has half a step to land.
 #include <stdlib.h>
 
 #include "gemm_common.h"
 
 #ifndef CK_ABLATE
-#define CK_ABLATE 0  // measurement builds only: 2 no loads in the loop, 4 no fragment reads, 32 no epilogue, 64 no MFMA, 128 no main loop
+#define CK_ABLATE 0  // measurement builds only: 2 no loads in the loop, 4 no fragment reads, 32 no epilogue, 64 no MFMA
 #endif
 
 namespace ck {
 namespace {
 
 constexpr int BM = 256, BN = 256;
-constexpr int WGM = 4, NW = WGM * 2, NT = 64 * NW;  // 8 waves: 4 along M, 2 along N
-constexpr int WM = BM / WGM, WN = BN / 2;           // 64 x 128 wave tile
-constexpr int MI = WM / 32, NI = WN / 32;
-constexpr int BK = 128, KS = BK / 64, NSTAGE = 2;
+constexpr int WGM = 2, NW = WGM * 2, NT = 64 * NW;  // 4 waves: 2 along M, 2 along N
+constexpr int WM = BM / WGM, WN = BN / 2;           // 128 x 128 wave tile
+constexpr int MI = WM / 16, NI = WN / 16;
+constexpr int BK = 128, NSTAGE = 2;
 constexpr int kRowBytes = BK;  // one cache line per tile row and K step
 constexpr int kStageBytes = (BM + BN) * kRowBytes;
 constexpr int A_LD = BM * kRowBytes / (1024 * NW), B_LD = BN * kRowBytes / (1024 * NW);
@@ -30,18 +35,23 @@ constexpr int A_LD = BM * kRowBytes / (1024 * NW), B_LD = BN * kRowBytes / (1024
 // all 64 banks once (even rows cover banks 0-31 with 8 distinct slots, odd rows 32-63)
 __device__ inline int swz128(int row) { return (row >> 1) & 7; }
 constexpr int kLoadsPerStep = A_LD + B_LD;
+constexpr int kLoadGap = 2;  // MFMAs between two loads of the next-but-one K step: all out in the first half of a step
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef int i32x8 __attribute__((ext_vector_type(8)));
-constexpr int kMetaOffset = NSTAGE * kStageBytes;  // after the stages: a_scale of the tile's rows, w_scale of its columns,
-constexpr int kMetaBytes = (BM + BN + BM) * 4;      // and the output row of every tile row (scatter epilogue)
-constexpr size_t kLdsBytes = (size_t)kMetaOffset + kMetaBytes;
-static_assert(NT == BM + BN, "one thread per tile row / tile column fetches the epilogue's scales");
+constexpr size_t kLdsBytes = (size_t)NSTAGE * kStageBytes;
+static_assert(kLoadsPerStep * kLoadGap <= MI * NI && NT == BM, "loads fit a step; one thread per tile row");
+
+__device__ inline void mfma_fp8(const i32x8& a, const i32x8& b, f32x4& c) {
+  // cbsz = blgp = 0: both operands e4m3; accumulator pinned to AGPRs and updated in place (see Mfma16::run_acc)
+  asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+}
 
 template <typename TO, int MODE>
 __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams prm) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   char* lds_c = reinterpret_cast<char*>(lds_raw);
-  const int tid = threadIdx.x, lane = tid & (kWave - 1), wave = tid / kWave;
+  const int tid = threadIdx.x, lane = tid & (kWave - 1);
+  const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
   const int wm = wave >> 1, wn = wave & 1;
 
   // ---- which tile (same XCD-aware order as the 16-bit kernel)
@@ -57,22 +67,13 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
   const int64_t m0 = (int64_t)mt * BM;
   const int64_t valid_end = (int64_t)prm.seg_starts[expert] + prm.counts[expert];
 
-#if (CK_ABLATE & 256)
-  auto stamp = [&](int i) {
-    __builtin_amdgcn_s_waitcnt(0);
-    if (prm.y_t != nullptr && tid == 0) static_cast<uint64_t*>(prm.y_t)[(size_t)blockIdx.x * 8 + i] = wall_clock64();
-  };
-#else
-  auto stamp = [&](int) {};
-#endif
-  stamp(0);
-  f32x16 acc[MI][NI];
+  f32x4 acc[MI][NI];
 #pragma unroll
   for (int i = 0; i < MI; ++i)
 #pragma unroll
     for (int j = 0; j < NI; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
 
   // ---- global -> LDS addressing: lane l of a wave-load fills slot l (16 bytes) of 64 consecutive slots = 8 rows of 128 B
   const char* a_base = static_cast<const char*>(prm.a);
@@ -92,7 +93,7 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
     const int j = (wave * B_LD + t) * 8 + (lane >> 3);
     const int c = (lane & 7) ^ swz128(j);
     int64_t n;
-    if constexpr (MODE == kSwiglu) {
+    if constexpr (MODE == kSwiglu) {  // a wave's WN tile columns: WN/2 up columns, then the gate columns of the same outputs
       const int half = (j % WN) / (WN / 2);
       const int within = (j / WN) * (WN / 2) + (j % (WN / 2));
       n = (int64_t)half * prm.I + min((int64_t)nt * (BN / 2) + within, (int64_t)prm.I - 1);
@@ -101,34 +102,31 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
     }
     b_off[t] = (uint32_t)(n * prm.ldw + c * 16);
   }
-  const int nk = (CK_ABLATE & 128) ? 0 : prm.K / BK;  // 128: no main loop at all
+  const int nk = prm.K / BK;
 
-  // ---- what the epilogue needs from global memory is fetched now and parked in LDS after the main loop: thread t < BM
-  // takes tile row t (its de-quantisation scale and, for the scatter epilogue, its output row), thread BM + j column j
+  // ---- what the epilogue needs per tile row is fetched now and parked in LDS after the main loop: thread t takes tile
+  // row t (its de-quantisation scale and, for the scatter epilogue, its output row)
   float meta_scale = 0.f;
   int meta_row = -1;
-  if (tid < BM) {
+  {
     const int64_t p = m0 + tid;
     if (p < valid_end) {
       const int slot = (prm.a_gather_div > 0 || MODE == kScatter) ? prm.row_slot[p] : 0;
       meta_scale = prm.a_scale[prm.a_gather_div > 0 ? (int64_t)(slot / prm.a_gather_div) : p];
       meta_row = (MODE == kScatter) ? slot : tid;
     }
-  } else {
-    const int j = tid - BM;
-    const float* w_scale = prm.w_scale + (int64_t)expert * prm.N;
-    if constexpr (MODE == kSwiglu) {  // columns 0 .. 127: up scales of the tile's activation columns; 128 .. 255: gate
-      const int64_t col = (int64_t)nt * (BN / 2) + (j & (BN / 2 - 1));
-      if (col < prm.I) meta_scale = w_scale[(j < BN / 2 ? 0 : prm.I) + col];
-    } else {
-      const int64_t n = (int64_t)nt * BN + j;
-      if (n < prm.N) meta_scale = w_scale[n];
-    }
   }
 
-  auto dma16 = [&](const char* src, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_addr), "v"(src) : "m0");
+  auto dma16 = [&](const char* base, uint32_t off, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(off), "s"(base) : "m0");
   };
+  auto uniform_ptr = [](const char* p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<const char*>(((uint64_t)hi << 32) | lo);
+  };
+  const char* a_base_u = uniform_ptr(a_base);
+  const char* b_base_u = uniform_ptr(b_base);
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds_c;
   const uint32_t wave_a = __builtin_amdgcn_readfirstlane(lds_base + wave * A_LD * 1024);
   const uint32_t wave_b = __builtin_amdgcn_readfirstlane(lds_base + BM * kRowBytes + wave * B_LD * 1024);
@@ -138,34 +136,28 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
     if constexpr ((CK_ABLATE & 2) != 0) {
       if (step >= NSTAGE) return;
     }
-    if (g < A_LD) dma16(a_base + kb + a_off[g], wave_a + st + g * 1024);
-    else dma16(b_base + kb + b_off[g - A_LD], wave_b + st + (g - A_LD) * 1024);
+    if (g < A_LD) dma16(a_base_u + kb, a_off[g], wave_a + st + g * 1024);
+    else dma16(b_base_u + kb, b_off[g - A_LD], wave_b + st + (g - A_LD) * 1024);
   };
   auto issue = [&](int step) {
 #pragma unroll
     for (int g = 0; g < kLoadsPerStep; ++g) issue_one(step, g);
   };
 
-  // ---- fragments for v_mfma_f32_32x32x64_f8f6f4: slice sl (64 of the row's 128 bytes) of row l % 32 -- lane l holds its
-  // 16-byte chunks 4 sl + 2 h and 4 sl + 2 h + 1, h = l / 32. Both operands use the same byte -> k assignment, which is
-  // all a dot product needs.
-  const int fsw = swz128(lane & 31), fh = lane >> 5;
-  int chunk_lo[KS], chunk_hi[KS];
-#pragma unroll
-  for (int sl = 0; sl < KS; ++sl) {
-    chunk_lo[sl] = ((4 * sl + 2 * fh) ^ fsw) * 16;
-    chunk_hi[sl] = ((4 * sl + 2 * fh + 1) ^ fsw) * 16;
-  }
-  const int fa_row = (wm * WM + (lane & 31)) * kRowBytes;
-  const int fb_row = BM * kRowBytes + (wn * WN + (lane & 31)) * kRowBytes;
+  // ---- fragments for v_mfma_f32_16x16x128_f8f6f4: row l % 16, contraction bytes 32 (l / 16) .. + 31 = the row's 16-byte
+  // chunks 2 (l / 16) and 2 (l / 16) + 1. Both operands use the same byte -> k assignment, which is all a dot product needs.
+  const int fsw = swz128(lane & 15), fq = lane >> 4;
+  const int chunk_lo = ((2 * fq) ^ fsw) * 16, chunk_hi = ((2 * fq + 1) ^ fsw) * 16;
+  const int fa_row = (wm * WM + (lane & 15)) * kRowBytes;
+  const int fb_row = BM * kRowBytes + (wn * WN + (lane & 15)) * kRowBytes;
   i32x8 fa[MI], fb[NI];
-  auto read_frag = [&](int stage, int sl, int g) {  // g < MI: A block g; else B block g - MI
+  auto read_frag = [&](int stage, int g) {  // g < MI: A block g; else B block g - MI
     if constexpr ((CK_ABLATE & 4) != 0) {
-      if (stage != 0 || sl != 0) return;
+      if (stage != 0) return;
     }
-    const char* row = lds_c + stage * kStageBytes + (g < MI ? fa_row + g * 32 * kRowBytes : fb_row + (g - MI) * 32 * kRowBytes);
-    const i32x4 lo = *reinterpret_cast<const i32x4*>(row + chunk_lo[sl]);
-    const i32x4 hi = *reinterpret_cast<const i32x4*>(row + chunk_hi[sl]);
+    const char* row = lds_c + stage * kStageBytes + (g < MI ? fa_row + g * 16 * kRowBytes : fb_row + (g - MI) * 16 * kRowBytes);
+    const i32x4 lo = *reinterpret_cast<const i32x4*>(row + chunk_lo);
+    const i32x4 hi = *reinterpret_cast<const i32x4*>(row + chunk_hi);
     const i32x8 v = __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
     if (g < MI) fa[g] = v;
     else fb[g - MI] = v;
@@ -175,10 +167,8 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
       asm volatile("" ::"v"(fa[i]), "v"(fb[j]));
       return;
     }
-    // scale operands 0: the compiler emits the unscaled v_mfma_f32_32x32x64_f8f6f4 (both operands e4m3: cbsz = blgp = 0)
-    acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa[i], fb[j], acc[i][j], 0, 0, 0, 0, 0, 0);
+    mfma_fp8(fb[j], fa[i], acc[i][j]);  // weight fragment first: a lane gets 4 consecutive output columns of one row
   };
-  static_assert(MI == 2 && NI == 4 && kLoadsPerStep == 8 && KS == 2, "the hand schedule below is written for this shape");
 
   if (nk > 0) {
     issue(0);
@@ -189,176 +179,171 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
       asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     }
 #pragma unroll
-    for (int g = 0; g < MI + NI; ++g) read_frag(0, 0, g);
-    // One 64-byte slice = one MFMA per 32 x 32 block. Fragments are single-buffered and rotate: as soon as the last MFMA
-    // that needs a fragment has issued, the same registers are reloaded for the next slice.
-    // Slice 0: the next slice is in the same stage. Slice 1 (last): the next slice is slice 0 of step kt + 1 in the other
-    // stage -- phase 0 / 1: wait for that stage (the only loads in flight) and for this wave's own fragment reads, then
-    // meet the other waves; the whole current stage has been read by everyone, so in phase 0 the loads of step kt + 2
-    // overwrite it under this slice's MFMAs. Phase 1 is step nk - 2 (nothing left to fetch), phase 2 the last step.
-    auto slice = [&](int kt, auto sl, auto phase) {
-      constexpr bool kLast = decltype(sl)::value == KS - 1;
+    for (int g = 0; g < MI + NI; ++g) read_frag(0, g);
+
+    // One K step: MI x NI MFMAs, row block by row block. Phase 0 / 1 (not the last step): first wait for the next stage
+    // (the only loads in flight) and for this wave's own fragment reads of the step before, then meet the other waves --
+    // every wave holds the current step's fragments in registers, so the current stage is free: in phase 0 the loads of
+    // step kt + 2 overwrite it, one every kLoadGap MFMAs. fa[i] is reloaded from the next stage once row block i is
+    // done, fb[j] after the MFMA (MI - 1, j). Phase 1 is step nk - 2 (nothing left to fetch), phase 2 the last step
+    // (nothing to wait for, nothing to reload).
+    auto k_step = [&](int kt, auto phase, auto idle) {
+      constexpr bool kIdle = decltype(idle)::value;  // this wave's rows are all pad rows: no fragments, no MFMAs
       constexpr int kPhase = decltype(phase)::value;
-      const int ns = kLast ? (kt + 1) & (NSTAGE - 1) : kt & (NSTAGE - 1);
-      constexpr int nsl = kLast ? 0 : decltype(sl)::value + 1;
-      constexpr bool kReload = !(kLast && kPhase == 2);
-      constexpr bool kIssue = kLast && kPhase == 0;
-      if constexpr (kLast && kPhase < 2) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+      const int ns = (kt + 1) & (NSTAGE - 1);
+      if constexpr (kPhase < 2) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
 #pragma unroll
-      for (int j = 0; j < NI; ++j) {
-        mfma(0, j);
-        if constexpr (kIssue) issue_one(kt + 2, j);
+      for (int n = 0; n < MI * NI; ++n) {
+        const int i = n / NI, j = n % NI;
+        if constexpr (!kIdle) mfma(i, j);
+        if constexpr (kPhase == 0) {
+          if (n % kLoadGap == 0 && n / kLoadGap < kLoadsPerStep) issue_one(kt + 2, n / kLoadGap);
+        }
         __builtin_amdgcn_sched_barrier(0);
+        if constexpr (kPhase < 2 && !kIdle) {
+          if (j == NI - 1) read_frag(ns, i);
+          if (i == MI - 1) read_frag(ns, MI + j);
+        }
       }
-      if constexpr (kReload) read_frag(ns, nsl, 0);
-#pragma unroll
-      for (int j = 0; j < NI; ++j) {
-        mfma(1, j);
-        if constexpr (kIssue) issue_one(kt + 2, NI + j);
-        __builtin_amdgcn_sched_barrier(0);
-        if constexpr (kReload) read_frag(ns, nsl, MI + j);
-      }
-      if constexpr (kReload) read_frag(ns, nsl, 1);
       __builtin_amdgcn_sched_barrier(0);
     };
-    auto k_step = [&](int kt, auto phase) { static_for<KS>([&](auto sl) { slice(kt, sl, phase); }); };
-    int kt = 0;
-    for (; kt + 2 < nk; ++kt) k_step(kt, std::integral_constant<int, 0>{});
-    if (kt + 2 == nk) k_step(kt++, std::integral_constant<int, 1>{});
-    k_step(kt, std::integral_constant<int, 2>{});
-  }
-
-  // ---- epilogue through LDS (see the 16-bit kernel): slab S[col][row] of 128 tile columns, 8-byte writes from the
-  // accumulator layout, ds_read_b64_tr_b16 back out so that a lane stores 8 consecutive columns of one row
-  typedef __attribute__((__vector_size__(4 * sizeof(short)))) short s16x4;
-  constexpr int kSlabCols = 128, kSlabLd = BM + 4;
-  TO* slab = reinterpret_cast<TO*>(lds_raw);
-  stamp(2);
-  float* meta_f = reinterpret_cast<float*>(lds_c + kMetaOffset);    // [0, BM): a scales; [BM, BM + BN): w scales
-  int* meta_rows = reinterpret_cast<int*>(lds_c + kMetaOffset) + BM + BN;  // [BM]: output row, -1 for a pad row
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-  meta_f[tid] = meta_scale;
-  if (tid < BM) meta_rows[tid] = meta_row;
-  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
-  stamp(3);
-  const int col_in_block = lane & 31;
-  const int row_quad = (lane >> 5) * 4;
-
-  // de-quantisation scales of the rows this lane holds (0 for pad rows)
-  float rs[MI][4][4];
-#pragma unroll
-  for (int i = 0; i < MI; ++i)
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-      const float4 v = *reinterpret_cast<const float4*>(meta_f + wm * WM + i * 32 + 8 * q + row_quad);
-      rs[i][q][0] = v.x;
-      rs[i][q][1] = v.y;
-      rs[i][q][2] = v.z;
-      rs[i][q][3] = v.w;
-    }
-
-  stamp(4);
-  auto stage_blocks = [&](auto&& value) {
-    static_for<MI>([&](auto i) {
-      static_for<2>([&](auto jj) {
-        static_for<4>([&](auto q) {
-          const int r = wm * WM + i * 32 + 8 * q + row_quad;
-          const int c = wn * 64 + jj * 32 + col_in_block;
-          store4(slab + c * kSlabLd + r, value(i, jj, q, std::integral_constant<int, 0>{}),
-                 value(i, jj, q, std::integral_constant<int, 1>{}), value(i, jj, q, std::integral_constant<int, 2>{}),
-                 value(i, jj, q, std::integral_constant<int, 3>{}));
-        });
-      });
-    });
-  };
-  // Row-major drain as in the 16-bit kernel: 16 lanes take a 4-row x 32-column block, the four lane groups of a wave two
-  // adjacent column blocks of two adjacent row blocks (whole 128-byte lines per store instruction); rows and column pairs
-  // are walked in unrolled loops, so every address is a per-lane base plus a compile-time offset. row_ptr(tile row) ->
-  // address of the output row at the tile's first column (nullptr: pad row), block_col(cb) -> output column of slab
-  // column block cb relative to that, cols_left = valid columns from there on, tile_cols = columns the tile spans.
-  auto drain_rows = [&](auto&& row_ptr, auto&& block_col, int64_t cols_left, int tile_cols) {
-    const int l16 = tid & 15, csel = (tid >> 4) & 1, rsel = (tid >> 5) & 1;
-    const int tq = l16 & 3, tj = l16 >> 2;
-    const int oq = l16 >> 2, oe = l16 & 3;
-    constexpr int kColPairs = kSlabCols / 64, kRowIters = (BM / 4) / (2 * NT / kWave);
-    static_assert(kSlabCols % 64 == 0 && (BM / 4) % (2 * NT / kWave) == 0, "whole column pairs and row iterations");
-    const bool cols_full = cols_left >= tile_cols;
-    auto body = [&](auto checked) {
-      static_for<kRowIters>([&](auto it) {
-        const int rb = (it * (NT / kWave) + wave) * 2 + rsel;
-        TO* dst_row = row_ptr(rb * 4 + oe);
-        if (dst_row != nullptr) dst_row += 8 * oq;
-        const TO* src_row = slab + (csel * 32 + 8 * tq + tj) * kSlabLd + rb * 4;
-        static_for<kColPairs>([&](auto cp) {
-          const TO* src = src_row + cp * 64 * kSlabLd;
-          const s16x4 lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(src));
-          const s16x4 hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(src + 4 * kSlabLd));
-          const int col = csel ? block_col(std::integral_constant<int, 2 * decltype(cp)::value + 1>{})
-                               : block_col(std::integral_constant<int, 2 * decltype(cp)::value>{});
-          if (dst_row != nullptr && (!checked || col + 8 * oq < cols_left)) {
-            vec16 v;
-            v.w[0] = (uint16_t)lo[0] | ((uint32_t)(uint16_t)lo[1] << 16);
-            v.w[1] = (uint16_t)lo[2] | ((uint32_t)(uint16_t)lo[3] << 16);
-            v.w[2] = (uint16_t)hi[0] | ((uint32_t)(uint16_t)hi[1] << 16);
-            v.w[3] = (uint16_t)hi[2] | ((uint32_t)(uint16_t)hi[3] << 16);
-            store16_nt(dst_row + col, v);
-          }
-        });
-      });
+    auto k_loop = [&](auto idle) {
+      int kt = 0;
+      for (; kt + 2 < nk; ++kt) k_step(kt, std::integral_constant<int, 0>{}, idle);
+      if (kt + 2 == nk) k_step(kt++, std::integral_constant<int, 1>{}, idle);
+      k_step(kt, std::integral_constant<int, 2>{}, idle);
     };
-    if (cols_full) body(std::false_type{});
-    else body(std::true_type{});
-  };
-  const float* w_sc = meta_f + BM;
+    const bool wave_idle = m0 + wm * WM >= valid_end;
+    if (__builtin_amdgcn_readfirstlane(wave_idle)) k_loop(std::true_type{});
+    else k_loop(std::false_type{});
+  }
+  mfma_drain();
 
+  // ---- epilogue, straight from the accumulators (as in the 16-bit kernel): a lane holds, per 16x16 block (i, j), the 4
+  // consecutive output columns j * 16 + 4 (lane / 16) + 0..3 of tile row i * 16 + lane % 16; both scales are applied in
+  // fp32, pairs are rounded and packed by one conversion, and v_permlane16_swap regroups two column blocks into 8
+  // consecutive columns per lane, so that every lane stores 16 bytes.
+  float* meta_f = reinterpret_cast<float*>(lds_c);  // [BM] a_scale of the tile's rows, then [BM] output rows (scatter)
+  int* meta_rows = reinterpret_cast<int*>(lds_c + BM * 4);
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");  // every wave is done with the stages
+  meta_f[tid] = meta_scale;
+  meta_rows[tid] = meta_row;
+  __syncthreads();
   if constexpr ((CK_ABLATE & 32) != 0) {
     float sum = 0.f;
-    static_for<MI>([&](auto i) { static_for<NI>([&](auto j) { static_for<16>([&](auto r) { sum += acc[i][j][(int)r]; }); }); });
-    if (sum == 12345.678f) static_cast<TO*>(prm.y ? prm.y : prm.aux)[tid] = Elem<TO>::down(sum + rs[0][0][0]);
-  } else if constexpr (MODE == kGrouped || MODE == kScatter) {
-    TO* y = static_cast<TO*>(prm.y);
-    static_for<2>([&](auto pass) {
-      float cs[2];
-      static_for<2>([&](auto jj) { cs[jj] = w_sc[wn * WN + (pass * 2 + jj) * 32 + col_in_block]; });
-      stage_blocks([&](auto i, auto jj, auto q, auto s) {
-        return Elem<TO>::down(acc[i][pass * 2 + jj][4 * q + s] * rs[i][q][s] * cs[jj]);
-      });
-      __syncthreads();
-      if constexpr (pass == 0) stamp(6);
-      drain_rows(
-          [&](int r) -> TO* {
-            const int out_row = meta_rows[r];
-            if (out_row < 0) return nullptr;
-            const int64_t row = (MODE == kScatter) ? (int64_t)out_row : m0 + r;
-            return y + row * prm.N + (int64_t)nt * BN;
-          },
-          [&](auto cb) { return ((cb * 32) >> 6) * WN + pass * 64 + ((cb * 32) & 63); }, prm.N - (int64_t)nt * BN, BN);
-      if constexpr (pass == 0) stamp(7);
-      __syncthreads();
-    });
-  } else {  // kSwiglu: blocks 0, 1 = up, blocks 2, 3 = gate of the same activation columns; only the activation is kept
-    TO* act = static_cast<TO*>(prm.aux);
-    float cs_up[2], cs_gate[2];
-    static_for<2>([&](auto jj) {
-      cs_up[jj] = w_sc[wn * (WN / 2) + jj * 32 + col_in_block];
-      cs_gate[jj] = w_sc[BN / 2 + wn * (WN / 2) + jj * 32 + col_in_block];
-    });
-    stage_blocks([&](auto i, auto jj, auto q, auto s) {
-      // rounded to the output type first, like a pre-activation tensor would be
-      const TO up = Elem<TO>::down(acc[i][jj][4 * q + s] * rs[i][q][s] * cs_up[jj]);
-      const TO gate = Elem<TO>::down(acc[i][jj + 2][4 * q + s] * rs[i][q][s] * cs_gate[jj]);
-      const float gf = Elem<TO>::up(gate);
-      return Elem<TO>::down(Elem<TO>::up(up) * gf * sigmoid_fast(gf));
-    });
-    __syncthreads();
-    drain_rows(
-        [&](int r) -> TO* {
-          const int64_t p = m0 + r;
-          return p < valid_end ? act + p * prm.I + (int64_t)nt * (BN / 2) : nullptr;
-        },
-        [&](auto cb) { return ((cb * 32) >> 6) * (WN / 2) + ((cb * 32) & 63); }, prm.I - (int64_t)nt * (BN / 2), BN / 2);
+    static_for<MI>([&](auto i) { static_for<NI>([&](auto j) { static_for<4>([&](auto r) { sum += acc[i][j][(int)r]; }); }); });
+    if (sum == 12345.678f) static_cast<TO*>(prm.y ? prm.y : prm.aux)[tid] = Elem<TO>::down(sum);
+    return;
   }
-  stamp(5);
+  const int lrow = lane & 15, lg = lane >> 4;
+  const bool odd_group = (lg & 1) != 0;
+  auto gather8 = [&](uint32_t p0, uint32_t p1, uint32_t q0, uint32_t q1) {
+    const auto s0 = __builtin_amdgcn_permlane16_swap(p0, q0, false, false);  // odd rows of p <-> even rows of q
+    const auto s1 = __builtin_amdgcn_permlane16_swap(p1, q1, false, false);
+    vec16 v;
+    v.w[0] = s0[0];
+    v.w[1] = s1[0];
+    v.w[2] = s0[1];
+    v.w[3] = s1[1];
+    return v;
+  };
+  auto pair_col = [&](int j) { return (j + (odd_group ? 1 : 0)) * 16 + 4 * (lg & ~1); };
+  auto store_at = [&](char* base_u, uint32_t off, const vec16& v) {
+    const u32x4_t d = {v.w[0], v.w[1], v.w[2], v.w[3]};
+    asm volatile("global_store_dwordx4 %0, %1, %2" ::"v"(off), "v"(d), "s"(base_u) : "memory");
+  };
+  auto uniform_out = [](char* p) {
+    const uint64_t v = reinterpret_cast<uint64_t>(p);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+    return reinterpret_cast<char*>(((uint64_t)hi << 32) | lo);
+  };
+  const float4* w_scale4 = reinterpret_cast<const float4*>(prm.w_scale + (int64_t)expert * prm.N);  // N % 8 == 0: 16-byte pieces
+  const int64_t tile_row0 = m0 + wm * WM;
+  const int rows_left = (int)min((int64_t)WM, valid_end - tile_row0);  // valid rows of this wave; may be <= 0
+
+  if constexpr (MODE == kGrouped || MODE == kScatter) {
+    TO* y = static_cast<TO*>(prm.y);
+    const int64_t col0 = (int64_t)nt * BN + wn * WN;
+    const int cols_left = (int)min((int64_t)WN, (int64_t)prm.N - col0);
+    float4 cs[NI];  // the lane's 4 column scales of every column block
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const int c = j * 16 + 4 * lg;
+      cs[j] = c < cols_left ? w_scale4[(col0 + c) / 4] : float4{0.f, 0.f, 0.f, 0.f};
+    }
+    char* base = uniform_out(reinterpret_cast<char*>(y + tile_row0 * prm.N + col0));
+    const uint32_t row_pitch = (uint32_t)prm.N * (uint32_t)sizeof(TO);
+    uint32_t row_off = (uint32_t)lrow * row_pitch;
+    static_for<MI>([&](auto i) {
+      const int r = i * 16 + lrow;
+      const float rs = meta_f[wm * WM + r];
+      char* row_ptr = nullptr;
+      if constexpr (MODE == kScatter) {
+        const int out_row = meta_rows[wm * WM + r];
+        row_ptr = reinterpret_cast<char*>(y + (int64_t)(out_row < 0 ? 0 : out_row) * prm.N + col0);
+      }
+      static_for<NI / 2>([&](auto jp) {
+        const f32x4& p = acc[i][2 * jp];
+        const f32x4& q = acc[i][2 * jp + 1];
+        const float4 cp = cs[2 * jp], cq = cs[2 * jp + 1];
+        const vec16 v = gather8(pack_pair<TO>(p[0] * rs * cp.x, p[1] * rs * cp.y), pack_pair<TO>(p[2] * rs * cp.z, p[3] * rs * cp.w),
+                                pack_pair<TO>(q[0] * rs * cq.x, q[1] * rs * cq.y), pack_pair<TO>(q[2] * rs * cq.z, q[3] * rs * cq.w));
+        const int c = pair_col(2 * jp);
+        if (r < rows_left && c < cols_left) {
+          if constexpr (MODE == kScatter) store16(row_ptr + (uint32_t)c * (uint32_t)sizeof(TO), v);
+          else store_at(base, row_off + (uint32_t)c * (uint32_t)sizeof(TO), v);
+        }
+      });
+      row_off += 16u * row_pitch;
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  } else {  // kSwiglu: the first half of a wave's column blocks are up, the second half the gate of the same activation
+            // columns; only the activation is kept (inference)
+    TO* act = static_cast<TO*>(prm.aux);
+    const int64_t col0 = (int64_t)nt * (BN / 2) + wn * (WN / 2);  // the wave's first activation column
+    const int cols_left = (int)min((int64_t)(WN / 2), (int64_t)prm.I - col0);
+    constexpr int NH = NI / 2;
+    float4 cs_up[NH], cs_gate[NH];
+#pragma unroll
+    for (int j = 0; j < NH; ++j) {
+      const int c = j * 16 + 4 * lg;
+      const bool ok = c < cols_left;
+      cs_up[j] = ok ? w_scale4[(col0 + c) / 4] : float4{0.f, 0.f, 0.f, 0.f};
+      cs_gate[j] = ok ? w_scale4[(prm.I + col0 + c) / 4] : float4{0.f, 0.f, 0.f, 0.f};
+    }
+    char* base = uniform_out(reinterpret_cast<char*>(act + tile_row0 * prm.I + col0));
+    const uint32_t row_pitch = (uint32_t)prm.I * (uint32_t)sizeof(TO);
+    uint32_t row_off = (uint32_t)lrow * row_pitch;
+    static_for<MI>([&](auto i) {
+      const int r = i * 16 + lrow;
+      const float rs = meta_f[wm * WM + r];
+      static_for<NH / 2>([&](auto jp) {
+        uint32_t pk[2][2];
+#pragma unroll
+        for (int b = 0; b < 2; ++b) {
+          const f32x4& u = acc[i][2 * jp + b];
+          const f32x4& g = acc[i][2 * jp + b + NH];
+          const float su[4] = {cs_up[2 * jp + b].x, cs_up[2 * jp + b].y, cs_up[2 * jp + b].z, cs_up[2 * jp + b].w};
+          const float sg[4] = {cs_gate[2 * jp + b].x, cs_gate[2 * jp + b].y, cs_gate[2 * jp + b].z, cs_gate[2 * jp + b].w};
+          float a[4];
+#pragma unroll
+          for (int s = 0; s < 4; ++s) {
+            // rounded to the output type first, like a pre-activation tensor would be
+            const float up = Elem<TO>::up(Elem<TO>::down(u[s] * rs * su[s]));
+            const float gf = Elem<TO>::up(Elem<TO>::down(g[s] * rs * sg[s]));
+            a[s] = up * gf * sigmoid_fast(gf);
+          }
+          pk[b][0] = pack_pair<TO>(a[0], a[1]);
+          pk[b][1] = pack_pair<TO>(a[2], a[3]);
+        }
+        const vec16 v = gather8(pk[0][0], pk[0][1], pk[1][0], pk[1][1]);
+        const int c = pair_col(2 * jp);
+        if (r < rows_left && c < cols_left) store_at(base, row_off + (uint32_t)c * (uint32_t)sizeof(TO), v);
+      });
+      row_off += 16u * row_pitch;
+      __builtin_amdgcn_sched_barrier(0);
+    });
+  }
 }
 
 template <typename TO, int MODE>
@@ -492,6 +477,7 @@ extern "C" int ck_grouped_gemm_fp8(const void* a8, const float* a_scale, int32_t
   if (int rc = check_segments(seg, name)) return rc;
   CK_REQUIRE(seg->align == 256, "%s: fp8 tiles are 256 rows high; sort with align = 256", name);
   CK_REQUIRE(N >= 8 && N % 8 == 0, "%s: N=%d must be a positive multiple of 8", name, N);
+  CK_REQUIRE((reinterpret_cast<uintptr_t>(w_scale) & 15) == 0, "%s: w_scale must be 16-byte aligned", name);
   CK_REQUIRE(K >= 128 && K % 128 == 0, "%s: K=%d must be a positive multiple of 128", name, K);
   CK_REQUIRE(a_gather_div >= 0, "%s: a_gather_div=%d is negative", name, a_gather_div);
   CK_REQUIRE(epilogue == CK_EPI_GROUPED || epilogue == CK_EPI_SCATTER || epilogue == CK_EPI_SWIGLU,
@@ -520,9 +506,6 @@ extern "C" int ck_grouped_gemm_fp8(const void* a8, const float* a_scale, int32_t
   prm.aux = aux;
   prm.a_scale = a_scale;
   prm.w_scale = w_scale;
-#if (CK_ABLATE & 256)
-  if (const char* t = getenv("CK_TRACE_PTR")) prm.y_t = reinterpret_cast<void*>(strtoull(t, nullptr, 16));
-#endif
   int out_cols = N;
   if (epilogue == CK_EPI_SWIGLU) {
     CK_REQUIRE(N % 16 == 0 && aux != nullptr, "%s: the SwiGLU epilogue needs N = 2*I with I %% 8 == 0 and aux", name);
