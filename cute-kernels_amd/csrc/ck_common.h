@@ -138,6 +138,19 @@ __device__ inline float sigmoid_fast(float x) {
   return __builtin_amdgcn_rcpf(1.0f + __expf(-xc));  // v_rcp_f32: 1 ulp, one instruction (a rounded division is ten)
 }
 
+// tanh-approximated GELU, 0.5 x (1 + tanh(u)) with u = sqrt(2/pi) (x + 0.044715 x^3) (torch.nn.GELU("tanh"), the non-GLU
+// activation of the reference's layer test, tests/test_commons.py:85-86), written as x * sigmoid(2u); and its derivative
+// sigmoid(2u) + x * sigmoid(2u) (1 - sigmoid(2u)) * 2 du/dx
+__device__ inline float gelu_tanh_fast(float x) {
+  const float u2 = 1.5957691216057308f * (x + 0.044715f * x * x * x);
+  return x * sigmoid_fast(u2);
+}
+__device__ inline float gelu_tanh_grad_fast(float x) {
+  const float u2 = 1.5957691216057308f * (x + 0.044715f * x * x * x);
+  const float s = sigmoid_fast(u2);
+  return s + x * s * (1.f - s) * 1.5957691216057308f * (1.f + 0.134145f * x * x);
+}
+
 // fp32 tensors get the accurate form, 16-bit tensors the fast one
 template <typename T>
 __device__ inline float sigmoid_for(float x) {

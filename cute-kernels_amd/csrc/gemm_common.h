@@ -37,7 +37,8 @@ struct GemmParams {
   const void* aux_in;
   const float* a_scale;  // fp8 only: per-row dequantisation scale of a (indexed like the rows of a)
   const float* w_scale;  // fp8 only: per-output-channel scale of w, [E, N]
-  int act_kind;          // kSwiglu epilogue: CK_ACT_SWIGLU (up * gate * sigmoid(gate)) or CK_ACT_GLU (up * sigmoid(gate))
+  int act_kind;          // kSwiglu epilogue: CK_ACT_SWIGLU (up * gate * sigmoid(gate)) or CK_ACT_GLU (up * sigmoid(gate));
+                         // kGrouped epilogue with aux: CK_ACT_GELU_TANH (aux = gelu(y), second output)
   void* trace;           // measurement builds only: per-workgroup phase timestamps (8 x uint64 each), else NULL
 };
 

@@ -345,7 +345,7 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
 #ifndef CK_LOAD_MOD
 #define CK_LOAD_MOD ""
 #endif
-      asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, off" CK_LOAD_MOD ::"s"(lds_addr), "v"(src) : "m0");
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" CK_LOAD_MOD ::"s"(lds_addr), "v"(src) : "m0");
     };
     const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds_c;
     const uint32_t wave_a = __builtin_amdgcn_readfirstlane(lds_base + wave * A_LD * 1024);
@@ -581,6 +581,18 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
           });
         }
         sync_slab();
+        if (MODE == kGrouped && prm.aux != nullptr) {  // CK_ACT_GELU_TANH: the activation of the rounded output, to aux
+          T* act = static_cast<T*>(prm.aux);
+          stage_blocks([&](auto i, auto jj, auto q, auto sidx) {
+            return Elem<T>::down(gelu_tanh_fast(Elem<T>::up(Elem<T>::down(acc[i][pass * 2 + jj][4 * q + sidx]))));
+          });
+          sync_slab();
+          drain_rows([&](int r, int sc) -> T* {
+            const int64_t p = m0 + r, n = (int64_t)nt * BN + tile_col(sc, pass);
+            return (p < valid_end && n < prm.N) ? act + p * prm.N + n : nullptr;
+          });
+          sync_slab();
+        }
       });
     } else {  // kSwiglu: blocks j = 0, 1 are up, j = 2, 3 are gate of the same activation columns
       T* pre = static_cast<T*>(prm.y);
@@ -641,6 +653,7 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
   } else if constexpr (MODE == kGrouped || MODE == kScatter) {
     T* y = static_cast<T*>(prm.y);
     T* y_t = static_cast<T*>(prm.y_t);
+    T* act = MODE == kGrouped ? static_cast<T*>(prm.aux) : nullptr;  // CK_ACT_GELU_TANH: second output
     static_for<MI>([&](auto i) {
       static_for<4>([&](auto q) {
         const int64_t p_base = m0 + wm * WM + i * 32 + 8 * q + row_quad;
@@ -656,8 +669,12 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
             T v[4];
             static_for<4>([&](auto s) {
               v[s] = Elem<T>::down(acc[i][j][4 * q + s]);
-              if (out_row[s] >= 0) y[out_row[s] * prm.N + n] = v[s];
-              else v[s] = Elem<T>::down(0.f);
+              if (out_row[s] >= 0) {
+                y[out_row[s] * prm.N + n] = v[s];
+                if (act != nullptr) act[out_row[s] * prm.N + n] = Elem<T>::down(gelu_tanh_fast(Elem<T>::up(v[s])));
+              } else {
+                v[s] = Elem<T>::down(0.f);
+              }
             });
             if (MODE == kGrouped && y_t != nullptr) store4(y_t + n * prm.ld_t + p_base, v[0], v[1], v[2], v[3]);
           }
@@ -781,6 +798,13 @@ extern "C" int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* 
   if (epilogue == CK_EPI_GLU) {  // same tiles and outputs as the SwiGLU epilogue, another gate function
     act_kind = CK_ACT_GLU;
     epilogue = CK_EPI_SWIGLU;
+  } else if (epilogue == CK_EPI_GELU_TANH) {  // the grouped epilogue with the activation as a second output
+    CK_REQUIRE(aux != nullptr && y_t == nullptr, "%s: the GELU epilogue needs aux and takes no y_t", name);
+    CK_REQUIRE(aligned16(aux), "%s: aux must be 16-byte aligned", name);
+    act_kind = CK_ACT_GELU_TANH;
+    epilogue = CK_EPI_GROUPED;
+  } else if (epilogue == CK_EPI_GROUPED || epilogue == CK_EPI_SCATTER) {
+    aux = nullptr;  // no second output
   }
   CK_REQUIRE(epilogue >= CK_EPI_GROUPED && epilogue <= CK_EPI_SWIGLU_BWD, "%s: unknown epilogue %d", name, epilogue);
   if (seg->max_rows == 0) return CK_OK;

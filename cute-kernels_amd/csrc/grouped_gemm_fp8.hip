@@ -117,8 +117,10 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
     }
   }
 
+  // (one wait state between the scalar write of M0 and the load that reads it: the compiler inserts it for its own
+  // instructions and cannot see into the asm)
   auto dma16 = [&](const char* base, uint32_t off, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(off), "s"(base) : "m0");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(off), "s"(base) : "m0");
   };
   auto uniform_ptr = [](const char* p) {
     const uint64_t v = reinterpret_cast<uint64_t>(p);
@@ -250,7 +252,9 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
   auto pair_col = [&](int j) { return (j + (odd_group ? 1 : 0)) * 16 + 4 * (lg & ~1); };
   auto store_at = [&](char* base_u, uint32_t off, const vec16& v) {
     const u32x4_t d = {v.w[0], v.w[1], v.w[2], v.w[3]};
-    asm volatile("global_store_dwordx4 %0, %1, %2" ::"v"(off), "v"(d), "s"(base_u) : "memory");
+    // two wait states: a store of more than 8 bytes followed by a vector write to its data registers needs them, and the
+    // compiler cannot see into the asm to insert them
+    asm volatile("global_store_dwordx4 %0, %1, %2\n\ts_nop 1" ::"v"(off), "v"(d), "s"(base_u) : "memory");
   };
   auto uniform_out = [](char* p) {
     const uint64_t v = reinterpret_cast<uint64_t>(p);

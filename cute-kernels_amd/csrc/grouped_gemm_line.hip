@@ -212,8 +212,10 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
 
   // One 1 KiB wave-load: scalar base (the operand at this K step, uniform over the wave) + the lane's 32-bit byte offset,
   // so that a load costs no vector arithmetic (a 64-bit vector add per load delayed the MFMA behind it)
+  // (one wait state between the scalar write of M0 and the load that reads it: the compiler inserts it for its own
+  // instructions and cannot see into the asm)
   auto dma16 = [&](const char* base, uint32_t off, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(off), "s"(base) : "m0");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" ::"s"(lds_addr), "v"(off), "s"(base) : "m0");
   };
   auto uniform_ptr = [](const char* p) {
     const uint64_t v = reinterpret_cast<uint64_t>(p);
@@ -490,8 +492,10 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   // arithmetic; `inside`: the wave's whole tile lies inside the matrix and nothing is tested per store.
   auto store_at = [&](char* base_u, uint32_t off, const vec16& v) {
     const u32x4_t d = {v.w[0], v.w[1], v.w[2], v.w[3]};
-    if constexpr ((CK_ABLATE & 256) != 0) asm volatile("global_store_dwordx4 %0, %1, %2 nt" ::"v"(off), "v"(d), "s"(base_u) : "memory");
-    else asm volatile("global_store_dwordx4 %0, %1, %2" ::"v"(off), "v"(d), "s"(base_u) : "memory");
+    // The two wait states behind the store are the hardware's rule for a store of more than 8 bytes whose data registers
+    // the next vector instruction overwrites; the compiler inserts them for its own stores and cannot see into this one.
+    if constexpr ((CK_ABLATE & 256) != 0) asm volatile("global_store_dwordx4 %0, %1, %2 nt\n\ts_nop 1" ::"v"(off), "v"(d), "s"(base_u) : "memory");
+    else asm volatile("global_store_dwordx4 %0, %1, %2\n\ts_nop 1" ::"v"(off), "v"(d), "s"(base_u) : "memory");
   };
   auto store_lines_at = [&](const vec16& v1, const vec16& v2, int j, char* base_u, uint32_t row_off, bool inside, bool row_in,
                             int cols_left) {
@@ -580,6 +584,20 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
       });
     }
     char* base = uniform_out(reinterpret_cast<char*>(y + tile_row0 * prm.N + col0));
+    // second output of the grouped epilogue (aux, same shape as y): the tanh-approximated GELU of the 8 rounded outputs
+    char* act_base = nullptr;
+    if constexpr (MODE == kGrouped && EXTRA && !BT) {
+      if (prm.aux != nullptr) act_base = uniform_out(reinterpret_cast<char*>(static_cast<T*>(prm.aux) + tile_row0 * prm.N + col0));
+    }
+    auto gelu8 = [&](const vec16& v) {
+      Pack16<T> in;
+      in.v = v;
+      vec16 o;
+#pragma unroll
+      for (int w = 0; w < 4; ++w)
+        o.w[w] = pack_pair<T>(gelu_tanh_fast(Elem<T>::up(in.e[2 * w])), gelu_tanh_fast(Elem<T>::up(in.e[2 * w + 1])));
+      return o;
+    };
     const uint32_t row_pitch = (uint32_t)prm.N * 2u;
     const bool inside = rows_left >= WM && cols_left >= WN;
     uint32_t row_off = (uint32_t)lrow * row_pitch;
@@ -596,6 +614,9 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
                       [&](int c) { return c < cols_left; });
         } else {
           store_lines_at(v1, v2, 4 * jq, base, row_off, inside, i * 16 + lrow < rows_left, cols_left);
+          if constexpr (EXTRA && !BT) if (act_base != nullptr) {  // CK_ACT_GELU_TANH: the activation of the rounded output
+            store_lines_at(gelu8(v1), gelu8(v2), 4 * jq, act_base, row_off, inside, i * 16 + lrow < rows_left, cols_left);
+          }
         }
       });
       row_off += 16u * row_pitch;
@@ -689,7 +710,8 @@ int launch_extra(const GemmParams& prm, unsigned blocks, hipStream_t s, const ch
 template <typename T, int MODE, int BN, bool BT, int WGM>
 int launch_mode(const GemmParams& prm, unsigned blocks, hipStream_t s, const char* name) {
   if constexpr (!BT && MODE != kDw) {
-    if (prm.aux_in != nullptr || prm.y_t != nullptr) return launch_extra<T, MODE, BN, BT, WGM, true>(prm, blocks, s, name);
+    if (prm.aux_in != nullptr || prm.y_t != nullptr || (MODE == kGrouped && prm.aux != nullptr))
+      return launch_extra<T, MODE, BN, BT, WGM, true>(prm, blocks, s, name);
   }
   return launch_extra<T, MODE, BN, BT, WGM, false>(prm, blocks, s, name);
 }

@@ -128,6 +128,21 @@ inline Shape shape_for(int64_t rows, int64_t chunks_per_row) {
   return s;
 }
 
+// d_pre = d_act * gelu'(pre) for the tanh-approximated GELU, over a flat range: the backward of the activation that the
+// grouped GEMM's CK_EPI_GELU_TANH epilogue applies
+template <typename T, int P>
+__global__ __launch_bounds__(kBlock) void gelu_tanh_bwd_kernel(const T* __restrict__ pre, const T* __restrict__ d_act,
+                                                                T* __restrict__ d_pre, int64_t chunks) {
+  for (int64_t ch = (int64_t)blockIdx.x * kBlock + threadIdx.x; ch < chunks; ch += (int64_t)gridDim.x * kBlock) {
+    const Chunk<T, P> x = Chunk<T, P>::load(pre + ch * P);
+    const Chunk<T, P> g = Chunk<T, P>::load(d_act + ch * P);
+    Chunk<T, P> o;
+#pragma unroll
+    for (int i = 0; i < P; ++i) o.e[i] = Elem<T>::down(Elem<T>::up(g.e[i]) * gelu_tanh_grad_fast(Elem<T>::up(x.e[i])));
+    o.store(d_pre + ch * P);
+  }
+}
+
 }  // namespace
 }  // namespace ck
 
@@ -198,5 +213,29 @@ extern "C" int ck_swiglu_bwd(const void* gate, int64_t gate_stride, const void* 
     }
   });
   CK_CHECK_LAUNCH("ck_swiglu_bwd");
+  return CK_OK;
+}
+
+extern "C" int ck_gelu_tanh_bwd(const void* pre, const void* d_act, void* d_pre, int64_t n, int32_t dtype, void* stream) {
+  CK_REQUIRE(n >= 0, "ck_gelu_tanh_bwd: negative size");
+  if (n == 0) return CK_OK;
+  CK_REQUIRE(pre && d_act && d_pre, "ck_gelu_tanh_bwd: NULL argument");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  CK_DISPATCH_HALF(dtype, "ck_gelu_tanh_bwd", {
+    constexpr int P = Elem<scalar_t>::per16;
+    const scalar_t* x = static_cast<const scalar_t*>(pre);
+    const scalar_t* g = static_cast<const scalar_t*>(d_act);
+    scalar_t* o = static_cast<scalar_t*>(d_pre);
+    const bool vec = ((reinterpret_cast<uintptr_t>(pre) | reinterpret_cast<uintptr_t>(d_act) | reinterpret_cast<uintptr_t>(d_pre)) & 15) == 0;
+    const int64_t done = vec ? n / P * P : 0;
+    auto grid_for = [](int64_t chunks) {
+      const int64_t blocks = (chunks + kBlock - 1) / kBlock;
+      return dim3((unsigned)(blocks < 256 * 16 ? blocks : 256 * 16));
+    };
+    if (done > 0) hipLaunchKernelGGL((gelu_tanh_bwd_kernel<scalar_t, P>), grid_for(done / P), dim3(kBlock), 0, s, x, g, o, done / P);
+    if (done < n)
+      hipLaunchKernelGGL((gelu_tanh_bwd_kernel<scalar_t, 1>), grid_for(n - done), dim3(kBlock), 0, s, x + done, g + done, o + done, n - done);
+  });
+  CK_CHECK_LAUNCH("ck_gelu_tanh_bwd");
   return CK_OK;
 }

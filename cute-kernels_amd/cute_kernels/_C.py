@@ -24,7 +24,8 @@ if os.environ.get("CK_MI355_LIB"):
 CK_F32, CK_F16, CK_BF16 = 0, 1, 2
 CK_EPI_GROUPED, CK_EPI_SCATTER, CK_EPI_SWIGLU, CK_EPI_SWIGLU_BWD = 0, 1, 2, 3
 CK_EPI_GLU = 5
-CK_ACT_SWIGLU, CK_ACT_GLU = 0, 1
+CK_EPI_GELU_TANH = 6
+CK_ACT_SWIGLU, CK_ACT_GLU, CK_ACT_GELU_TANH = 0, 1, 2
 
 _DTYPE_CODES = {torch.float32: CK_F32, torch.float16: CK_F16, torch.bfloat16: CK_BF16}
 
@@ -78,6 +79,11 @@ _SIGNATURES = {
         [c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_int32, c_int32, POINTER(ck_segments), c_int32, c_void_p, c_void_p, c_int32, c_void_p],
     ),
     "ck_swiglu_fwd": (c_int32, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int32, c_void_p]),
+    "ck_rmsnorm_route": (
+        c_int32,
+        [c_void_p, c_void_p, c_void_p, c_float, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_void_p],
+    ),
+    "ck_gelu_tanh_bwd": (c_int32, [c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_void_p]),
     "ck_swiglu_bwd": (
         c_int32,
         [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_int64, c_int64, c_int64, c_int32, c_void_p],

@@ -1,8 +1,9 @@
 """MI355X-native implementation of the MoE hot path of cute-kernels, under the reference's Python API.
 
 Exports mirror the names the reference exposes for this path (cute_kernels/__init__.py:15-58 of the reference):
-the MoE layer, continuous_count_cute, swiglu_cute / swiglu_packed_cute, rmsnorm_cute. Everything runs through the
-ahead-of-time built libck_mi355.so; there is no other backend and no CPU path.
+the MoE layer, continuous_count_cute, swiglu_cute / swiglu_packed_cute, rmsnorm_cute. Every `*_cute` name and the MoE layer
+run through the ahead-of-time built libck_mi355.so; there is no other backend and no CPU path for them. The `*_torch`
+names are eager PyTorch statements of the same operators (torch_ops.py), kept for import compatibility.
 """
 
 from .fp8 import MoE_E4M3, quantize_expert_weights_e4m3, quantize_rows_e4m3, swiglu_experts_e4m3
@@ -10,6 +11,7 @@ from .continuous_count import continuous_count_and_offsets_cute, continuous_coun
 from .modules import Experts, MoE, MoE_Triton
 from .fused_residual_add_rmsnorm import fused_residual_add_rmsnorm_cute
 from .rmsnorm import rmsnorm_cute
+from .rmsnorm_route import rmsnorm_route_cute
 from .scattermoe import (
     ExpertSegments,
     experts_down,
@@ -23,6 +25,15 @@ from .scattermoe import (
 from .softmax import softmax_cute
 from .router_stats import load_balancing_loss, load_balancing_stats
 from .swiglu import swiglu_cute, swiglu_packed_cute
+from .torch_ops import (
+    MoE_Torch,
+    continuous_count_torch,
+    fused_residual_add_rmsnorm_torch,
+    rmsnorm_torch,
+    softmax_torch,
+    swiglu_packed_torch,
+    swiglu_torch,
+)
 from .utils import (
     KernelBackend,
     ceil_divide,

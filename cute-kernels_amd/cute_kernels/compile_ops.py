@@ -470,7 +470,7 @@ def experts_up_backward(
     ctx = _Ctx((need_x, need_w, False, False, need_bias))
     ctx.seg, ctx.k = _segments(seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, align), k
     ctx.saved_tensors = (x.contiguous(), w.contiguous())
-    d_x, d_w, _, _, d_bias = _moe._ExpertsUp.backward(ctx, d_y)
+    d_x, d_w, _, _, d_bias = _moe._ExpertsUp.backward(ctx, d_y)[:5]
     return _or_empty(d_x, x), _or_empty(d_w, x), _or_empty(d_bias, x)
 
 
@@ -497,6 +497,60 @@ def _experts_up_bwd(ctx, d_y):
 
 
 experts_up.register_autograd(_experts_up_bwd, setup_context=_experts_up_setup)
+
+
+@custom_op(f"{NS}::experts_up_gelu", mutates_args=())
+def experts_up_gelu(
+    x: Tensor, w: Tensor, bias: Optional[Tensor], seg_starts: Tensor, counts: Tensor, tile_expert: Tensor, row_slot: Tensor,
+    max_rows: int, num_experts: int, align: int, k: int,
+) -> tuple[Tensor, Tensor]:
+    """(gelu_tanh(y) [max_rows, N], y [max_rows, N]): the c_fc GEMM with the activation in its epilogue"""
+    ctx = _Ctx()
+    seg = _segments(seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, align)
+    act = _moe._ExpertsUp.forward(ctx, x, w, seg, k, bias, True)
+    return act, ctx.saved_tensors[2]
+
+
+@experts_up_gelu.register_fake
+def _(x, w, bias, seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, align, k):
+    return x.new_empty(max_rows, w.shape[1]), x.new_empty(max_rows, w.shape[1])
+
+
+@custom_op(f"{NS}::experts_up_gelu_backward", mutates_args=())
+def experts_up_gelu_backward(
+    d_act: Tensor, pre: Tensor, x: Tensor, w: Tensor, seg_starts: Tensor, counts: Tensor, tile_expert: Tensor,
+    row_slot: Tensor, max_rows: int, num_experts: int, align: int, k: int, need_x: bool, need_w: bool, need_bias: bool,
+) -> tuple[Tensor, Tensor, Tensor]:
+    ctx = _Ctx((need_x, need_w, False, False, need_bias, False))
+    ctx.seg, ctx.k, ctx.gelu = _segments(seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, align), k, True
+    ctx.saved_tensors = (x.contiguous(), w.contiguous(), pre)
+    d_x, d_w, _, _, d_bias, _ = _moe._ExpertsUp.backward(ctx, d_act)
+    return _or_empty(d_x, x), _or_empty(d_w, x), _or_empty(d_bias, x)
+
+
+@experts_up_gelu_backward.register_fake
+def _(d_act, pre, x, w, seg_starts, counts, tile_expert, row_slot, max_rows, num_experts, align, k, need_x, need_w, need_bias):
+    e = x.new_empty(0)
+    return (
+        torch.empty_like(x) if need_x else e,
+        torch.empty_like(w) if need_w else e,
+        x.new_empty(num_experts, w.shape[1]) if need_bias else e,
+    )
+
+
+def _experts_up_gelu_setup(ctx, inputs, output):
+    x, w, _bias, seg_starts, counts, tile_expert, row_slot, *rest = inputs
+    ctx.save_for_backward(output[1], x, w, seg_starts, counts, tile_expert, row_slot)
+    ctx.rest = tuple(rest)
+
+
+def _experts_up_gelu_bwd(ctx, d_act, _d_pre):
+    need_x, need_w, need_bias = ctx.needs_input_grad[:3]
+    d_x, d_w, d_bias = experts_up_gelu_backward(d_act.contiguous(), *ctx.saved_tensors, *ctx.rest, need_x, need_w, need_bias)
+    return (d_x if need_x else None), (d_w if need_w else None), (d_bias if need_bias else None), *(None,) * 8
+
+
+experts_up_gelu.register_autograd(_experts_up_gelu_bwd, setup_context=_experts_up_gelu_setup)
 
 
 @custom_op(f"{NS}::experts_down", mutates_args=())

@@ -75,17 +75,19 @@ def swiglu_experts_e4m3(
     w_proj_scale: torch.Tensor,
     gates: torch.Tensor,
     seg: ExpertSegments,
+    x_quantized: tuple[torch.Tensor, torch.Tensor] | None = None,
 ) -> torch.Tensor:
     """out[t] = sum_j gates[t, j] * c_proj_e( swiglu_packed( c_fc_e( x[t] ) ) ) with e4m3 GEMM operands.
 
     x [T, H] bf16 / fp16; w_fc8 [E, 2I, H] packed [up | gate]; w_proj8 [E, H, I]; seg from sort_by_expert(..., align=256).
+    x_quantized: (x8, scale) = quantize_rows_e4m3(x) if the caller has it already (rmsnorm_route_cute(..., quantize=True)).
     """
     assert seg.align == 256, "the fp8 GEMMs use 256-row tiles: sort_by_expert(..., align=256)"
     T, H = x.shape
     k = gates.size(1)
     E, two_i, _ = w_fc8.shape
     I = two_i // 2
-    x8, x_scale = quantize_rows_e4m3(x)  # per token
+    x8, x_scale = quantize_rows_e4m3(x) if x_quantized is None else x_quantized  # per token
     act = torch.empty(seg.max_rows, I, dtype=x.dtype, device=x.device)  # pad rows: never written, quantised, never used
     _gemm_fp8(x8, x_scale, k, w_fc8, w_fc_scale, seg, _C.CK_EPI_SWIGLU, None, act, x.dtype)
     act8, act_scale = quantize_rows_e4m3(act)  # per routed row
@@ -127,5 +129,25 @@ class MoE_E4M3(nn.Module):
         out = swiglu_experts_e4m3(
             hidden_states, self.c_fc_weight_e4m3, self.c_fc_scale, self.c_proj_weight_e4m3, self.c_proj_scale,
             router_weights, seg,
+        )
+        return out.view(original_shape), router_logits
+
+    @torch.no_grad()
+    def forward_with_norm(
+        self, hidden_states: torch.Tensor, norm_weight: torch.Tensor | None, eps: float | None
+    ) -> tuple[torch.Tensor, torch.Tensor]:
+        """forward(rmsnorm_cute(hidden_states, norm_weight, eps)) with one kernel ahead of the router that reads
+        hidden_states once and writes the normalised rows, the router logits and the e4m3 rows with their scales."""
+        from .rmsnorm_route import rmsnorm_route_cute
+
+        original_shape = hidden_states.shape
+        normed, router_logits, x8, x_scale = rmsnorm_route_cute(
+            hidden_states.view(-1, self.hidden_size), norm_weight, self.gate.weight, eps, quantize=True
+        )
+        router_weights, selected_experts = route_topk_softmax(router_logits, self.top_k, long_indices=False)
+        seg = sort_by_expert(selected_experts, self.num_experts, 256)
+        out = swiglu_experts_e4m3(
+            normed, self.c_fc_weight_e4m3, self.c_fc_scale, self.c_proj_weight_e4m3, self.c_proj_scale, router_weights, seg,
+            x_quantized=(x8, x_scale),
         )
         return out.view(original_shape), router_logits

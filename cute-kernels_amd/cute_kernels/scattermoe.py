@@ -251,6 +251,8 @@ _EPILOGUE_NAMES = {
     _C.CK_EPI_SCATTER: "grouped_gemm<scatter>",
     _C.CK_EPI_SWIGLU: "grouped_gemm<swiglu>",
     _C.CK_EPI_SWIGLU_BWD: "grouped_gemm<swiglu_bwd>",
+    _C.CK_EPI_GLU: "grouped_gemm<swiglu>",
+    _C.CK_EPI_GELU_TANH: "grouped_gemm<grouped>",
 }
 
 
@@ -478,29 +480,43 @@ def _check_expert_dtypes(x: torch.Tensor, *weights: torch.Tensor) -> None:
 # generic expert linears (any activation between them)
 # ---------------------------------------------------------------------------------------------------------------
 class _ExpertsUp(torch.autograd.Function):
-    """x [T, H] (token order) -> y [max_rows, N] (padded grouped): the reference's c_fc with grouped_out=True."""
+    """x [T, H] (token order) -> y [max_rows, N] (padded grouped): the reference's c_fc with grouped_out=True.
+    gelu=True: returns gelu_tanh(y) instead, computed in the GEMM's epilogue from the rounded y (the activation module
+    applied to y would read the same values); y is kept for the backward pass only."""
 
     @staticmethod
-    def forward(ctx, x, w, seg: ExpertSegments, k: int, bias=None):
+    def forward(ctx, x, w, seg: ExpertSegments, k: int, bias=None, gelu: bool = False):
         x = x.contiguous()
         w = w.contiguous()
         E, N, K = w.shape
         # pad rows are never written by the kernel; zeros keep any activation applied on top finite
         y = torch.zeros(seg.max_rows, N, dtype=x.dtype, device=x.device)
-        fused_bias = bias is not None and _bias_in_epilogue(seg, K)
-        _gemm(x, k, w, seg, _C.CK_EPI_GROUPED, y, aux_in=bias.contiguous() if fused_bias else None)
+        act = torch.zeros_like(y) if gelu else None
+        fused_bias = bias is not None and (gelu or _bias_in_epilogue(seg, K))
+        _gemm(x, k, w, seg, _C.CK_EPI_GELU_TANH if gelu else _C.CK_EPI_GROUPED, y, aux=act,
+              aux_in=bias.contiguous() if fused_bias else None)
         if bias is not None and not fused_bias:
             _add_expert_bias(y, bias.contiguous(), seg, None)
-        ctx.save_for_backward(x, w)
+        ctx.gelu = gelu
+        if gelu:
+            ctx.save_for_backward(x, w, y)
+        else:
+            ctx.save_for_backward(x, w)
         ctx.seg, ctx.k = seg, k
-        return y
+        return act if gelu else y
 
     @staticmethod
     def backward(ctx, d_y):
-        x, w = ctx.saved_tensors
+        x, w = ctx.saved_tensors[:2]
         seg, k = ctx.seg, ctx.k
         T, K = x.shape
         d_y = d_y.contiguous()
+        if getattr(ctx, "gelu", False):  # d_y arrives as d_act: through the activation first
+            pre, d_act = ctx.saved_tensors[2], d_y
+            d_y = torch.empty_like(d_act)
+            with torch.cuda.device(d_act.device):
+                _C.check(_C.lib().ck_gelu_tanh_bwd(_C.ptr(pre), _C.ptr(d_act), _C.ptr(d_y), d_act.numel(),
+                                                   _C.dtype_code(d_act.dtype), _C.stream()))
         d_x = d_w = d_bias = None
         if len(ctx.needs_input_grad) > 4 and ctx.needs_input_grad[4]:
             d_bias = _expert_bias_grad(d_y, seg)
@@ -517,7 +533,7 @@ class _ExpertsUp(torch.autograd.Function):
             d_expanded = torch.empty(T * k, K, dtype=x.dtype, device=x.device)
             _gemm_dx(d_y, w, seg, _C.CK_EPI_SCATTER, d_expanded)
             d_x = d_expanded if k == 1 else _combine(d_expanded, None, T, k, K)[0]
-        return d_x, d_w, None, None, d_bias
+        return d_x, d_w, None, None, d_bias, None
 
 
 class _ExpertsDown(torch.autograd.Function):
@@ -570,18 +586,22 @@ class _ExpertsDown(torch.autograd.Function):
 
 
 def experts_up(
-    x: torch.Tensor, weight: torch.Tensor, seg: ExpertSegments, k: int, bias: torch.Tensor | None = None
+    x: torch.Tensor, weight: torch.Tensor, seg: ExpertSegments, k: int, bias: torch.Tensor | None = None,
+    gelu_tanh: bool = False,
 ) -> torch.Tensor:
-    """x [T, H] -> c_fc output in padded grouped order [max_rows, N] (+ bias[e] on expert e's rows)."""
+    """x [T, H] -> c_fc output in padded grouped order [max_rows, N] (+ bias[e] on expert e's rows); with gelu_tanh, the
+    tanh-approximated GELU of that output, applied in the GEMM's epilogue."""
     _check_expert_dtypes(x, weight)
     assert bias is None or (bias.dtype == x.dtype and bias.shape == weight.shape[:2]), "bias should be [E, out] in x.dtype"
     if is_tracing():
-        return _ops.experts_up(
+        op = _ops.experts_up_gelu if gelu_tanh else _ops.experts_up
+        out = op(
             x, weight, bias, seg.seg_starts, seg.counts, seg.tile_expert, seg.row_slot, seg.max_rows, seg.num_experts,
             seg.align, k,
         )
+        return out[0] if gelu_tanh else out
     _C.require_gpu(x, weight, bias)
-    return _ExpertsUp.apply(x, weight, seg, k, bias)
+    return _ExpertsUp.apply(x, weight, seg, k, bias, gelu_tanh)
 
 
 def experts_down(

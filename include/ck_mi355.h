@@ -172,6 +172,9 @@ typedef struct ck_segments {
  *   CK_EPI_SCATTER        : y [R, N]: valid row p is written to row row_slot[p] (back to (token, slot) order)
  *                           both: aux_in, if not NULL, is a bias [E, N] whose row e joins the fp32 accumulators of expert
  *                           e's rows before the one rounding (F.linear with a bias, torch_implementation.py:42)
+ *   CK_EPI_GELU_TANH      : as CK_EPI_GROUPED (bias included), and aux [max_rows, N] = tanh-approximated GELU of y, computed
+ *                           from the rounded y as the activation module applied to y would (torch.nn.GELU("tanh"), the
+ *                           non-GLU activation of the reference's layer test, tests/test_commons.py:85-86); no y_t
  *   CK_EPI_SWIGLU         : N = 2*I packed [up | gate] (cute_kernels/kernels/swiglu/__init__.py:121): writes the
  *                           pre-activation to y [max_rows, 2I], act = up*silu(gate) (computed from the rounded
  *                           pre-activation, as the unfused path would) to aux [max_rows, I], and act^T to
@@ -185,8 +188,10 @@ typedef struct ck_segments {
 #define CK_EPI_SWIGLU 2
 #define CK_EPI_SWIGLU_BWD 3
 #define CK_EPI_GLU 5 /* as CK_EPI_SWIGLU with act = up * sigmoid(gate): torch.nn.GLU() on the packed c_fc output */
+#define CK_EPI_GELU_TANH 6
 #define CK_ACT_SWIGLU 0
 #define CK_ACT_GLU 1
+#define CK_ACT_GELU_TANH 2
 int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* w, int32_t N, int32_t K,
                     const ck_segments* seg, int32_t epilogue, void* y, void* y_t, int64_t ld_t, void* aux,
                     const void* aux_in, int32_t dtype, void* stream);
@@ -247,6 +252,9 @@ int ck_swiglu_fwd(const void* gate, int64_t gate_stride, const void* up, int64_t
 int ck_swiglu_bwd(const void* gate, int64_t gate_stride, const void* up, int64_t up_stride, const void* d_out,
                   int64_t d_out_stride, void* d_gate, int64_t d_gate_stride, void* d_up, int64_t d_up_stride,
                   int64_t rows, int64_t cols, int32_t dtype, void* stream);
+/* Backward of the activation of CK_EPI_GELU_TANH: d_pre[i] = d_act[i] * gelu_tanh'(pre[i]) over n contiguous elements
+ * (what autograd derives for torch.nn.GELU("tanh"), the activation of tests/test_commons.py:85-86). bf16 / f16. */
+int ck_gelu_tanh_bwd(const void* pre, const void* d_act, void* d_pre, int64_t n, int32_t dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------------------------------
  * (d) RMSNorm
@@ -263,6 +271,19 @@ int ck_rmsnorm_fwd(const void* x, const void* weight, float eps, int64_t B, int3
 int64_t ck_rmsnorm_bwd_partial_rows(int64_t B);
 int ck_rmsnorm_bwd(const void* x, const void* weight, const void* d_out, const float* rstd, float eps, int64_t B,
                    int32_t H, void* d_x, float* d_weight_partial, float* d_weight, int32_t dtype, void* stream);
+
+/* RMSNorm fused ahead of the router: one pass over x that writes y = rmsnorm(x) (as ck_rmsnorm_fwd), rstd, and the router
+ * logits y @ gate_weight^T computed from the 16-bit y while the rows are in registers (fp32 accumulation, rounded to the
+ * rows' dtype); with x8 / scale8, also the e4m3 rows and per-row scales that ck_quant_rows_e4m3 would derive from y.
+ * Replaces, as one kernel: rmsnorm_forward_triton -- cute_kernels/kernels/rmsnorm/triton_implementation/forward.py:14-53 --
+ *           and the router's linear layer, self.gate(hidden_states) -- cute_kernels/kernels/scattermoe/
+ *           torch_implementation.py:122-124 (and the per-row quantiser ahead of ck_grouped_gemm_fp8).
+ * x, y [B, H]; norm_weight [H] or NULL; gate_weight [E, H]; logits [B, E]; rstd [B] fp32 or NULL; x8 [B, H] bytes and
+ * scale8 [B] fp32, both or neither; gate_packed: workspace of 16 * ceil(E / 16) * H elements of the rows' dtype, written by
+ * the call (the gate weight in the order the kernel's lanes read it). bf16 / f16. Needs H % 512 == 0, H <= 4096, E <= 128. */
+int ck_rmsnorm_route(const void* x, const void* norm_weight, const void* gate_weight, float eps, int64_t B, int32_t H,
+                     int32_t E, void* y, float* rstd, void* logits, void* x8, float* scale8, void* gate_packed,
+                     int32_t dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------------------------------
  * Expert biases

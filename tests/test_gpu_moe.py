@@ -94,6 +94,54 @@ def test_grouped_gemm_grouped_in_scatter_out(device, dtype, align, K, N, gemm_ti
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("with_bias", [False, True])
+@pytest.mark.parametrize("align,K,N", [(128, 200, 136), (256, 64, 128), (256, 576, 264), (256, 192, 840)])
+def test_grouped_gemm_gelu_tanh_epilogue(device, dtype, align, K, N, with_bias, gemm_tile):
+    """CK_EPI_GELU_TANH: y as the grouped epilogue writes it (bias in the accumulators), and aux = the tanh GELU of the
+    rounded y -- against torch's F.gelu(approximate="tanh") (the reference test's activation module, test_commons.py:85-86)
+    applied to the kernel's own y (within one rounding step of the 16-bit type) and to the fp32 reference."""
+    T, k, E = 300, 2, 5
+    g, seg = _make_case(device, dtype, T, k, E, align, seed=3)
+    x = torch.randn(T, K, generator=g).to(dtype)
+    w = (0.1 * torch.randn(E, N, K, generator=g)).to(dtype)
+    bias = torch.randn(E, N, generator=g).to(dtype) if with_bias else None
+    y = torch.zeros(seg.max_rows, N, dtype=dtype, device=device)
+    act = torch.full((seg.max_rows, N), 9.0, dtype=dtype, device=device)
+    scattermoe._gemm(x.to(device), k, w.to(device), seg, _C.CK_EPI_GELU_TANH, y, aux=act,
+                     aux_in=bias.to(device) if with_bias else None)
+    expect = _expected_grouped(lambda p, slot: x[slot // k], w, seg, N)
+    seg_starts, counts, _ = _layout(seg)
+    valid = torch.zeros(seg.max_rows, dtype=torch.bool)
+    for e in range(E):
+        s, c = int(seg_starts[e]), int(counts[e])
+        valid[s : s + c] = True
+        if with_bias:
+            expect[s : s + c] += bias[e].float()
+    y_c, act_c = y.float().cpu(), act.float().cpu()
+    torch.testing.assert_close(y_c[valid], expect[valid], rtol=RTOL, atol=ATOL)
+    torch.testing.assert_close(act_c[valid], F.gelu(expect[valid], approximate="tanh"), rtol=RTOL, atol=ATOL)
+    # from the rounded y, like the module applied to y: at most one rounding step of the output type apart
+    eps = 2.0**-8 if dtype == torch.bfloat16 else 2.0**-11
+    same_input = F.gelu(y.cpu()[valid].float(), approximate="tanh")
+    assert float(((act_c[valid] - same_input).abs() / (same_input.abs() + 1e-3)).max()) <= 2 * eps
+    assert torch.all(act_c[~valid] == 9.0)  # pad rows are not written
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("n", [8 * 1000, 12345])
+def test_gelu_tanh_backward_kernel(device, dtype, n):
+    g = torch.Generator().manual_seed(n)
+    pre = (2.5 * torch.randn(n, generator=g)).to(dtype)
+    d_act = torch.randn(n, generator=g).to(dtype)
+    out = torch.empty(n, dtype=dtype, device=device)
+    pre_d, d_act_d = pre.to(device), d_act.to(device)
+    _C.check(_C.lib().ck_gelu_tanh_bwd(_C.ptr(pre_d), _C.ptr(d_act_d), _C.ptr(out), n, _C.dtype_code(dtype), _C.stream()))
+    p64 = pre.double().requires_grad_()
+    F.gelu(p64, approximate="tanh").backward(d_act.double())
+    torch.testing.assert_close(out.cpu().double(), p64.grad, rtol=RTOL, atol=ATOL)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("epilogue", ["grouped", "scatter"])
 @pytest.mark.parametrize("n_out,n_in", [(64, 128), (192, 264), (576, 840), (128, 8)])
 def test_grouped_gemm_input_gradient_form(device, dtype, epilogue, n_out, n_in):
@@ -539,19 +587,22 @@ def test_moe_layer_at_full_baseline_shapes(device, name, T, E, k, H, I, skew, no
     )
 
 
-@pytest.mark.parametrize("act,kind", [("swiglu", _C.CK_ACT_SWIGLU), ("glu", _C.CK_ACT_GLU), ("gelu", None)])
-def test_gated_activations_take_the_fused_expert_block(device, monkeypatch, act, kind):
-    """Packed SwiGLU and torch.nn.GLU run inside the c_fc epilogue (swiglu_experts with the matching act_kind); any other
-    callable goes GEMM -> callable -> GEMM. Results of both routes are covered by the layer parity tests above."""
+@pytest.mark.parametrize("act,kind", [("swiglu", _C.CK_ACT_SWIGLU), ("glu", _C.CK_ACT_GLU), ("gelu", None), ("silu", None)])
+def test_known_activations_run_in_the_c_fc_epilogue(device, monkeypatch, act, kind):
+    """Packed SwiGLU and torch.nn.GLU run inside the c_fc epilogue (swiglu_experts with the matching act_kind), and so does
+    nn.GELU("tanh") (experts_up with gelu_tanh=True); any other callable goes GEMM -> callable -> GEMM. Results of all
+    routes are covered by the layer parity tests above."""
     from cute_kernels.modules import moe as moe_module
 
-    act_gpu, _, is_glu = _acts(act)
+    act_gpu, is_glu = (nn.SiLU(), False) if act == "silu" else (_acts(act)[0], _acts(act)[2])
     layer = cute_kernels.MoE(4, 2, 128, 256, act_gpu, is_glu, False, 0.02).to(torch.bfloat16).to(device)
-    seen = []
-    real = moe_module.swiglu_experts
+    seen, seen_up = [], []
+    real, real_up = moe_module.swiglu_experts, moe_module.experts_up
     monkeypatch.setattr(moe_module, "swiglu_experts", lambda *a: (seen.append(a[5]), real(*a))[1])
+    monkeypatch.setattr(moe_module, "experts_up", lambda *a, **kw: (seen_up.append(kw.get("gelu_tanh", False)), real_up(*a, **kw))[1])
     layer(torch.randn(300, 128, device=device, dtype=torch.bfloat16))
     assert seen == ([kind] if kind is not None else [])
+    assert seen_up == ({"gelu": [True], "silu": [False]}.get(act, []))
 
 
 def test_bias_in_the_gemm_epilogue_equals_the_separate_bias_kernel(device, monkeypatch):
