@@ -222,6 +222,7 @@ __global__ __launch_bounds__(kBlock) void group_rows_stream_kernel(
     const T* __restrict__ src, const T* __restrict__ coeff, int fan_out, const int32_t* __restrict__ row_slot,
     const int32_t* __restrict__ seg_starts, const uint32_t* __restrict__ counts, const int32_t* __restrict__ tile_expert,
     int align, int64_t max_rows, int chunks_per_row, T* __restrict__ grouped) {
+  constexpr int P = Elem<T>::per16;  // elements per 16-byte chunk
   const int64_t total = max_rows * chunks_per_row;
   const int64_t stride = (int64_t)gridDim.x * kBlock;
   for (int64_t c = (int64_t)blockIdx.x * kBlock + threadIdx.x; c < total; c += stride) {
@@ -233,13 +234,13 @@ __global__ __launch_bounds__(kBlock) void group_rows_stream_kernel(
     if (p < (int64_t)seg_starts[e] + counts[e]) {
       if (fan_out > 0) {
         const int32_t slot = row_slot[p];
-        v = load16(src + ((int64_t)(slot / fan_out) * chunks_per_row + ch) * 8);
+        v = load16(src + ((int64_t)(slot / fan_out) * chunks_per_row + ch) * P);
         if (coeff != nullptr) v = scale16<T>(v, Elem<T>::up(coeff[slot]));
       } else {
-        v = load16(src + c * 8);
+        v = load16(src + c * P);
       }
     }
-    store16_nt(grouped + c * 8, v);
+    store16_nt(grouped + c * P, v);
   }
 }
 
@@ -466,11 +467,13 @@ extern "C" int ck_group_rows_padded(const void* src, const void* coeff, int32_t 
   CK_REQUIRE(max_rows / kTile <= 65535, "ck_group_rows_padded: too many rows for one launch");
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)ceil_div(H, kTile), (unsigned)(max_rows / kTile));
-  if (grouped_t == nullptr) {
-    CK_DISPATCH_HALF(dtype, "ck_group_rows_padded", {
-      hipLaunchKernelGGL((group_rows_stream_kernel<scalar_t>), dim3(grid_for(max_rows * (H / 8), 2)), dim3(kBlock), 0, s,
+  if (grouped_t == nullptr) {  // the row-major copy alone: also for fp32 rows
+    CK_DISPATCH_FLOAT(dtype, "ck_group_rows_padded", {
+      constexpr int P = Elem<scalar_t>::per16;
+      CK_REQUIRE(H % P == 0, "ck_group_rows_padded: H=%d must be a multiple of %d", H, P);
+      hipLaunchKernelGGL((group_rows_stream_kernel<scalar_t>), dim3(grid_for(max_rows * (H / P), 2)), dim3(kBlock), 0, s,
                          static_cast<const scalar_t*>(src), static_cast<const scalar_t*>(coeff), (int)fan_out, row_slot,
-                         seg_starts, counts, tile_expert, (int)align, max_rows, (int)(H / 8),
+                         seg_starts, counts, tile_expert, (int)align, max_rows, (int)(H / P),
                          static_cast<scalar_t*>(grouped));
     });
     CK_CHECK_LAUNCH("ck_group_rows_padded");
@@ -571,7 +574,7 @@ extern "C" int ck_expert_bias_grad(const void* d_y, int32_t N, const ck_segments
   CK_REQUIRE(d_bias != nullptr && (seg->max_rows == 0 || d_y != nullptr), "%s: NULL argument", name);
   hipStream_t s = static_cast<hipStream_t>(stream);
   const dim3 grid((unsigned)ceil_div(N, kWave), (unsigned)seg->num_experts);
-  CK_DISPATCH_HALF(dtype, name, {
+  CK_DISPATCH_FLOAT(dtype, name, {
     hipLaunchKernelGGL((expert_bias_grad_kernel<scalar_t>), grid, dim3(kBlock), 0, s, static_cast<const scalar_t*>(d_y),
                        (int)N, seg->seg_starts, seg->counts, static_cast<scalar_t*>(d_bias));
   });

@@ -83,6 +83,11 @@ _SIGNATURES = {
         c_int32,
         [c_void_p, c_void_p, c_void_p, c_float, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int32, c_void_p],
     ),
+    "ck_grouped_gemm_f32": (
+        c_int32,
+        [c_void_p, c_int32, c_void_p, c_int32, c_int32, c_int32, POINTER(ck_segments), c_int32, c_void_p, c_void_p, c_void_p],
+    ),
+    "ck_grouped_gemm_dw_f32": (c_int32, [c_void_p, c_void_p, c_int32, c_int32, POINTER(ck_segments), c_void_p, c_void_p]),
     "ck_gelu_tanh_bwd": (c_int32, [c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_void_p]),
     "ck_swiglu_bwd": (
         c_int32,

@@ -256,8 +256,23 @@ _EPILOGUE_NAMES = {
 }
 
 
+def _gemm_f32(a, gather_div, w, w_is_kn: bool, N: int, K: int, seg: ExpertSegments, scatter: bool, y, bias=None):
+    """The grouped GEMMs of fp32 tensors (fp32 MFMA; see ck_grouped_gemm_f32)."""
+    cs = seg.c_struct()
+    with torch.cuda.device(w.device):
+        _C.check(
+            _C.lib().ck_grouped_gemm_f32(
+                _C.ptr(a), gather_div, _C.ptr(w), int(w_is_kn), N, K, ctypes.byref(cs), int(scatter), _C.ptr(y), _C.ptr(bias),
+                _C.stream(),
+            )
+        )
+
+
 def _gemm(a, gather_div, w, seg: ExpertSegments, epilogue, y, y_t=None, aux=None, aux_in=None):
     E, N, K = w.shape
+    if w.dtype == torch.float32:
+        assert epilogue in (_C.CK_EPI_GROUPED, _C.CK_EPI_SCATTER) and y_t is None and aux is None
+        return _gemm_f32(a, gather_div, w, False, N, K, seg, epilogue == _C.CK_EPI_SCATTER, y, aux_in)
     cs = seg.c_struct()
     if gather_div > 0:  # gathered rows are addressed with 32-bit byte offsets from the start of `a` (the library is not
         # told how many rows `a` has, so this limit is checked here)
@@ -287,11 +302,19 @@ def _bias_in_epilogue(seg: ExpertSegments, K: int) -> bool:
     return os.environ.get("CK_GEMM_BIAS_FUSED", "1") != "0"
 
 
+def _fp32(t: torch.Tensor) -> bool:
+    """fp32 expert tensors: always the row-major weight-gradient form and the bias in the GEMM's epilogue (the fp32
+    kernels have no other form)."""
+    return t.dtype == torch.float32
+
+
 def _gemm_dx(d_y, w, seg: ExpertSegments, epilogue, out):
     """out = d_y @ w[e] per expert, w [E, out_features, in_features] as the forward stores it: the input-gradient GEMM.
     Reads w contraction-strided where the kernel for that exists (256-row tiles, out_features % 64 == 0); otherwise
     through a transposed copy."""
     E, n_out, n_in = w.shape
+    if w.dtype == torch.float32:
+        return _gemm_f32(d_y, 0, w, True, n_in, n_out, seg, epilogue == _C.CK_EPI_SCATTER, out)
     if seg.align == 256 and n_out % 64 == 0 and _nn_enabled():
         cs = seg.c_struct()
 
@@ -341,6 +364,10 @@ def _gemm_dw_rows(a, b, seg: ExpertSegments, dw):
     """dw[e] = a[rows of e]^T @ b[rows of e] from row-major padded-grouped operands (no transposed copies)."""
     E, M, N = dw.shape
     cs = seg.c_struct()
+    if dw.dtype == torch.float32:
+        with torch.cuda.device(dw.device):
+            _C.check(_C.lib().ck_grouped_gemm_dw_f32(_C.ptr(a), _C.ptr(b), M, N, ctypes.byref(cs), _C.ptr(dw), _C.stream()))
+        return
 
     def launch():
         with torch.cuda.device(dw.device):
@@ -467,10 +494,8 @@ def _slot_experts(seg: ExpertSegments) -> torch.Tensor:
 
 
 def _check_expert_dtypes(x: torch.Tensor, *weights: torch.Tensor) -> None:
-    if x.dtype not in (torch.bfloat16, torch.float16):
-        raise NotImplementedError(
-            f"the MI355X expert GEMMs take bf16 / fp16 inputs with fp32 accumulation; got {x.dtype}"
-        )
+    if x.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        raise NotImplementedError(f"the MI355X expert GEMMs take bf16 / fp16 / fp32 inputs; got {x.dtype}")
     for w in weights:
         assert w.dtype == x.dtype, "expert weights and activations should have the same dtype"
     assert x.size(-1) % 8 == 0, "hidden size should be a multiple of 8"
@@ -492,7 +517,7 @@ class _ExpertsUp(torch.autograd.Function):
         # pad rows are never written by the kernel; zeros keep any activation applied on top finite
         y = torch.zeros(seg.max_rows, N, dtype=x.dtype, device=x.device)
         act = torch.zeros_like(y) if gelu else None
-        fused_bias = bias is not None and (gelu or _bias_in_epilogue(seg, K))
+        fused_bias = bias is not None and (gelu or _fp32(x) or _bias_in_epilogue(seg, K))
         _gemm(x, k, w, seg, _C.CK_EPI_GELU_TANH if gelu else _C.CK_EPI_GROUPED, y, aux=act,
               aux_in=bias.contiguous() if fused_bias else None)
         if bias is not None and not fused_bias:
@@ -522,7 +547,7 @@ class _ExpertsUp(torch.autograd.Function):
             d_bias = _expert_bias_grad(d_y, seg)
         if ctx.needs_input_grad[1]:
             d_w = torch.empty_like(w)
-            if _dw_from_rows(seg.max_rows, seg.num_experts, seg.align, tuple(w.shape[1:])):
+            if _fp32(x) or _dw_from_rows(seg.max_rows, seg.num_experts, seg.align, tuple(w.shape[1:])):
                 x_g, _ = _group_rows(x, None, k, seg, True, False)
                 _gemm_dw_rows(d_y, x_g, seg, d_w)
             else:
@@ -548,7 +573,7 @@ class _ExpertsDown(torch.autograd.Function):
         T, k = gates.shape
         E, N, K = w.shape
         expanded = torch.empty(T * k, N, dtype=h.dtype, device=h.device)
-        fused_bias = bias is not None and _bias_in_epilogue(seg, K)
+        fused_bias = bias is not None and (_fp32(h) or _bias_in_epilogue(seg, K))
         _gemm(h, 0, w, seg, _C.CK_EPI_SCATTER, expanded, aux_in=bias.contiguous() if fused_bias else None)
         if bias is not None and not fused_bias:  # before the gate multiply, as torch_implementation.py:160-163
             _add_expert_bias(expanded, bias.contiguous(), seg, slot_expert if slot_expert is not None else _slot_experts(seg))
@@ -568,7 +593,7 @@ class _ExpertsDown(torch.autograd.Function):
         if ctx.needs_input_grad[2]:
             d_gates = _gate_grad(expanded, grad_out, T, k, N, gates.dtype, ctx.gate_slot)
         need_w = ctx.needs_input_grad[1]
-        rows_form = _dw_from_rows(seg.max_rows, seg.num_experts, seg.align, (N, K))
+        rows_form = _fp32(h) or _dw_from_rows(seg.max_rows, seg.num_experts, seg.align, (N, K))
         d_y, d_y_t = _group_rows(grad_out, gates, k, seg, True, need_w and not rows_form)
         if len(ctx.needs_input_grad) > 4 and ctx.needs_input_grad[4]:
             d_bias = _expert_bias_grad(d_y, seg)  # d_y: the gate-scaled grad_out rows in padded grouped order
@@ -727,6 +752,7 @@ def swiglu_experts(
     """Fused expert block for `is_glu=True` (c_fc columns [up | gate]) with `activation_function = swiglu_packed_cute`
     (act_kind CK_ACT_SWIGLU: up * silu(gate)) or `torch.nn.GLU()` (CK_ACT_GLU: up * sigmoid(gate))."""
     _check_expert_dtypes(x, w_fc, w_proj)
+    assert x.dtype != torch.float32, "the fused expert block is 16-bit; fp32 layers run experts_up -> activation -> experts_down"
     assert w_fc.size(1) % 16 == 0, "intermediate size should be a multiple of 8"
     if is_tracing():
         grad = torch.is_grad_enabled()

@@ -127,7 +127,8 @@ int ck_gate_grad_f32(const void* expanded, const void* grad_out, int64_t T, int3
  *   row p valid : grouped[p, :] = src[row_slot[p] / fan_out, :] * (coeff ? coeff[row_slot[p]] : 1)
  *   row p pad   : zeros
  * fan_out == 0 (coeff must be NULL): src is itself padded-grouped [max_rows, H] and valid row p reads src[p, :].
- * grouped [max_rows, H] may be NULL; grouped_t [H, ld_t] (ld_t >= max_rows) may be NULL. bf16 / f16 only. */
+ * grouped [max_rows, H] may be NULL; grouped_t [H, ld_t] (ld_t >= max_rows) may be NULL. bf16 / f16; fp32 for the
+ * row-major copy alone (grouped_t NULL). */
 int ck_group_rows_padded(const void* src, const void* coeff, int32_t fan_out, int32_t H, const int32_t* row_slot,
                          const int32_t* seg_starts, const uint32_t* counts, const int32_t* tile_expert,
                          int32_t align, int64_t max_rows, void* grouped, void* grouped_t, int64_t ld_t,
@@ -204,6 +205,20 @@ int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* w, int32_t 
  * Needs seg->align == 256, K % 64 == 0, N % 8 == 0. */
 int ck_grouped_gemm_nn(const void* a, const void* w, int32_t N, int32_t K, const ck_segments* seg, int32_t epilogue,
                        void* y, int32_t dtype, void* stream);
+
+/* The same grouped GEMMs for fp32 tensors (the dtype of the reference's test grid, tests/test_commons.py:26-27): fp32
+ * products and fp32 accumulation on v_mfma_f32_32x32x2_f32 (the reference's Triton kernels round fp32 operands to TF32,
+ * kernels.py:131,218). y[out_row(p), :] = a[a_row(p), :] @ W_e (+ bias[e, :]) for every valid padded row p:
+ *   a_row(p) = row_slot[p] / a_gather_div (a_gather_div > 0, token order) or p (0, padded grouped rows), a [*, K];
+ *   W_e = w[e]^T with w [E, N, K] (w_is_kn == 0: the forward linears) or w[e] with w [E, K, N] (w_is_kn != 0: the input
+ *   gradient, reading the forward's weight as stored); out_row(p) = row_slot[p] (scatter != 0) or p; bias [E, N] or NULL.
+ * Replaces: scatter2scatter for fp32 inputs -- triton_implementation/ops.py:31-78. seg->align % 64 == 0; N, K % 4 == 0. */
+int ck_grouped_gemm_f32(const float* a, int32_t a_gather_div, const float* w, int32_t w_is_kn, int32_t N, int32_t K,
+                        const ck_segments* seg, int32_t scatter, float* y, const float* bias, void* stream);
+/* dw[e] = a[rows of e]^T @ b[rows of e] for fp32 padded-grouped rows a [max_rows, M], b [max_rows, N]; dw [E, M, N], exact
+ * zeros for experts without rows. Replaces: group_bwd_W for fp32 inputs -- ops.py:81-105. M, N % 4 == 0. */
+int ck_grouped_gemm_dw_f32(const float* a, const float* b, int32_t M, int32_t N, const ck_segments* seg, float* dw,
+                           void* stream);
 
 /* dW[e] = A_t[:, seg_e] * B_t[:, seg_e]^T : A_t [M, ld_t], B_t [N, ld_t] are transposed padded-grouped operands with
  * zeros in pad rows; dw [E, M, N]. Experts with no rows get exact zeros (ops.py:252, kernels.py:181). */
