@@ -224,6 +224,8 @@ __global__ __launch_bounds__(kBlock) void count_kernel(const id_t* __restrict__ 
 // ------------------------------------------------------------------------------------------------------------
 // sort
 // ------------------------------------------------------------------------------------------------------------
+constexpr int kSortUnroll = 8;  // ids a lane fetches before it consumes them
+
 struct SortPlan {
   int segments;    // multiple of kWavesPerBlock
   int64_t seg_len; // multiple of kWave
@@ -262,9 +264,17 @@ __global__ __launch_bounds__(kBlock) void sort_hist_kernel(const id_t* __restric
   const int seg = blockIdx.x * kWavesPerBlock + wave;
   const int64_t begin = (int64_t)seg * seg_len;
   const int64_t end = min(R, begin + seg_len);
-  for (int64_t i = begin + lane; i < end; i += kWave) {
-    const int id = load_id(ids + i);
-    if ((unsigned)id < (unsigned)E) atomicAdd(&my_hist[id], 1u);
+  // kSortUnroll loads in flight per lane: a segment is a handful of dependent-latency round trips otherwise
+  for (int64_t base = begin + lane; base < end; base += kSortUnroll * kWave) {
+    int id[kSortUnroll];
+#pragma unroll
+    for (int u = 0; u < kSortUnroll; ++u) {
+      const int64_t i = base + u * kWave;
+      id[u] = i < end ? load_id(ids + i) : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < kSortUnroll; ++u)
+      if ((unsigned)id[u] < (unsigned)E) atomicAdd(&my_hist[id[u]], 1u);
   }
   __syncthreads();
   uint32_t* table = ws + 1;
@@ -331,10 +341,19 @@ __global__ __launch_bounds__(kBlock) void sort_scatter_kernel(const id_t* __rest
   const int64_t begin = (int64_t)seg * seg_len;
   const int64_t end = min(R, begin + seg_len);
   const uint64_t lanes_below = (lane == 0) ? 0ull : (~0ull >> (kWave - lane));
-  for (int64_t base = begin; base < end; base += kWave) {
+  for (int64_t chunk = begin; chunk < end; chunk += kSortUnroll * kWave) {
+    int ids_ahead[kSortUnroll];  // the ids of the next kSortUnroll rounds, fetched together
+#pragma unroll
+    for (int u = 0; u < kSortUnroll; ++u) {
+      const int64_t i = chunk + u * kWave + lane;
+      ids_ahead[u] = i < end ? load_id(ids + i) : -1;
+    }
+#pragma unroll
+    for (int u = 0; u < kSortUnroll; ++u) {
+    const int64_t base = chunk + u * kWave;
+    if (base >= end) break;
     const int64_t i = base + lane;
-    int id = -1;
-    if (i < end) id = load_id(ids + i);
+    const int id = ids_ahead[u];
     const bool valid = (unsigned)id < (unsigned)E;
     uint64_t peers = __ballot(valid);
     for (int b = 0; b < id_bits; ++b) {
@@ -350,6 +369,7 @@ __global__ __launch_bounds__(kBlock) void sort_scatter_kernel(const id_t* __rest
       sorted_expert_idxs[pos] = id;
       sorted_scattered_idxs[pos] = (int32_t)i;
       row_slot[(uint32_t)seg_starts[id] + (pos - starts[id])] = (int32_t)i;
+    }
     }
   }
 }
