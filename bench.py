@@ -30,21 +30,22 @@ PEAK_HBM_GBS = 8000.0  # MI355X HBM3E
 # this same command, FETCH_SIZE scaled x2.0 and WRITE_SIZE x1.0 against a 1 GiB device copy (known size);
 # summary and commands: profiles/grouped_gemm_c3_moe_fwd_bwd.md. Not measurable from inside this process.
 TRAFFIC_BYTES_PER_LAUNCH = {
-    "grouped_gemm_dw_rows": 2 * 5.883e6 * 1024 + 1.376e6 * 1024,  # both weight gradients, row-major operands
-    "grouped_gemm<swiglu>": 2 * 8.886e6 * 1024 + 2.753e6 * 1024,  # c_fc forward
-    "grouped_gemm_nn<scatter>": 2 * 8.130e6 * 1024 + 2.622e5 * 1024,  # c_fc dX, contraction-strided weights
-    "grouped_gemm_nn<grouped>": 2 * 3.811e6 * 1024 + 9.175e5 * 1024,  # c_proj dX, contraction-strided weights
-    "grouped_gemm<scatter>": 2 * 3.316e6 * 1024 + 3.275e5 * 1024,  # c_proj forward, 256 x 384 tiles
+    "grouped_gemm_dw_rows": 2 * 5.930e6 * 1024 + 1.376e6 * 1024,  # both weight gradients, row-major operands
+    "grouped_gemm<swiglu>": 2 * 7.045e6 * 1024 + 2.753e6 * 1024,  # c_fc forward
+    "grouped_gemm_nn<scatter>": 2 * 8.243e6 * 1024 + 2.621e5 * 1024,  # c_fc dX, contraction-strided weights
+    "grouped_gemm_nn<grouped>": 2 * 3.723e6 * 1024 + 9.175e5 * 1024,  # c_proj dX, contraction-strided weights
+    "grouped_gemm<scatter>": 2 * 3.905e6 * 1024 + 2.621e5 * 1024,  # c_proj forward
 }
 
 # the kernel instantiation each launch name runs at this workload, as rocprofv3's kernel trace spells it
-# (grouped_gemm_line_kernel<T, MODE, BN, BT>: MODE 0 grouped, 1 scatter, 2 swiglu, 4 dw)
+# (grouped_gemm_line_kernel<T, MODE, BN, BT, WGM, EXTRA>: MODE 0 grouped, 1 scatter, 2 swiglu, 4 dw; BT: contraction-strided
+# operands; WGM = 2: four waves, one per SIMD; EXTRA: bias / side outputs)
 ROCPROF_KERNEL = {
-    "grouped_gemm_dw_rows": "grouped_gemm_line_kernel<bf16, 4, 256, true>",
-    "grouped_gemm<swiglu>": "grouped_gemm_line_kernel<bf16, 2, 256, false>",
-    "grouped_gemm_nn<scatter>": "grouped_gemm_line_kernel<bf16, 1, 256, true>",
-    "grouped_gemm_nn<grouped>": "grouped_gemm_line_kernel<bf16, 0, 256, true>",
-    "grouped_gemm<scatter>": "grouped_gemm_line_kernel<bf16, 1, 384, false>",
+    "grouped_gemm_dw_rows": "grouped_gemm_line_kernel<bf16, 4, 256, true, 2, false>",
+    "grouped_gemm<swiglu>": "grouped_gemm_line_kernel<bf16, 2, 256, false, 2, false>",
+    "grouped_gemm_nn<scatter>": "grouped_gemm_line_kernel<bf16, 1, 256, true, 2, false>",
+    "grouped_gemm_nn<grouped>": "grouped_gemm_line_kernel<bf16, 0, 256, true, 2, false>",
+    "grouped_gemm<scatter>": "grouped_gemm_line_kernel<bf16, 1, 256, false, 2, false>",
 }
 
 # workload: configs[2] of the baseline, the configuration its headline metric (MoE fwd+bwd TFLOP/s) is quoted on
@@ -241,7 +242,21 @@ def secondary_hbm_kernels(dev):
         timed(lambda: torch.autograd.grad((yf, af), (xn, rn, wn), (gn, ga), retain_graph=True)),
         5 * Bn * Hn * 2 + 4 * Bn,
     )
-    del xn, wn, yn, gn, rn, yf, af, ga
+    del yn, gn, rn, yf, af, ga
+    # RMSNorm fused ahead of the router (one pass: normalised rows + router logits, optionally the e4m3 rows) against the
+    # separate kernels (rmsnorm, the router's linear layer on the BLAS library, the row quantiser); algorithmic bytes:
+    # rows in and out once, logits out (+ 1 byte per element and a scale per row with the e4m3 rows)
+    for tag, (Bp, Hp, Ep) in {"C4": (8192, 2048, 64), "C5": (65536, 4096, 128)}.items():
+        xr_, wr_ = xn.detach()[:Bp, :Hp].contiguous(), wn.detach()[:Hp].contiguous()
+        gr_ = (torch.randn(Ep, Hp, device=dev) * Hp**-0.5).to(torch.bfloat16)
+        b_plain, b_quant = 2 * Bp * Hp * 2 + Bp * Ep * 2, 2 * Bp * Hp * 2 + Bp * Ep * 2 + Bp * Hp + 4 * Bp
+        with torch.no_grad():
+            rec(f"rmsnorm_route_{tag}", timed(lambda: cute_kernels.rmsnorm_route_cute(xr_, wr_, gr_, 1e-6, fused=True)), b_plain)
+            rec(f"rmsnorm_route_e4m3_{tag}", timed(lambda: cute_kernels.rmsnorm_route_cute(xr_, wr_, gr_, 1e-6, quantize=True, fused=True)), b_quant)
+            rec(f"rmsnorm_then_linear_{tag}", timed(lambda: cute_kernels.rmsnorm_route_cute(xr_, wr_, gr_, 1e-6, fused=False)), b_plain)
+            rec(f"rmsnorm_then_linear_then_quant_{tag}", timed(lambda: cute_kernels.rmsnorm_route_cute(xr_, wr_, gr_, 1e-6, quantize=True, fused=False)), b_quant)
+        del xr_, wr_, gr_
+    del xn, wn
     # router-logit statistics: softmax over all experts at the C5 router shape (65,536 x 128)
     lg = torch.randn(Bn, 128, device=dev, dtype=torch.bfloat16, requires_grad=True)
     rec("softmax_fwd_C5_router", timed(lambda: cute_kernels.softmax_cute(lg.detach())), 2 * Bn * 128 * 2)
@@ -264,7 +279,7 @@ def secondary_hbm_kernels(dev):
             p_.grad = None
         x4.grad = None
         w4.grad = None
-        y4, _ = moe4(cute_kernels.rmsnorm_cute(x4, w4, 1e-6))
+        y4, _ = moe4.forward_with_norm(x4, w4, 1e-6)  # the norm fused ahead of the router: one kernel for rows + logits
         y4.backward(g4)
 
     dt = timed(step4, iters=10)
@@ -291,8 +306,8 @@ def secondary_hbm_kernels(dev):
     torch.cuda.empty_cache()
 
     def step5():
-        with torch.no_grad():
-            q5(cute_kernels.rmsnorm_cute(x5, w5, 1e-6))
+        with torch.no_grad():  # separate norm: at E * H = 128 * 4096 the one-pass prologue kernel does not pay (see the
+            q5(cute_kernels.rmsnorm_cute(x5, w5, 1e-6))  # rmsnorm_route_* lines), and the Zipf bias enters through the gate's hook
 
     dt = timed(step5, iters=5)
     timer = scattermoe.LaunchTimer()
