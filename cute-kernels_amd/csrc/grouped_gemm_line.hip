@@ -25,6 +25,9 @@
 #define CK_ABLATE 0  // measurement builds only (build.py --define CK_ABLATE=n --output ...): 1 no barrier, 2 no loads in the loop, 4 no fragment reads, 8 no wait for the loads, 16 every step loads the first two K steps again (L2 hits), 32 no epilogue, 64 no MFMA, 128 no row-major output stores
 #endif
 
+#ifndef CK_L2_PREFETCH
+#define CK_L2_PREFETCH 0  // > 0: every wave touches, with two 4-byte loads per K step, the lines its loads of step kt + n will fetch
+#endif
 #ifndef CK_LOAD_GAP
 #define CK_LOAD_GAP 0  // measurement builds only: MFMAs between two loads of the next-but-one K step (0: spread over the whole last slice)
 #endif
@@ -239,6 +242,53 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
 #pragma unroll
     for (int g = 0; g < kLoadsPerStep; ++g) issue_one(step, g);
   };
+  // L2 warm-up (measurement switch): lane l asks for 4 bytes of line l of the 64 lines of each operand that this wave's
+  // loads of a later step will fetch, so that those loads find their lines in L2 (27 % of them miss otherwise)
+  uint32_t pf_a = 0, pf_b = 0, pf_d0 = 0, pf_d1 = 0;
+  if constexpr (CK_L2_PREFETCH > 0) {
+    if constexpr (AT) {
+      const int n = wave * 16 + (lane >> 2);
+      int64_t col = m0 + (lane & 3) * 64;
+      if (col >= prm.M) col = m0;
+      pf_a = (uint32_t)(((int64_t)n * prm.lda + col) * 2);
+    } else {
+      const int r = wave * 64 + lane;
+      int64_t row;
+      if constexpr (MODE == kDw) {
+        row = min(m0 + r, (int64_t)prm.M - 1);
+      } else {
+        int64_t p = m0 + r;
+        if (p >= valid_end) p = valid_end - 1;
+        row = prm.a_gather_div > 0 ? (int64_t)(prm.row_slot[p] / prm.a_gather_div) : p - m0;
+      }
+      pf_a = (uint32_t)((row * prm.lda + k_begin) * 2);
+    }
+    if constexpr (BT) {
+      const int n = wave * 16 + (lane >> 2);
+      int64_t col = (int64_t)nt * BN + (lane & 3) * 64;
+      if (col >= prm.N) col = (int64_t)nt * BN;
+      pf_b = (uint32_t)(((int64_t)n * prm.ldw + col) * 2);
+    } else {
+      const int j = wave * 64 + lane;
+      int64_t n;
+      if constexpr (MODE == kSwiglu) {
+        const int half = (j % WN) / (WN / 2);
+        const int within = (j / WN) * (WN / 2) + (j % (WN / 2));
+        n = (int64_t)half * prm.I + min((int64_t)nt * (BN / 2) + within, (int64_t)prm.I - 1);
+      } else {
+        n = min((int64_t)nt * BN + j, (int64_t)prm.N - 1);
+      }
+      pf_b = (uint32_t)((n * prm.ldw + k_begin) * 2);
+    }
+  }
+  // the destination registers stay allocated for the whole loop ("+v"): a load may land long after it was issued
+  auto warm_l2 = [&](int step) {
+    const int64_t kb = (int64_t)step * kRowBytes;
+    const int64_t kb_b = BT ? (int64_t)step * BK * prm.ldw * 2 : kb;
+    const int64_t kb_a = AT ? (int64_t)step * BK * prm.lda * 2 : kb;
+    asm volatile("global_load_dword %0, %1, %2" : "+v"(pf_d0) : "v"(pf_a), "s"(a_base_u + kb_a));
+    asm volatile("global_load_dword %0, %1, %2" : "+v"(pf_d1) : "v"(pf_b), "s"(b_base_u + kb_b));
+  };
 
   // ---- fragments: slice sl of a row is its 16-byte chunks 4 sl + lane / 16 (the lane's 8 contraction values)
   typedef typename Mfma16<T>::frag frag_t;
@@ -391,10 +441,13 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
           st_bar += t2 - t1;
           st_s0 += t0 - st_mark;  // slice 0 of this step (the slice in front of the wait)
           st_mark = t2;
+        } else if constexpr (CK_L2_PREFETCH > 0 && kPhase == 0) {
+          asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)\n\ts_barrier" ::: "memory");  // all but this step's two warm-up loads
         } else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       }
       constexpr int cur = kDouble ? (decltype(sl)::value & 1) : 0;
       constexpr int nxt = kDouble ? (cur ^ 1) : 0;
+      if constexpr (CK_L2_PREFETCH > 0 && decltype(sl)::value == 0 && kPhase == 0) warm_l2(min(kt + CK_L2_PREFETCH, nk - 1));
 #pragma unroll
       for (int n = 0; n < MI * NI; ++n) {
         const int i = n / NI, j = n % NI;
