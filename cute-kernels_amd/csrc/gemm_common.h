@@ -40,7 +40,16 @@ struct GemmParams {
   int act_kind;          // kSwiglu epilogue: CK_ACT_SWIGLU (up * gate * sigmoid(gate)) or CK_ACT_GLU (up * sigmoid(gate));
                          // kGrouped epilogue with aux: CK_ACT_GELU_TANH (aux = gelu(y), second output)
   void* trace;           // measurement builds only: per-workgroup phase timestamps (8 x uint64 each), else NULL
+  // Split contraction for the last, partial round of tiles (128-byte-row kernel, grouped / scatter epilogues):
+  // split_ws = [tiles][parts][4 waves][64 blocks][64 lanes] f32x4 partial accumulators (at most kSplitMaxTail tiles in
+  // kSplitParts parts or twice as many in half as many parts), followed by 2 * kSplitMaxTail int32 arrival counters (zero between launches); NULL = never split. split_base = the launch's grid
+  // without the extra workgroups (they are blockIdx split_base ..).
+  float* split_ws;
+  int split_base;
 };
+constexpr int kSplitParts = 4, kSplitMaxTail = 64, kSplitMaxRounds = 16, kSplitMinSteps = 32;
+constexpr int64_t kSplitPartFloats = 4 * 64 * 64 * 4;  // one workgroup's 256 x 256 fp32 tile
+constexpr int64_t kSplitWorkspaceBytes = kSplitMaxTail * kSplitParts * kSplitPartFloats * 4 + 2 * kSplitMaxTail * 4;
 
 // The 16-bit kernel with 128-byte LDS rows (grouped_gemm_line.hip): 256 x bn tiles, bn = 256 or 384, contraction length a
 // multiple of 64, modes kGrouped, kScatter, kSwiglu, kDw. The caller fills `prm` for these tile dimensions (n_tiles,
@@ -106,6 +115,11 @@ struct Mfma16<bf16_t> {
   __device__ static inline void run_acc(const frag& a, const frag& b, f32x4& c) {
     asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
   }
+  // the first product of a tile: c = a * b + 0 (the constant as the third operand), so that nothing has to zero the
+  // accumulators first -- 256 v_accvgpr_write per wave, which the compiler also re-materialised in front of the loop
+  __device__ static inline void run_acc_first(const frag& a, const frag& b, f32x4& c) {
+    asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
+  }
 };
 template <>
 struct Mfma16<f16_t> {
@@ -115,6 +129,9 @@ struct Mfma16<f16_t> {
   }
   __device__ static inline void run_acc(const frag& a, const frag& b, f32x4& c) {
     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
+  }
+  __device__ static inline void run_acc_first(const frag& a, const frag& b, f32x4& c) {
+    asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
   }
 };
 // after the last run_acc, before anything else reads the accumulators: longer than any MFMA's result latency

@@ -787,9 +787,17 @@ int launch_by_tile(const GemmParams& prm, int align, unsigned blocks_256, unsign
 
 using namespace ck;
 
-extern "C" int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* w, int32_t N, int32_t K,
-                               const ck_segments* seg, int32_t epilogue, void* y, void* y_t, int64_t ld_t, void* aux,
-                               const void* aux_in, int32_t dtype, void* stream) {
+namespace {
+// workspace for the split last round (NULL: never split): kSplitWorkspaceBytes, 16-byte aligned, counters zero
+inline float* split_workspace(void* workspace, int64_t workspace_bytes) {
+  if (workspace == nullptr || workspace_bytes < kSplitWorkspaceBytes || !aligned16(workspace)) return nullptr;
+  return static_cast<float*>(workspace);
+}
+}  // namespace
+
+static int grouped_gemm_impl(const void* a, int32_t a_gather_div, const void* w, int32_t N, int32_t K,
+                             const ck_segments* seg, int32_t epilogue, void* y, void* y_t, int64_t ld_t, void* aux,
+                             const void* aux_in, int32_t dtype, void* stream, void* workspace, int64_t workspace_bytes) {
   const char* name = "ck_grouped_gemm";
   if (int rc = check_segments(seg, name)) return rc;
   CK_REQUIRE(N >= 8 && K >= 8 && N % 8 == 0 && K % 8 == 0, "%s: N=%d and K=%d must be positive multiples of 8", name, N, K);
@@ -842,6 +850,7 @@ extern "C" int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* 
   prm.ld_t = ld_t;
   prm.aux = aux;
   prm.aux_in = aux_in;
+  prm.split_ws = split_workspace(workspace, workspace_bytes);
 #if (CK_ABLATE & 256) || defined(CK_STAMP)
   if (const char* t = getenv("CK_TRACE_PTR")) prm.trace = reinterpret_cast<void*>(strtoull(t, nullptr, 16));
 #endif
@@ -886,8 +895,25 @@ extern "C" int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* 
   return CK_OK;
 }
 
-extern "C" int ck_grouped_gemm_nn(const void* a, const void* w, int32_t N, int32_t K, const ck_segments* seg,
-                                  int32_t epilogue, void* y, int32_t dtype, void* stream) {
+extern "C" int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* w, int32_t N, int32_t K,
+                               const ck_segments* seg, int32_t epilogue, void* y, void* y_t, int64_t ld_t, void* aux,
+                               const void* aux_in, int32_t dtype, void* stream) {
+  return grouped_gemm_impl(a, a_gather_div, w, N, K, seg, epilogue, y, y_t, ld_t, aux, aux_in, dtype, stream, nullptr, 0);
+}
+
+extern "C" int ck_grouped_gemm_ws(const void* a, int32_t a_gather_div, const void* w, int32_t N, int32_t K,
+                                  const ck_segments* seg, int32_t epilogue, void* y, void* y_t, int64_t ld_t, void* aux,
+                                  const void* aux_in, int32_t dtype, void* stream, void* workspace,
+                                  int64_t workspace_bytes) {
+  return grouped_gemm_impl(a, a_gather_div, w, N, K, seg, epilogue, y, y_t, ld_t, aux, aux_in, dtype, stream, workspace,
+                           workspace_bytes);
+}
+
+extern "C" int64_t ck_grouped_gemm_workspace_bytes(void) { return kSplitWorkspaceBytes; }
+
+static int grouped_gemm_nn_impl(const void* a, const void* w, int32_t N, int32_t K, const ck_segments* seg,
+                                int32_t epilogue, void* y, int32_t dtype, void* stream, void* workspace,
+                                int64_t workspace_bytes) {
   const char* name = "ck_grouped_gemm_nn";
   if (int rc = check_segments(seg, name)) return rc;
   CK_REQUIRE(seg->align == kLineBM, "%s: needs 256-row tiles (sort with align = 256)", name);
@@ -913,10 +939,22 @@ extern "C" int ck_grouped_gemm_nn(const void* a, const void* w, int32_t N, int32
   prm.tile_expert = seg->tile_expert;
   prm.row_slot = seg->row_slot;
   prm.y = y;
+  prm.split_ws = split_workspace(workspace, workspace_bytes);
   prm.n_tiles = (int)ceil_div(N, 256);
   const int64_t blocks = (seg->max_rows / seg->align) * prm.n_tiles;
   CK_REQUIRE(blocks < (int64_t)0x7fffffff, "%s: grid too large", name);
   return launch_line(prm, epilogue, 256, true, dtype, (unsigned)blocks, static_cast<hipStream_t>(stream), name);
+}
+
+extern "C" int ck_grouped_gemm_nn(const void* a, const void* w, int32_t N, int32_t K, const ck_segments* seg,
+                                  int32_t epilogue, void* y, int32_t dtype, void* stream) {
+  return grouped_gemm_nn_impl(a, w, N, K, seg, epilogue, y, dtype, stream, nullptr, 0);
+}
+
+extern "C" int ck_grouped_gemm_nn_ws(const void* a, const void* w, int32_t N, int32_t K, const ck_segments* seg,
+                                     int32_t epilogue, void* y, int32_t dtype, void* stream, void* workspace,
+                                     int64_t workspace_bytes) {
+  return grouped_gemm_nn_impl(a, w, N, K, seg, epilogue, y, dtype, stream, workspace, workspace_bytes);
 }
 
 extern "C" int ck_grouped_gemm_dw_rows(const void* a, const void* b, int32_t M, int32_t N, const ck_segments* seg,

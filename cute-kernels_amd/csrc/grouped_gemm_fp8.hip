@@ -45,6 +45,9 @@ __device__ inline void mfma_fp8(const i32x8& a, const i32x8& b, f32x4& c) {
   // cbsz = blgp = 0: both operands e4m3; accumulator pinned to AGPRs and updated in place (see Mfma16::run_acc)
   asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, %0" : "+a"(c) : "v"(a), "v"(b));
 }
+__device__ inline void mfma_fp8_first(const i32x8& a, const i32x8& b, f32x4& c) {  // c = a * b + 0 (see run_acc_first)
+  asm volatile("v_mfma_f32_16x16x128_f8f6f4 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
+}
 
 template <typename TO, int MODE>
 __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams prm) {
@@ -67,25 +70,29 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
   const int64_t m0 = (int64_t)mt * BM;
   const int64_t valid_end = (int64_t)prm.seg_starts[expert] + prm.counts[expert];
 
-  f32x4 acc[MI][NI];
-#pragma unroll
-  for (int i = 0; i < MI; ++i)
-#pragma unroll
-    for (int j = 0; j < NI; ++j)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+  f32x4 acc[MI][NI];  // started by the first K step's MFMAs (constant 0 as their third operand): nothing zeroes them
 
   // ---- global -> LDS addressing: lane l of a wave-load fills slot l (16 bytes) of 64 consecutive slots = 8 rows of 128 B
   const char* a_base = static_cast<const char*>(prm.a);
   const char* b_base = static_cast<const char*>(prm.w) + (int64_t)expert * prm.w_expert_stride;
   uint32_t a_off[A_LD], b_off[B_LD];
+  // gathered input: the row_slot entries of this lane's tile rows are fetched together (one wait, not one per load)
+  // into the registers that then take the offsets
+  if (prm.a_gather_div > 0) {
+#pragma unroll
+    for (int t = 0; t < A_LD; ++t) {
+      int64_t p = m0 + (wave * A_LD + t) * 8 + (lane >> 3);
+      if (p >= valid_end) p = valid_end - 1;
+      a_off[t] = (uint32_t)prm.row_slot[p];
+    }
+  }
 #pragma unroll
   for (int t = 0; t < A_LD; ++t) {
     const int r = (wave * A_LD + t) * 8 + (lane >> 3);
     const int c = (lane & 7) ^ swz128(r);
     int64_t p = m0 + r;
     if (p >= valid_end) p = valid_end - 1;  // pad rows re-read a valid row; their results are never stored
-    const int64_t row = prm.a_gather_div > 0 ? (int64_t)(prm.row_slot[p] / prm.a_gather_div) : p;
+    const int64_t row = prm.a_gather_div > 0 ? (int64_t)((int32_t)a_off[t] / prm.a_gather_div) : p;
     a_off[t] = (uint32_t)(row * prm.lda + c * 16);
   }
 #pragma unroll
@@ -164,12 +171,15 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
     if (g < MI) fa[g] = v;
     else fb[g - MI] = v;
   };
-  auto mfma = [&](int i, int j) {
+  auto mfma = [&](int i, int j, auto first) {
     if constexpr ((CK_ABLATE & 64) != 0) {
       asm volatile("" ::"v"(fa[i]), "v"(fb[j]));
+      if constexpr (decltype(first)::value) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
       return;
     }
-    mfma_fp8(fb[j], fa[i], acc[i][j]);  // weight fragment first: a lane gets 4 consecutive output columns of one row
+    // weight fragment first: a lane gets 4 consecutive output columns of one row
+    if constexpr (decltype(first)::value) mfma_fp8_first(fb[j], fa[i], acc[i][j]);
+    else mfma_fp8(fb[j], fa[i], acc[i][j]);
   };
 
   if (nk > 0) {
@@ -189,7 +199,7 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
     // step kt + 2 overwrite it, one every kLoadGap MFMAs. fa[i] is reloaded from the next stage once row block i is
     // done, fb[j] after the MFMA (MI - 1, j). Phase 1 is step nk - 2 (nothing left to fetch), phase 2 the last step
     // (nothing to wait for, nothing to reload).
-    auto k_step = [&](int kt, auto phase, auto idle) {
+    auto k_step = [&](int kt, auto phase, auto idle, auto first) {
       constexpr bool kIdle = decltype(idle)::value;  // this wave's rows are all pad rows: no fragments, no MFMAs
       constexpr int kPhase = decltype(phase)::value;
       const int ns = (kt + 1) & (NSTAGE - 1);
@@ -197,7 +207,7 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
 #pragma unroll
       for (int n = 0; n < MI * NI; ++n) {
         const int i = n / NI, j = n % NI;
-        if constexpr (!kIdle) mfma(i, j);
+        if constexpr (!kIdle) mfma(i, j, first);
         if constexpr (kPhase == 0) {
           if (n % kLoadGap == 0 && n / kLoadGap < kLoadsPerStep) issue_one(kt + 2, n / kLoadGap);
         }
@@ -209,11 +219,24 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
       }
       __builtin_amdgcn_sched_barrier(0);
     };
-    auto k_loop = [&](auto idle) {
-      int kt = 0;
-      for (; kt + 2 < nk; ++kt) k_step(kt, std::integral_constant<int, 0>{}, idle);
-      if (kt + 2 == nk) k_step(kt++, std::integral_constant<int, 1>{}, idle);
-      k_step(kt, std::integral_constant<int, 2>{}, idle);
+    auto k_loop = [&](auto idle) {  // the first step is peeled: its MFMAs start the accumulators
+      constexpr std::integral_constant<int, 0> p0{};
+      constexpr std::integral_constant<int, 1> p1{};
+      constexpr std::integral_constant<int, 2> p2{};
+      constexpr std::true_type first{};
+      constexpr std::false_type later{};
+      if (nk >= 3) {
+        k_step(0, p0, idle, first);
+        int kt = 1;
+        for (; kt + 2 < nk; ++kt) k_step(kt, p0, idle, later);
+        k_step(kt++, p1, idle, later);
+        k_step(kt, p2, idle, later);
+      } else if (nk == 2) {
+        k_step(0, p1, idle, first);
+        k_step(1, p2, idle, later);
+      } else {
+        k_step(0, p2, idle, first);
+      }
     };
     const bool wave_idle = m0 + wm * WM >= valid_end;
     if (__builtin_amdgcn_readfirstlane(wave_idle)) k_loop(std::true_type{});

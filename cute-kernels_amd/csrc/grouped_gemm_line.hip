@@ -25,9 +25,6 @@
 #define CK_ABLATE 0  // measurement builds only (build.py --define CK_ABLATE=n --output ...): 1 no barrier, 2 no loads in the loop, 4 no fragment reads, 8 no wait for the loads, 16 every step loads the first two K steps again (L2 hits), 32 no epilogue, 64 no MFMA, 128 no row-major output stores
 #endif
 
-#ifndef CK_L2_PREFETCH
-#define CK_L2_PREFETCH 0  // > 0: every wave touches, with two 4-byte loads per K step, the lines its loads of step kt + n will fetch
-#endif
 #ifndef CK_LOAD_GAP
 #define CK_LOAD_GAP 0  // measurement builds only: MFMAs between two loads of the next-but-one K step (0: spread over the whole last slice)
 #endif
@@ -85,9 +82,11 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   if constexpr (CK_STAMP != 0) st_begin = clock64();
 
   // ---- which tile (same XCD-aware orders as the 256 x 256 kernel)
+  constexpr bool kSplit = WGM == 2 && (MODE == kGrouped || MODE == kScatter);  // see the split below
   int mt, nt, expert;
   int64_t k_begin = 0;
   int k_len;
+  [[maybe_unused]] int split_slot = -1, split_part = -1, split_parts = kSplitParts;
   if constexpr (MODE == kDw) {
     const int per_expert = prm.m_tiles * prm.n_tiles;
     const bool m_major = prm.m_tiles >= prm.n_tiles;
@@ -111,12 +110,40 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
     const int live_m = prm.seg_starts[prm.num_experts] / prm.align;
     const int total = live_m * prm.n_tiles;
     int pid = blockIdx.x;
+    k_len = prm.K;
+    if constexpr (kSplit) {
+      // The tiles of the last, partial round (the highest block indices: the hardware hands blocks out in order) would
+      // each keep one CU busy for a whole tile time while the rest of the chip idles. When that round is at most half
+      // full, every such tile is computed by 2 to 4 workgroups (as many as fill the chip), an equal share of the contraction each: part
+      // 0 is the tile's own block, parts 1.. are extra blocks behind the regular grid. All write their fp32 accumulators
+      // to the workspace; the last to arrive (ticket) adds the parts up in part order and runs the epilogue.
+      const int cus = kXcds * 32;
+      const int tail = total % cus;
+      const bool active = prm.split_ws != nullptr && tail > 0 && tail <= 2 * kSplitMaxTail && total / cus <= kSplitMaxRounds &&
+                          prm.K / BK >= kSplitMinSteps;
+      split_parts = active ? min(kSplitParts, cus / tail) : kSplitParts;  // as many parts as fill the chip: 4, 3 or 2
+      if (pid >= prm.split_base) {  // an extra block
+        const int x = pid - prm.split_base;
+        split_slot = x / (split_parts - 1);
+        split_part = x % (split_parts - 1) + 1;
+        if (!active || split_slot >= tail) return;
+        pid = total - tail + split_slot;
+      } else if (active && pid >= total - tail && pid < total) {
+        split_slot = pid - (total - tail);
+        split_part = 0;
+      }
+      if (split_part >= 0) {
+        const int steps = prm.K / BK;
+        const int first = (int)((int64_t)steps * split_part / split_parts), last = (int)((int64_t)steps * (split_part + 1) / split_parts);
+        k_begin = (int64_t)first * BK;
+        k_len = (last - first) * BK;
+      }
+    }
     if (pid >= total) return;
     const int per_xcd = total / kXcds;
     if (pid < per_xcd * kXcds) pid = (pid % kXcds) * per_xcd + pid / kXcds;
     grouped_order(pid, live_m, prm.n_tiles, mt, nt);
     expert = prm.tile_expert[mt];
-    k_len = prm.K;
   }
   const int64_t m0 = (int64_t)mt * BM;
   int64_t valid_end = 0;  // forward modes: first pad row of this expert's segment
@@ -127,13 +154,18 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
     if (tid < BM && m0 + tid < valid_end) scatter_row = prm.row_slot[m0 + tid];
   }
 
+  // One wave per SIMD (WGM == 2): nothing zeroes the accumulators; the first slice of the tile multiplies with the
+  // constant 0 as its third operand (run_acc_first). A tile without K steps (an expert without rows, weight gradients)
+  // zeroes them where it finds that out.
   f32x4 acc[MI][NI];
+  if constexpr (WGM != 2) {
 #pragma unroll
-  for (int i = 0; i < MI; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int j = 0; j < NI; ++j)
+      for (int j = 0; j < NI; ++j)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+        for (int r = 0; r < 4; ++r) acc[i][j][r] = 0.f;
+  }
 
   // ---- global -> LDS addressing: lane l of a wave-load fills slot l (16 bytes) of 64 consecutive slots = 8 rows of 128 B;
   // the lane fetches the chunk that belongs in its slot, so the 8 lanes of a row read one whole line of global memory
@@ -147,6 +179,8 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   if constexpr (AT) {
     a_base += k_begin * prm.lda * 2;
     b_base += k_begin * prm.ldw * 2;
+  } else if constexpr (BT) {
+    b_base += k_begin * prm.ldw * 2;  // a part of a split contraction starts further down the contraction rows
   }
   if constexpr (MODE != kDw) {
     if (prm.a_gather_div <= 0) a_base += m0 * prm.lda * 2;
@@ -157,6 +191,18 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   // window position swap02(q) ^ tr_swz(n) of the row
   auto tr_swz = [](int n) { return (n & 3) | (((n >> 3) & 1) << 2); };
   uint32_t a_off[A_LD], b_off[B_LD];
+  // gathered input: the row_slot entries of this lane's A_LD tile rows, fetched together (one wait, not one per load)
+  // into the registers that then take the offsets
+  if constexpr (!AT && MODE != kDw) {
+    if (prm.a_gather_div > 0) {
+#pragma unroll
+      for (int t = 0; t < A_LD; ++t) {
+        int64_t p = m0 + (wave * A_LD + t) * 8 + (lane >> 3);
+        if (p >= valid_end) p = valid_end - 1;
+        a_off[t] = (uint32_t)prm.row_slot[p];
+      }
+    }
+  }
 #pragma unroll
   for (int t = 0; t < A_LD; ++t) {
     if constexpr (AT) {
@@ -177,7 +223,7 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
         if (p >= valid_end) p = valid_end - 1;  // pad rows re-read a valid row; their results are never stored
         // grouped input: offsets are taken from the tile's first row (a_base is moved there below), so that only a tile,
         // not the whole operand, has to fit 32-bit offsets; gathered input: from the start of the token-order tensor
-        row = prm.a_gather_div > 0 ? (int64_t)(prm.row_slot[p] / prm.a_gather_div) : p - m0;
+        row = prm.a_gather_div > 0 ? (int64_t)((int32_t)a_off[t] / prm.a_gather_div) : p - m0;
       }
       a_off[t] = (uint32_t)((row * prm.lda + k_begin) * 2 + c * 16);
     }
@@ -242,53 +288,6 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
 #pragma unroll
     for (int g = 0; g < kLoadsPerStep; ++g) issue_one(step, g);
   };
-  // L2 warm-up (measurement switch): lane l asks for 4 bytes of line l of the 64 lines of each operand that this wave's
-  // loads of a later step will fetch, so that those loads find their lines in L2 (27 % of them miss otherwise)
-  uint32_t pf_a = 0, pf_b = 0, pf_d0 = 0, pf_d1 = 0;
-  if constexpr (CK_L2_PREFETCH > 0) {
-    if constexpr (AT) {
-      const int n = wave * 16 + (lane >> 2);
-      int64_t col = m0 + (lane & 3) * 64;
-      if (col >= prm.M) col = m0;
-      pf_a = (uint32_t)(((int64_t)n * prm.lda + col) * 2);
-    } else {
-      const int r = wave * 64 + lane;
-      int64_t row;
-      if constexpr (MODE == kDw) {
-        row = min(m0 + r, (int64_t)prm.M - 1);
-      } else {
-        int64_t p = m0 + r;
-        if (p >= valid_end) p = valid_end - 1;
-        row = prm.a_gather_div > 0 ? (int64_t)(prm.row_slot[p] / prm.a_gather_div) : p - m0;
-      }
-      pf_a = (uint32_t)((row * prm.lda + k_begin) * 2);
-    }
-    if constexpr (BT) {
-      const int n = wave * 16 + (lane >> 2);
-      int64_t col = (int64_t)nt * BN + (lane & 3) * 64;
-      if (col >= prm.N) col = (int64_t)nt * BN;
-      pf_b = (uint32_t)(((int64_t)n * prm.ldw + col) * 2);
-    } else {
-      const int j = wave * 64 + lane;
-      int64_t n;
-      if constexpr (MODE == kSwiglu) {
-        const int half = (j % WN) / (WN / 2);
-        const int within = (j / WN) * (WN / 2) + (j % (WN / 2));
-        n = (int64_t)half * prm.I + min((int64_t)nt * (BN / 2) + within, (int64_t)prm.I - 1);
-      } else {
-        n = min((int64_t)nt * BN + j, (int64_t)prm.N - 1);
-      }
-      pf_b = (uint32_t)((n * prm.ldw + k_begin) * 2);
-    }
-  }
-  // the destination registers stay allocated for the whole loop ("+v"): a load may land long after it was issued
-  auto warm_l2 = [&](int step) {
-    const int64_t kb = (int64_t)step * kRowBytes;
-    const int64_t kb_b = BT ? (int64_t)step * BK * prm.ldw * 2 : kb;
-    const int64_t kb_a = AT ? (int64_t)step * BK * prm.lda * 2 : kb;
-    asm volatile("global_load_dword %0, %1, %2" : "+v"(pf_d0) : "v"(pf_a), "s"(a_base_u + kb_a));
-    asm volatile("global_load_dword %0, %1, %2" : "+v"(pf_d1) : "v"(pf_b), "s"(b_base_u + kb_b));
-  };
 
   // ---- fragments: slice sl of a row is its 16-byte chunks 4 sl + lane / 16 (the lane's 8 contraction values)
   typedef typename Mfma16<T>::frag frag_t;
@@ -352,13 +351,15 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
       fb[set][j] = *reinterpret_cast<const frag_t*>(lds_c + stage * kStageBytes + slice_off[sl] + fb_row + j * 16 * kRowBytes);
     }
   };
-  auto mfma = [&](int set, int i, int j) {
+  auto mfma = [&](int set, int i, int j, auto first) {
     if constexpr ((CK_ABLATE & 64) != 0) {
       asm volatile("" ::"v"(fa[set][i]), "v"(fb[set][j]));
+      if constexpr (decltype(first)::value && WGM == 2) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
       return;
     }
     // weight fragment first: a lane gets 4 consecutive output columns of one row
-    if constexpr (WGM == 2) Mfma16<T>::run_acc(fb[set][j], fa[set][i], acc[i][j]);
+    if constexpr (WGM == 2 && decltype(first)::value) Mfma16<T>::run_acc_first(fb[set][j], fa[set][i], acc[i][j]);
+    else if constexpr (WGM == 2) Mfma16<T>::run_acc(fb[set][j], fa[set][i], acc[i][j]);
     else acc[i][j] = Mfma16<T>::run(fb[set][j], fa[set][i], acc[i][j]);
   };
 
@@ -416,7 +417,7 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
     //   every kLoadGap MFMAs. Phase 1 is step nk - 2 (nothing left to fetch), phase 2 the last step (nothing to wait
     //   for, nothing to reload).
     constexpr int kLoadGap = CK_LOAD_GAP > 0 ? CK_LOAD_GAP : (MI * NI) / kLoadsPerStep;
-    auto slice = [&](int kt, auto sl, auto phase, auto idle) {
+    auto slice = [&](int kt, auto sl, auto phase, auto idle, auto first) {
       constexpr bool kIdle = decltype(idle)::value;  // this wave's rows are all pad rows: no fragments, no MFMAs
       constexpr bool kLast = decltype(sl)::value == KS - 1;
       constexpr int kPhase = decltype(phase)::value;
@@ -441,17 +442,14 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
           st_bar += t2 - t1;
           st_s0 += t0 - st_mark;  // slice 0 of this step (the slice in front of the wait)
           st_mark = t2;
-        } else if constexpr (CK_L2_PREFETCH > 0 && kPhase == 0) {
-          asm volatile("s_waitcnt vmcnt(2) lgkmcnt(0)\n\ts_barrier" ::: "memory");  // all but this step's two warm-up loads
         } else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       }
       constexpr int cur = kDouble ? (decltype(sl)::value & 1) : 0;
       constexpr int nxt = kDouble ? (cur ^ 1) : 0;
-      if constexpr (CK_L2_PREFETCH > 0 && decltype(sl)::value == 0 && kPhase == 0) warm_l2(min(kt + CK_L2_PREFETCH, nk - 1));
 #pragma unroll
       for (int n = 0; n < MI * NI; ++n) {
         const int i = n / NI, j = n % NI;
-        if constexpr (!kIdle) mfma(cur, i, j);
+        if constexpr (!kIdle) mfma(cur, i, j, first);
         if constexpr (kLast && kPhase == 0 && !(CK_ABLATE & 2)) {
           if (n % kLoadGap == 0 && n / kLoadGap < kLoadsPerStep) issue_one(kt + 2, n / kLoadGap);
         }
@@ -474,20 +472,38 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
         st_mark = t3;
       }
     };
+    // The first slice of the tile is peeled (its MFMAs start the accumulators); the loop body is the second slice of step
+    // kt followed by the first slice of step kt + 1 (the first slice of a step does not depend on the phase).
     auto k_loop = [&](auto idle) {
-      auto k_step = [&](int kt, auto phase) { static_for<KS>([&](auto sl) { slice(kt, sl, phase, idle); }); };
+      constexpr std::integral_constant<int, 0> s0{}, p0{};
+      constexpr std::integral_constant<int, 1> s1{}, p1{};
+      constexpr std::integral_constant<int, 2> p2{};
+      if constexpr (WGM == 2) slice(0, s0, p0, idle, std::true_type{});
+      else slice(0, s0, p0, idle, std::false_type{});
       int kt = 0;
-      for (; kt + 2 < nk; ++kt) k_step(kt, std::integral_constant<int, 0>{});
-      if (kt + 2 == nk) k_step(kt++, std::integral_constant<int, 1>{});
-      k_step(kt, std::integral_constant<int, 2>{});
+      for (; kt + 2 < nk; ++kt) {
+        slice(kt, s1, p0, idle, std::false_type{});
+        slice(kt + 1, s0, p0, idle, std::false_type{});
+      }
+      if (kt + 2 == nk) {
+        slice(kt, s1, p1, idle, std::false_type{});
+        slice(kt + 1, s0, p0, idle, std::false_type{});
+        ++kt;
+      }
+      slice(kt, s1, p2, idle, std::false_type{});
     };
     // A wave whose tile rows all lie past the expert's last row (the tile is the ragged end of a segment) still issues
     // its share of the loads and meets every barrier, but multiplies nothing: the wave it shares a SIMD with then has
-    // the matrix pipe to itself. Its accumulators stay zero and its rows are never stored.
+    // the matrix pipe to itself. Its accumulators hold nothing meaningful and its rows are never stored.
     bool wave_idle = false;
     if constexpr (MODE != kDw) wave_idle = m0 + wm * WM >= valid_end;
     if (__builtin_amdgcn_readfirstlane(wave_idle)) k_loop(std::true_type{});
     else k_loop(std::false_type{});
+  } else if constexpr (WGM == 2 && MODE == kDw) {  // only a weight-gradient tile can have no K step (the host requires K >= 64)
+#pragma unroll
+    for (int i = 0; i < MI; ++i)
+#pragma unroll
+      for (int j = 0; j < NI; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
   }
 
   // ---- epilogue, straight from the accumulators. The weight fragment is the MFMA's first operand, so a lane holds, per
@@ -500,6 +516,39 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   // Plain (cached) stores: L2 merges the two 64-byte halves of an output line before it leaves for memory (measured
   // against non-temporal stores: 3 % faster launches at K = 4096).
   if constexpr (WGM == 2) mfma_drain();
+  if constexpr (kSplit) {
+    if (split_part >= 0) {
+      // every part leaves its accumulators in the workspace, in its own register layout (16 bytes per lane)
+      float* slot_ws = prm.split_ws + (int64_t)split_slot * split_parts * kSplitPartFloats;
+      float* mine = slot_ws + (int64_t)split_part * kSplitPartFloats + ((int64_t)wave * MI * NI * kWave + lane) * 4;
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) *reinterpret_cast<f32x4*>(mine + (i * NI + j) * kWave * 4) = acc[i][j];
+      int* counters = reinterpret_cast<int*>(prm.split_ws + (int64_t)kSplitMaxTail * kSplitParts * kSplitPartFloats);
+      int* flag = reinterpret_cast<int*>(lds_c);  // the stages are dead
+      __threadfence();  // the partial tile is visible device-wide before the ticket is taken
+      __syncthreads();
+      if (tid == 0) *flag = atomicAdd(&counters[split_slot], 1);
+      __syncthreads();
+      const bool last = *flag == split_parts - 1;
+      __syncthreads();  // everyone has read the flag before the epilogue reuses LDS
+      if (!last) return;
+      __threadfence();  // the other parts' tiles are read from memory, not from a stale cache line
+      if (tid == 0) counters[split_slot] = 0;  // zero again for the next launch
+      const float* theirs = slot_ws + ((int64_t)wave * MI * NI * kWave + lane) * 4;
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) {  // a fixed order of additions whichever part arrived last
+          const float* q = theirs + (i * NI + j) * kWave * 4;
+          f32x4 sum = *reinterpret_cast<const f32x4*>(q) + *reinterpret_cast<const f32x4*>(q + kSplitPartFloats);
+          if (split_parts > 2) sum += *reinterpret_cast<const f32x4*>(q + 2 * kSplitPartFloats);
+          if (split_parts > 3) sum += *reinterpret_cast<const f32x4*>(q + 3 * kSplitPartFloats);
+          acc[i][j] = sum;
+        }
+    }
+  }
   if constexpr (CK_STAMP != 0) st_end = clock64();
   if constexpr ((CK_ABLATE & 32) != 0) {
     float keep = 0.f;
@@ -795,7 +844,14 @@ int launch_bn(const GemmParams& prm, int mode, bool bt, unsigned blocks, hipStre
 
 int launch_line(const GemmParams& prm_in, int mode, int bn, bool bt, int dtype, unsigned blocks, hipStream_t stream,
                 const char* name) {
-  const GemmParams& prm = prm_in;
+  GemmParams prm = prm_in;
+  if (prm.split_ws != nullptr && (mode == kGrouped || mode == kScatter)) {
+    prm.split_base = (int)blocks;  // the extra workgroups of a split last round sit behind the regular grid
+    blocks += kSplitMaxTail * (kSplitParts - 1);
+  } else {
+    prm.split_ws = nullptr;
+    prm.split_base = 0x7fffffff;
+  }
   CK_DISPATCH_HALF(dtype, name, { return launch_bn<scalar_t, 256, 2>(prm, mode, bt, blocks, stream, name); });
   return CK_ERR_ARG;
 }

@@ -70,6 +70,15 @@ _SIGNATURES = {
         c_int32,
         [c_void_p, c_int32, c_void_p, c_int32, c_int32, POINTER(ck_segments), c_int32, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int32, c_void_p],
     ),
+    "ck_grouped_gemm_workspace_bytes": (c_int64, []),
+    "ck_grouped_gemm_ws": (
+        c_int32,
+        [c_void_p, c_int32, c_void_p, c_int32, c_int32, POINTER(ck_segments), c_int32, c_void_p, c_void_p, c_int64, c_void_p, c_void_p, c_int32, c_void_p, c_void_p, c_int64],
+    ),
+    "ck_grouped_gemm_nn_ws": (
+        c_int32,
+        [c_void_p, c_void_p, c_int32, c_int32, POINTER(ck_segments), c_int32, c_void_p, c_int32, c_void_p, c_void_p, c_int64],
+    ),
     "ck_grouped_gemm_nn": (c_int32, [c_void_p, c_void_p, c_int32, c_int32, POINTER(ck_segments), c_int32, c_void_p, c_int32, c_void_p]),
     "ck_grouped_gemm_dw": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_int32, POINTER(ck_segments), c_void_p, c_int32, c_void_p]),
     "ck_grouped_gemm_dw_rows": (c_int32, [c_void_p, c_void_p, c_int32, c_int32, POINTER(ck_segments), c_void_p, c_int32, c_void_p]),

@@ -256,6 +256,24 @@ _EPILOGUE_NAMES = {
 }
 
 
+_split_workspaces: dict = {}
+
+
+def _split_workspace(device: torch.device) -> torch.Tensor:
+    """Workspace of ck_grouped_gemm_ws / ck_grouped_gemm_nn_ws (split last round of tiles): one zero-initialised buffer
+    per device and stream (the kernels leave its counters zero; two streams must not share one). CK_GEMM_SPLIT=0 in the
+    environment switches the split off (measurement knob)."""
+    import os
+
+    if os.environ.get("CK_GEMM_SPLIT", "1") == "0":
+        return None
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    ws = _split_workspaces.get(key)
+    if ws is None:
+        ws = _split_workspaces[key] = torch.zeros(_C.lib().ck_grouped_gemm_workspace_bytes(), dtype=torch.uint8, device=device)
+    return ws
+
+
 def _gemm_f32(a, gather_div, w, w_is_kn: bool, N: int, K: int, seg: ExpertSegments, scatter: bool, y, bias=None):
     """The grouped GEMMs of fp32 tensors (fp32 MFMA; see ck_grouped_gemm_f32)."""
     cs = seg.c_struct()
@@ -280,10 +298,11 @@ def _gemm(a, gather_div, w, seg: ExpertSegments, epilogue, y, y_t=None, aux=None
 
     def launch():
         with torch.cuda.device(w.device):
+            ws = _split_workspace(w.device) if epilogue in (_C.CK_EPI_GROUPED, _C.CK_EPI_SCATTER) else None
             _C.check(
-                _C.lib().ck_grouped_gemm(
+                _C.lib().ck_grouped_gemm_ws(
                     _C.ptr(a), gather_div, _C.ptr(w), N, K, ctypes.byref(cs), epilogue, _C.ptr(y), _C.ptr(y_t), seg.ld_t,
-                    _C.ptr(aux), _C.ptr(aux_in), _C.dtype_code(w.dtype), _C.stream(),
+                    _C.ptr(aux), _C.ptr(aux_in), _C.dtype_code(w.dtype), _C.stream(), _C.ptr(ws), 0 if ws is None else ws.numel(),
                 )
             )
 
@@ -320,10 +339,11 @@ def _gemm_dx(d_y, w, seg: ExpertSegments, epilogue, out):
 
         def launch():
             with torch.cuda.device(w.device):
+                ws = _split_workspace(w.device)
                 _C.check(
-                    _C.lib().ck_grouped_gemm_nn(
+                    _C.lib().ck_grouped_gemm_nn_ws(
                         _C.ptr(d_y), _C.ptr(w), n_in, n_out, ctypes.byref(cs), epilogue, _C.ptr(out), _C.dtype_code(w.dtype),
-                        _C.stream(),
+                        _C.stream(), _C.ptr(ws), 0 if ws is None else ws.numel(),
                     )
                 )
 

@@ -196,6 +196,20 @@ typedef struct ck_segments {
 int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* w, int32_t N, int32_t K,
                     const ck_segments* seg, int32_t epilogue, void* y, void* y_t, int64_t ld_t, void* aux,
                     const void* aux_in, int32_t dtype, void* stream);
+/* The same call with a workspace that lets the kernel split the contraction of its last, partial round of tiles. A
+ * launch of t tiles runs in ceil(t / 256) rounds on the 256 CUs; when the last round is at most half full (and the
+ * launch has at most 16 rounds and at least 32 K steps of 64), each of its tiles is computed by two to four workgroups (as
+ * many as fill the chip), an equal share of the contraction each, which exchange fp32 partial tiles through the workspace; the last to arrive adds them in a
+ * fixed order (results do not depend on arrival order) and runs the epilogue. Grouped and scatter epilogues of the
+ * 256-row-tile kernel; every other case behaves like ck_grouped_gemm. No counterpart in the reference (its launches
+ * are not tile-quantised the same way).
+ * workspace: ck_grouped_gemm_workspace_bytes() bytes, 16-byte aligned; its last 512 bytes (arrival counters) must be zero
+ * before the first call and are zero again after every call, so one zero-initialised buffer per stream is reusable.
+ * workspace NULL or too small: never split. */
+int64_t ck_grouped_gemm_workspace_bytes(void);
+int ck_grouped_gemm_ws(const void* a, int32_t a_gather_div, const void* w, int32_t N, int32_t K,
+                       const ck_segments* seg, int32_t epilogue, void* y, void* y_t, int64_t ld_t, void* aux,
+                       const void* aux_in, int32_t dtype, void* stream, void* workspace, int64_t workspace_bytes);
 /* Input-gradient form of the grouped GEMM: y[p, :] = a[p, :] @ w[e(p)] with w [E, K, N] row-major, i.e. the weight
  * exactly as the forward pass stores it ([E, out, in] = [E, K, N] here: K = the forward's out, N = its in), read
  * contraction-strided instead of through a transposed copy.
@@ -205,6 +219,10 @@ int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* w, int32_t 
  * Needs seg->align == 256, K % 64 == 0, N % 8 == 0. */
 int ck_grouped_gemm_nn(const void* a, const void* w, int32_t N, int32_t K, const ck_segments* seg, int32_t epilogue,
                        void* y, int32_t dtype, void* stream);
+
+/* ck_grouped_gemm_nn with the workspace of ck_grouped_gemm_ws (same rules). */
+int ck_grouped_gemm_nn_ws(const void* a, const void* w, int32_t N, int32_t K, const ck_segments* seg, int32_t epilogue,
+                          void* y, int32_t dtype, void* stream, void* workspace, int64_t workspace_bytes);
 
 /* The same grouped GEMMs for fp32 tensors (the dtype of the reference's test grid, tests/test_commons.py:26-27): fp32
  * products and fp32 accumulation on v_mfma_f32_32x32x2_f32 (the reference's Triton kernels round fp32 operands to TF32,

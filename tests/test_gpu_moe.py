@@ -93,6 +93,57 @@ def test_grouped_gemm_grouped_in_scatter_out(device, dtype, align, K, N, gemm_ti
     torch.testing.assert_close(y.float().cpu(), expect, rtol=RTOL, atol=ATOL)
 
 
+@pytest.mark.parametrize("N", [5120, 6400, 7168])  # 13 row tiles x 20 / 25 / 28 column tiles: last round 4 / 69 / 108 tiles (4 / 3 / 2 parts)
+@pytest.mark.parametrize("form", ["nt_grouped", "nt_scatter", "nn_grouped", "nn_scatter"])
+def test_grouped_gemm_split_last_round(device, monkeypatch, form, N):
+    """A launch whose last round of tiles is at most a quarter full computes those tiles in four parts of the contraction
+    (ck_grouped_gemm_ws / ck_grouped_gemm_nn_ws with a workspace). Against the same launch without the workspace
+    (CK_GEMM_SPLIT=0): equal up to the fp32 re-association of four partial sums (rtol = atol = 1e-2, and at least 99 % of
+    the elements bit-equal); two split launches in a row are bit-identical (fixed order of additions) and leave the
+    counters zero; against the fp32 reference at the GEMM tolerance."""
+    T, k, E, align = 1400, 2, 6, 256
+    K = 2048
+    g, seg = _make_case(device, torch.bfloat16, T, k, E, align, empty=(3,), seed=11)
+    live_tiles = int(seg.seg_starts[E]) // align * (N // 256)
+    assert 0 < live_tiles % 256 <= 128 and live_tiles // 256 <= 16, live_tiles  # the split applies to this launch
+    scatter = form.endswith("scatter")
+    rows_out = T * k if scatter else seg.max_rows
+    epi = _C.CK_EPI_SCATTER if scatter else _C.CK_EPI_GROUPED
+    if form.startswith("nt"):
+        a = torch.randn(T, K, generator=g).to(torch.bfloat16).to(device)
+        w = (torch.randn(E, N, K, generator=g) * K**-0.5).to(torch.bfloat16).to(device)
+        run = lambda out: scattermoe._gemm(a, k, w, seg, epi, out)
+    else:
+        a = torch.randn(seg.max_rows, K, generator=g).to(torch.bfloat16).to(device)
+        w = (torch.randn(E, K, N, generator=g) * K**-0.5).to(torch.bfloat16).to(device)  # [E, out = K here, in = N]
+        run = lambda out: scattermoe._gemm_dx(a, w, seg, epi, out)
+    outs = []
+    for split in ("1", "1", "0"):
+        monkeypatch.setenv("CK_GEMM_SPLIT", split)
+        out = torch.zeros(rows_out, N, dtype=torch.bfloat16, device=device)
+        run(out)
+        outs.append(out)
+    monkeypatch.setenv("CK_GEMM_SPLIT", "1")
+    ws = scattermoe._split_workspace(device)
+    assert int(ws[-512:].sum()) == 0  # arrival counters back at zero
+    assert torch.equal(outs[0], outs[1])
+    torch.testing.assert_close(outs[0].float(), outs[2].float(), rtol=RTOL, atol=ATOL)
+    assert float((outs[0] == outs[2]).float().mean()) > 0.99
+    # fp32 reference on a sample of rows
+    seg_starts, counts, row_slot = _layout(seg)
+    checked = 0
+    for e in range(E):
+        s_, c_ = int(seg_starts[e]), int(counts[e])
+        for p in list(range(s_, s_ + c_))[:: max(1, c_ // 5)][:6]:
+            slot = int(row_slot[p])
+            src = a[slot // k] if form.startswith("nt") else a[p]
+            want = (src.float() @ (w[e].float().t() if form.startswith("nt") else w[e].float())).cpu()
+            got = outs[0][slot if scatter else p].float().cpu()
+            torch.testing.assert_close(got, want, rtol=RTOL, atol=ATOL)
+            checked += 1
+    assert checked > 10
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("with_bias", [False, True])
 @pytest.mark.parametrize("align,K,N", [(128, 200, 136), (256, 64, 128), (256, 576, 264), (256, 192, 840)])
