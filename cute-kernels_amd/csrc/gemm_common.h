@@ -47,7 +47,7 @@ struct GemmParams {
   float* split_ws;
   int split_base;
 };
-constexpr int kSplitParts = 4, kSplitMaxTail = 64, kSplitMaxRounds = 16, kSplitMinSteps = 32;
+constexpr int kSplitParts = 4, kSplitMaxTail = 64, kSplitMaxRounds = 64, kSplitMinSteps = 16;
 constexpr int64_t kSplitPartFloats = 4 * 64 * 64 * 4;  // one workgroup's 256 x 256 fp32 tile
 constexpr int64_t kSplitWorkspaceBytes = kSplitMaxTail * kSplitParts * kSplitPartFloats * 4 + 2 * kSplitMaxTail * 4;
 

@@ -198,7 +198,7 @@ int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* w, int32_t 
                     const void* aux_in, int32_t dtype, void* stream);
 /* The same call with a workspace that lets the kernel split the contraction of its last, partial round of tiles. A
  * launch of t tiles runs in ceil(t / 256) rounds on the 256 CUs; when the last round is at most half full (and the
- * launch has at most 16 rounds and at least 32 K steps of 64), each of its tiles is computed by two to four workgroups (as
+ * launch has at most 64 rounds and at least 16 K steps of 64), each of its tiles is computed by two to four workgroups (as
  * many as fill the chip), an equal share of the contraction each, which exchange fp32 partial tiles through the workspace; the last to arrive adds them in a
  * fixed order (results do not depend on arrival order) and runs the epilogue. Grouped and scatter epilogues of the
  * 256-row-tile kernel; every other case behaves like ck_grouped_gemm. No counterpart in the reference (its launches
