@@ -30,11 +30,11 @@ PEAK_HBM_GBS = 8000.0  # MI355X HBM3E
 # this same command, FETCH_SIZE scaled x2.0 and WRITE_SIZE x1.0 against a 1 GiB device copy (known size);
 # summary and commands: profiles/grouped_gemm_c3_moe_fwd_bwd.md. Not measurable from inside this process.
 TRAFFIC_BYTES_PER_LAUNCH = {
-    "grouped_gemm_dw_rows": 2 * 5.930e6 * 1024 + 1.376e6 * 1024,  # both weight gradients, row-major operands
-    "grouped_gemm<swiglu>": 2 * 7.045e6 * 1024 + 2.753e6 * 1024,  # c_fc forward
-    "grouped_gemm_nn<scatter>": 2 * 8.243e6 * 1024 + 2.621e5 * 1024,  # c_fc dX, contraction-strided weights
-    "grouped_gemm_nn<grouped>": 2 * 3.723e6 * 1024 + 9.175e5 * 1024,  # c_proj dX, contraction-strided weights
-    "grouped_gemm<scatter>": 2 * 3.905e6 * 1024 + 2.621e5 * 1024,  # c_proj forward
+    "grouped_gemm_dw_rows": 2 * 5.951e6 * 1024 + 1.376e6 * 1024,  # both weight gradients, row-major operands
+    "grouped_gemm<swiglu>": 2 * 7.674e6 * 1024 + 2.782e6 * 1024,  # c_fc forward
+    "grouped_gemm_nn<scatter>": 2 * 8.342e6 * 1024 + 3.282e5 * 1024,  # c_fc dX, contraction-strided weights
+    "grouped_gemm_nn<grouped>": 2 * 4.002e6 * 1024 + 9.571e5 * 1024,  # c_proj dX, contraction-strided weights
+    "grouped_gemm<scatter>": 2 * 3.993e6 * 1024 + 3.259e5 * 1024,  # c_proj forward
 }
 
 # the kernel instantiation each launch name runs at this workload, as rocprofv3's kernel trace spells it
