@@ -71,21 +71,30 @@ __global__ __launch_bounds__(kBlock) void route_topk_softmax_kernel(const T* __r
 }
 
 // d_values = g * (d_g - sum_i g_i d_g_i); scattered into an otherwise zero row of d_logits. One group of G lanes per token.
+// d_gates_rounded (optional): the gradient as it arrived in the 16-bit type. Where it is d_gates rounded to that type,
+// the unrounded d_gates is used, elsewhere (something scaled or replaced the gradient on its way) the value that arrived.
 template <typename T>
 __global__ __launch_bounds__(kBlock) void route_bwd_kernel(const float* __restrict__ gates, const float* __restrict__ d_gates,
+                                                            const T* __restrict__ d_gates_rounded,
                                                             const int32_t* __restrict__ selected, int64_t T_tokens, int E,
                                                             int k, T* __restrict__ d_logits) {
   const int64_t token = (int64_t)blockIdx.x * (kBlock / kWave) + threadIdx.x / kWave;
   if (token >= T_tokens) return;
   const int lane = threadIdx.x & (kWave - 1);
+  auto d_gate = [&](int j) {
+    const float exact = d_gates[token * k + j];
+    if (d_gates_rounded == nullptr) return exact;
+    const float arrived = Elem<T>::up(d_gates_rounded[token * k + j]);
+    return Elem<T>::up(Elem<T>::down(exact)) == arrived ? exact : arrived;
+  };
   float dot = 0.f;
-  for (int j = 0; j < k; ++j) dot += gates[token * k + j] * d_gates[token * k + j];
+  for (int j = 0; j < k; ++j) dot += gates[token * k + j] * d_gate(j);
   for (int e = lane; e < E; e += kWave) {
     float d = 0.f;
     for (int j = 0; j < k; ++j) {
       if (selected[token * k + j] == e) {
         const float g = gates[token * k + j];
-        d += g * (d_gates[token * k + j] - dot);
+        d += g * (d_gate(j) - dot);
       }
     }
     d_logits[token * (int64_t)E + e] = Elem<T>::down(d);
@@ -128,18 +137,33 @@ extern "C" int ck_route_topk_softmax(const void* logits, int32_t dtype, int64_t 
   return CK_OK;
 }
 
-extern "C" int ck_route_topk_softmax_bwd(const float* gates, const float* d_gates, const int32_t* selected, int64_t T,
-                                         int32_t E, int32_t k, void* d_logits, int32_t dtype, void* stream) {
-  CK_REQUIRE(E >= 1 && k >= 1 && k <= E && T >= 0, "ck_route_topk_softmax_bwd: bad sizes T=%lld E=%d k=%d",
-             (long long)T, E, k);
+static int route_bwd_impl(const char* name, const float* gates, const float* d_gates, const void* d_gates_rounded,
+                          const int32_t* selected, int64_t T, int32_t E, int32_t k, void* d_logits, int32_t dtype,
+                          void* stream) {
+  CK_REQUIRE(E >= 1 && k >= 1 && k <= E && T >= 0, "%s: bad sizes T=%lld E=%d k=%d", name, (long long)T, E, k);
   if (T == 0) return CK_OK;
-  CK_REQUIRE(gates && d_gates && selected && d_logits, "ck_route_topk_softmax_bwd: NULL argument");
+  CK_REQUIRE(gates && d_gates && selected && d_logits, "%s: NULL argument", name);
   const int64_t blocks = ceil_div(T, kBlock / kWave);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  CK_DISPATCH_FLOAT(dtype, "ck_route_topk_softmax_bwd", {
+  CK_DISPATCH_FLOAT(dtype, name, {
     hipLaunchKernelGGL((route_bwd_kernel<scalar_t>), dim3((unsigned)blocks), dim3(kBlock), 0, s, gates, d_gates,
-                       selected, T, (int)E, (int)k, static_cast<scalar_t*>(d_logits));
+                       static_cast<const scalar_t*>(d_gates_rounded), selected, T, (int)E, (int)k,
+                       static_cast<scalar_t*>(d_logits));
   });
-  CK_CHECK_LAUNCH("ck_route_topk_softmax_bwd");
+  CK_CHECK_LAUNCH(name);
   return CK_OK;
+}
+
+extern "C" int ck_route_topk_softmax_bwd(const float* gates, const float* d_gates, const int32_t* selected, int64_t T,
+                                         int32_t E, int32_t k, void* d_logits, int32_t dtype, void* stream) {
+  return route_bwd_impl("ck_route_topk_softmax_bwd", gates, d_gates, nullptr, selected, T, E, k, d_logits, dtype, stream);
+}
+
+extern "C" int ck_route_topk_softmax_bwd_exact(const float* gates, const float* d_gates_exact, const void* d_gates,
+                                               const int32_t* selected, int64_t T, int32_t E, int32_t k, void* d_logits,
+                                               int32_t dtype, void* stream) {
+  const char* name = "ck_route_topk_softmax_bwd_exact";
+  CK_REQUIRE(T == 0 || d_gates != nullptr, "%s: d_gates is required", name);
+  CK_REQUIRE(dtype != CK_F32, "%s: d_gates of a 16-bit type (fp32 gradients go to ck_route_topk_softmax_bwd)", name);
+  return route_bwd_impl(name, gates, d_gates_exact, d_gates, selected, T, E, k, d_logits, dtype, stream);
 }

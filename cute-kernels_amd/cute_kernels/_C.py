@@ -51,6 +51,7 @@ _SIGNATURES = {
     "ck_count_offsets_static": (c_int32, [c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ck_route_topk_softmax": (c_int32, [c_void_p, c_int32, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ck_route_topk_softmax_bwd": (c_int32, [c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_void_p, c_int32, c_void_p]),
+    "ck_route_topk_softmax_bwd_exact": (c_int32, [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int32, c_int32, c_void_p, c_int32, c_void_p]),
     "ck_sort_max_rows": (c_int64, [c_int64, c_int32, c_int32]),
     "ck_sort_workspace_words": (c_int64, [c_int64, c_int32]),
     "ck_sort_by_expert": (c_int32, [c_void_p, c_int32, c_int64, c_int32, c_int32] + [c_void_p] * 10),

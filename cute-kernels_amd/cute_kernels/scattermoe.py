@@ -69,14 +69,22 @@ class _RouteTopKSoftmax(torch.autograd.Function):
         gates, selected = ctx.saved_tensors
         T, k = gates.shape
         exact = ctx.slot.d_gates_f32 if ctx.slot is not None else None
-        if exact is not None and exact.shape == d_gates.shape and d_gates.dtype != torch.float32:
-            # the unrounded gradient, if what arrived is that tensor rounded (decided on the device: no host sync)
-            same = (exact.to(d_gates.dtype) == d_gates).all()
-            d_gates = torch.where(same, exact, d_gates.float())
-            ctx.slot.d_gates_f32 = None
-        d_gates = d_gates.float().contiguous()
         d_logits = torch.empty(T, ctx.E, dtype=ctx.dtype, device=gates.device)
         lib = _C.lib()
+        if exact is not None and exact.shape == d_gates.shape and d_gates.dtype == ctx.dtype != torch.float32:
+            # the unrounded gradient wherever what arrived is that gradient rounded (decided per element inside the
+            # kernel: no host sync, no extra launches)
+            ctx.slot.d_gates_f32 = None
+            d_gates = d_gates.contiguous()
+            with torch.cuda.device(gates.device):
+                _C.check(
+                    lib.ck_route_topk_softmax_bwd_exact(
+                        _C.ptr(gates), _C.ptr(exact), _C.ptr(d_gates), _C.ptr(selected), T, ctx.E, k, _C.ptr(d_logits),
+                        _C.dtype_code(ctx.dtype), _C.stream(),
+                    )
+                )
+            return d_logits, None, None, None
+        d_gates = d_gates.float().contiguous()
         with torch.cuda.device(gates.device):
             _C.check(
                 lib.ck_route_topk_softmax_bwd(

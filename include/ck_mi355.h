@@ -75,6 +75,14 @@ int ck_route_topk_softmax(const void* logits, int32_t dtype, int64_t T, int32_t 
  * d_gates [T, k] fp32. */
 int ck_route_topk_softmax_bwd(const float* gates, const float* d_gates, const int32_t* selected, int64_t T,
                               int32_t E, int32_t k, void* d_logits, int32_t dtype, void* stream);
+/* The same when the gates left the router in a 16-bit `dtype` and their gradient d_gates [T, k] came back in it, while
+ * the caller also holds that gradient unrounded (d_gates_exact [T, k] fp32, from ck_gate_grad_f32): per element, where
+ * d_gates equals d_gates_exact rounded to `dtype` the unrounded value is used, elsewhere (a hook scaled or replaced the
+ * gradient) the value that arrived. One launch instead of a compare / reduce / select chain in front of the plain entry
+ * point. Follows the same reference lines; the reference itself has only the rounded gradient (ops.py:214). */
+int ck_route_topk_softmax_bwd_exact(const float* gates, const float* d_gates_exact, const void* d_gates,
+                                    const int32_t* selected, int64_t T, int32_t E, int32_t k, void* d_logits,
+                                    int32_t dtype, void* stream);
 
 /* ---------------------------------------------------------------------------------------------------------------
  * (b2) stable sort of (token, slot) pairs by expert + tile-aligned expert segments

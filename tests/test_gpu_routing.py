@@ -126,6 +126,41 @@ def test_route_autograd_matches_torch(device):
     torch.testing.assert_close(a.grad.cpu(), b.grad, rtol=1e-5, atol=1e-7)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_route_backward_takes_the_unrounded_gate_gradient_where_it_arrived_rounded(device, dtype):
+    """ck_route_topk_softmax_bwd_exact against ck_route_topk_softmax_bwd fed with the gradient it has to pick: the fp32
+    d_gates where the 16-bit gradient that arrived is that value rounded, the arrived value elsewhere (here every third
+    row was doubled on its way, as a hook on the gates would). Bit-exact: same kernel arithmetic on the same inputs."""
+    from cute_kernels import _C
+
+    T, E, k = 777, 24, 4
+    g = torch.Generator().manual_seed(5)
+    logits = torch.randn(T, E, generator=g).to(dtype).to(device)
+    sel, gates, _ = cute_kernels.route_topk_softmax_raw(logits, k)
+    exact = torch.randn(T, k, generator=g).to(device)
+    arrived = exact.to(dtype)
+    arrived[::3] *= 2
+    picked = torch.where(exact.to(dtype) == arrived, exact, arrived.float())
+    assert 0 < int((picked != exact).sum()) < T * k
+    lib = _C.lib()
+    got = torch.full((T, E), 7.0, dtype=dtype, device=device)
+    want = torch.full((T, E), 9.0, dtype=dtype, device=device)
+    with torch.cuda.device(device):
+        _C.check(lib.ck_route_topk_softmax_bwd_exact(_C.ptr(gates), _C.ptr(exact), _C.ptr(arrived), _C.ptr(sel), T, E, k,
+                                                     _C.ptr(got), _C.dtype_code(dtype), _C.stream()))
+        _C.check(lib.ck_route_topk_softmax_bwd(_C.ptr(gates), _C.ptr(picked), _C.ptr(sel), T, E, k, _C.ptr(want),
+                                               _C.dtype_code(dtype), _C.stream()))
+    assert torch.equal(got, want)
+    # against autograd of softmax over the selected logits with the picked gradient
+    v = torch.gather(logits.float(), 1, sel.long()).requires_grad_()
+    torch.softmax(v, -1).backward(picked)
+    ref = torch.zeros(T, E, device=device).scatter_(1, sel.long(), v.grad)
+    torch.testing.assert_close(got.float(), ref, rtol=1e-2, atol=1e-3)
+    rc = lib.ck_route_topk_softmax_bwd_exact(_C.ptr(gates), _C.ptr(exact), _C.ptr(exact), _C.ptr(sel), T, E, k, _C.ptr(got),
+                                             _C.CK_F32, _C.stream())
+    assert rc != 0  # fp32 gradients have nothing to recover
+
+
 def _check_sort(device, ids: torch.Tensor, E: int, align: int):
     seg = cute_kernels.sort_by_expert(ids.to(device), E, align)
     idn = ids.numpy().astype(np.int64)
