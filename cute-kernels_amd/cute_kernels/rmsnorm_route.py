@@ -68,7 +68,7 @@ class _RMSNormRoute(torch.autograd.Function):
         d_total = None if d_y is None else d_y.reshape(-1, H)
         if d_logits is not None:
             if ctx.needs_input_grad[2]:
-                d_gate = d_logits.t() @ y
+                d_gate = _gate_weight_grad(d_logits, y)
             through_router = d_logits @ gate_weight
             d_total = through_router if d_total is None else d_total + through_router
         if d_total is None:
@@ -80,6 +80,19 @@ class _RMSNormRoute(torch.autograd.Function):
 
         d_x, d_norm_weight, _, _ = _RMSNorm_Cute.backward(_Saved, d_total)
         return d_x.view(ctx.shape), d_norm_weight, d_gate, None, None
+
+
+def _gate_weight_grad(d_logits: torch.Tensor, y: torch.Tensor) -> torch.Tensor:
+    """d_logits^T @ y ([E, tokens] x [tokens, H]). The BLAS library runs this skinny product (E rows, a contraction as long
+    as the batch) on a few workgroups; cut into 16 slices of the tokens it is a batched product that fills the chip, and
+    the 16 partial results are added in fp32 (measured on MI355X: 55 -> 27 us at 8,192 x 64 x 2,048, 331 -> 104 us at
+    65,536 x 128 x 4,096)."""
+    tokens, E = d_logits.shape
+    slices = 16
+    if tokens < 4096 or tokens % slices != 0 or not d_logits.is_contiguous() or not y.is_contiguous():
+        return d_logits.t() @ y
+    parts = torch.bmm(d_logits.view(slices, tokens // slices, E).transpose(1, 2), y.view(slices, tokens // slices, -1))
+    return parts.sum(0, dtype=torch.float32).to(y.dtype)
 
 
 def rmsnorm_route_pays(x: torch.Tensor, gate_weight: torch.Tensor) -> bool:
