@@ -326,10 +326,12 @@ def secondary_hbm_kernels(dev):
     return out, configs
 
 
-def gemm_only(dev, launches: int, stamps: bool = False):
+def gemm_only(dev, launches: int, stamps: bool = False, fine: bool = False):
     """Just the c_fc-forward-shape grouped GEMM (grouped epilogue) at the C3 shape: the target of counter runs.
     stamps: with a CK_STAMP measurement build (build.py --define CK_STAMP=1 --output libck_stamp.so, loaded through
-    CK_MI355_LIB), also print where a wave's cycles go: main loop, waiting for loads, waiting at the barrier, epilogue."""
+    CK_MI355_LIB), also print where a wave's cycles go: main loop, waiting for loads, waiting at the barrier, epilogue.
+    fine: with a CK_STAMP=3 build, print the cycles per MFMA of each group of 8 MFMAs of a K step's second slice (the
+    last group also holds the bookkeeping additions of the stamps themselves)."""
     import numpy as np
     import torch
 
@@ -347,7 +349,7 @@ def gemm_only(dev, launches: int, stamps: bool = False):
         w.zero_()
     y = torch.empty(seg.max_rows, 2 * I, device=dev, dtype=torch.bfloat16)
     trace = None
-    if stamps:
+    if stamps or fine:
         trace = torch.zeros(8 * 8 * 20000, dtype=torch.int64, device=dev)
         os.environ["CK_TRACE_PTR"] = hex(trace.data_ptr())  # read by the library at every call (stamp builds only)
     for _ in range(2):
@@ -362,7 +364,14 @@ def gemm_only(dev, launches: int, stamps: bool = False):
     flops = 4.0 * R * H * I
     rec = {"kernel": "grouped_gemm<grouped>", "shape": [R, 2 * I, H], "avg_launch_ms": ms,
            "TFLOP/s": flops / ms / 1e9, "frac_mfma": flops / ms / 1e9 / PEAK_BF16_TFLOPS}
-    if trace is not None:
+    if trace is not None and fine:
+        t = trace.view(-1, 8).cpu().numpy().astype(np.float64)
+        t = t[(t != 0).any(1)]
+        assert len(t) > 0, "no stamps: is CK_MI355_LIB a CK_STAMP=3 build?"
+        steps = H // 64 - 2  # the steady-state K steps carry the stamps (not the first, not the last two)
+        rec["second_slice_cycles_per_mfma_by_group_of_8"] = [round(float(v), 2) for v in t.mean(0) / steps / 8]
+        rec["waves"] = int(len(t))
+    elif trace is not None:
         t = trace.view(-1, 8).cpu().numpy().astype(np.float64)
         t = t[t[:, 5] > 0]  # waves that ran a main loop
         assert len(t) > 0, "no stamps: is CK_MI355_LIB a CK_STAMP build?"
@@ -431,6 +440,8 @@ def main() -> int:
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device copy (outside the timed region): the known-size kernel that "
                     "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
+    ap.add_argument("--fine-stamps", action="store_true",
+                    help="with --only-gemm and a CK_STAMP=3 measurement build: cycles per MFMA inside a K step's second slice")
     ap.add_argument("--stamps", action="store_true",
                     help="with --only-gemm and a CK_STAMP measurement build: print the per-wave cycle breakdown")
     ap.add_argument("--only-yardstick", action="store_true",
@@ -448,7 +459,7 @@ def main() -> int:
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     if args.only_gemm > 0:
-        gemm_only(dev, args.only_gemm, args.stamps)
+        gemm_only(dev, args.only_gemm, args.stamps, args.fine_stamps)
         return 0
     if args.only_yardstick:
         print(json.dumps({"library_gemm_yardstick": library_gemm_yardstick(dev)}))

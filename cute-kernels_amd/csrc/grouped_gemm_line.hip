@@ -28,8 +28,11 @@
 #ifndef CK_LOAD_GAP
 #define CK_LOAD_GAP 0  // measurement builds only: MFMAs between two loads of the next-but-one K step (0: spread over the whole last slice)
 #endif
+#ifndef CK_READ_SPREAD
+#define CK_READ_SPREAD 1
+#endif
 #ifndef CK_STAMP
-#define CK_STAMP 0  // measurement builds only: 1 = every wave adds up the cycles it spends waiting for the loads and at the barrier of each K step and writes them, with its main-loop and epilogue cycles, to GemmParams::trace
+#define CK_STAMP 0  // measurement builds only: 1 = every wave adds up the cycles it spends waiting for the loads and at the barrier of each K step and writes them, with its main-loop and epilogue cycles, to GemmParams::trace; 3 = instead, the cycles of every group of 8 MFMAs of the second slice of a K step (the additions behind the last group count into it)
 #endif
 
 namespace ck {
@@ -79,6 +82,7 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);  // uniform: everything derived from it stays in scalar registers
   const int wm = wave >> 1, wn = wave & 1;
   [[maybe_unused]] uint64_t st_begin = 0, st_loop = 0, st_end = 0, st_vm = 0, st_bar = 0, st_s0 = 0, st_s1 = 0, st_mark = 0;
+  [[maybe_unused]] uint64_t st_fine[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   if constexpr (CK_STAMP != 0) st_begin = clock64();
 
   // ---- which tile (same XCD-aware orders as the 256 x 256 kernel)
@@ -446,9 +450,17 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
       }
       constexpr int cur = kDouble ? (decltype(sl)::value & 1) : 0;
       constexpr int nxt = kDouble ? (cur ^ 1) : 0;
+      // CK_STAMP == 3: the clock is also read in front of every 8th MFMA of the second slice of a step (the
+      // reads are collected at the end of the slice, so that no wait for them sits between the MFMAs)
+      constexpr bool kFine = kPhase == 0 && !kIdle && !decltype(first)::value && CK_STAMP == 3 && kLast;
+      constexpr int kFineGroup = 8;
+      [[maybe_unused]] uint64_t fine_t[MI * NI / kFineGroup + 1];
 #pragma unroll
       for (int n = 0; n < MI * NI; ++n) {
         const int i = n / NI, j = n % NI;
+        if constexpr (kFine) {
+          if (n % kFineGroup == 0) asm volatile("s_memtime %0" : "=s"(fine_t[n / kFineGroup]));
+        }
         if constexpr (!kIdle) mfma(cur, i, j, first);
         if constexpr (kLast && kPhase == 0 && !(CK_ABLATE & 2)) {
           if (n % kLoadGap == 0 && n / kLoadGap < kLoadsPerStep) issue_one(kt + 2, n / kLoadGap);
@@ -457,8 +469,12 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
         if constexpr (kReload) {
           if constexpr (kDouble) {  // behind the first MI + NI MFMAs, in the order the next slice needs them (spreading
                                     // them over the whole slice measured the same)
-            if (n < MI) read_a(nxt, ns, nsl, n);
-            else if (n < MI + NI) read_b(nxt, ns, nsl, n - MI);
+            constexpr int kSpread = CK_READ_SPREAD;  // MFMAs between two fragment reads (measurement switch; 1 in the product)
+            if (n % kSpread == 0) {
+              const int r = n / kSpread;
+              if (r < MI) read_a(nxt, ns, nsl, r);
+              else if (r < MI + NI) read_b(nxt, ns, nsl, r - MI);
+            }
           } else {
             if (j == NI - 1) read_a(0, ns, nsl, i);
             if (i == MI - 1) read_b(0, ns, nsl, j);
@@ -466,6 +482,11 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
         }
       }
       __builtin_amdgcn_sched_barrier(0);
+      if constexpr (kFine) {
+        asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(fine_t[MI * NI / kFineGroup])::"memory");
+#pragma unroll
+        for (int g = 0; g < MI * NI / kFineGroup; ++g) st_fine[g] += fine_t[g + 1] - fine_t[g];
+      }
       if constexpr (CK_STAMP != 0 && kLast && kPhase < 2) {
         const uint64_t t3 = clock64();
         st_s1 += t3 - st_mark;  // slice 1: from the barrier to the end of the step
@@ -794,6 +815,10 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
       t[5] = (uint64_t)nk;
       t[6] = st_s0;
       t[7] = st_s1;
+      if constexpr (CK_STAMP == 3) {  // the eight groups of eight MFMAs of the second slice, summed over the K steps
+#pragma unroll
+        for (int g = 0; g < 8; ++g) t[g] = st_fine[g];
+      }
     }
   }
 }
