@@ -28,6 +28,12 @@
 #ifndef CK_LOAD_GAP
 #define CK_LOAD_GAP 0  // measurement builds only: MFMAs between two loads of the next-but-one K step (0: spread over the whole last slice)
 #endif
+#ifndef CK_B3
+#define CK_B3 0  // 1: three stages for the weight operand (its loads fly two K steps), see kB3 in the kernel
+#endif
+#ifndef CK_WARM
+#define CK_WARM 0  // n > 0: every K step also touches the weight lines of step kt + 2 + n (one 4-byte load per line), see warm_b
+#endif
 #ifndef CK_READ_SPREAD
 #define CK_READ_SPREAD 1
 #endif
@@ -57,10 +63,12 @@ struct Tile {
   static constexpr int B_LD = BN * kRowBytes / (1024 * NW);
   static constexpr int kLoadsPerStep = A_LD + B_LD;
   static constexpr size_t kLdsBytes = (size_t)NSTAGE * kStageBytes;
+  static constexpr size_t kLdsBytesWarm = kLdsBytes + 256 * NW;  // + a sink for the line-touching loads (CK_WARM)
+  static constexpr size_t kLdsBytesB3 = (size_t)(2 * BM + 3 * BN) * kRowBytes;  // two stages of A, three of the weights
   // two fragment sets (the next slice is read a whole slice ahead) where the registers allow: 512 per lane with one
   // wave per SIMD, 256 with two
   static constexpr bool kDouble = WGM == 2;  // (contraction-strided operands: see the kernel)
-  static_assert(kLdsBytes <= 160 * 1024, "two stages fit the LDS of a CU");
+  static_assert(kLdsBytes <= 160 * 1024 && kLdsBytesB3 <= 160 * 1024, "the stages fit the LDS of a CU");
   static_assert(kLoadsPerStep <= MI * NI, "every load of a step has an MFMA of the last slice to hide behind");
   static_assert(NI % 4 == 0, "whole column-block pairs in each half of a wave's columns");
   static_assert(NT >= BM, "one thread per tile row");
@@ -262,6 +270,16 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   }
   static_assert(!BT || kBtWindows % 8 == 0 || kBtWindows == 24, "window swizzle works on groups of 8 windows");
   const int nk = k_len / BK;
+  // Stage layout. Default: two stages, each A (BM rows) followed by B (BN rows). kB3 (forward and input-gradient
+  // launches of a CK_B3 build): A0 A1 B0 B1 B2 -- the loads of the weight operand are the ones that arrive late (with
+  // the activations re-read from L2 the wait for a stage stays, with the weights it goes), so they get a third stage and
+  // fly two K steps: step kt issues A(kt + 2) into A stage kt % 2 and then B(kt + 3) into B stage kt % 3, and the wait in
+  // front of step kt + 1's fragments leaves the B_LD youngest loads (B(kt + 2)) in flight.
+  constexpr bool kB3 = CK_B3 != 0 && WGM == 2 && MODE != kDw;
+  constexpr int kAStage = BM * kRowBytes, kBStage = BN * kRowBytes;
+  auto a_stage_at = [&](int sa) { return kB3 ? sa * kAStage : sa * kStageBytes; };
+  auto b_stage_at = [&](int sb) { return kB3 ? 2 * kAStage + sb * kBStage : sb * kStageBytes + kAStage; };
+  auto next3 = [](int sb) { return sb == 2 ? 0 : sb + 1; };
 
   // One 1 KiB wave-load: scalar base (the operand at this K step, uniform over the wave) + the lane's 32-bit byte offset,
   // so that a load costs no vector arithmetic (a 64-bit vector add per load delayed the MFMA behind it)
@@ -279,18 +297,65 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   const char* b_base_u = uniform_ptr(b_base);
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds_c;
   const uint32_t wave_a = __builtin_amdgcn_readfirstlane(lds_base + wave * A_LD * 1024);
-  const uint32_t wave_b = __builtin_amdgcn_readfirstlane(lds_base + BM * kRowBytes + wave * B_LD * 1024);
-  auto issue_one = [&](int step, int g) {
-    const int64_t kb = (CK_ABLATE & 16) ? (int64_t)(step & 1) * kRowBytes : (int64_t)step * kRowBytes;
-    const int64_t kb_b = BT ? (int64_t)((CK_ABLATE & 16) ? (step & 1) : step) * BK * prm.ldw * 2 : kb;  // BT: 64 contraction rows further down
+  const uint32_t wave_b = __builtin_amdgcn_readfirstlane(lds_base + wave * B_LD * 1024);
+  // load g of a step: g < A_LD: A of `step`; else B of `step_b` into B stage `sb` (kB3: step + 1 and its stage; otherwise
+  // `step` and step % 2)
+  auto issue_one_ab = [&](int step, int step_b, int sb, int g) {
+    const int64_t kb = (int64_t)step * kRowBytes;
+    const int64_t kb_b = BT ? (int64_t)step_b * BK * prm.ldw * 2 : (int64_t)step_b * kRowBytes;
     const int64_t kb_a = AT ? (int64_t)step * BK * prm.lda * 2 : kb;
+    if (g < A_LD) dma16(a_base_u + kb_a, a_off[g], wave_a + (uint32_t)a_stage_at(step & 1) + g * 1024);
+    else dma16(b_base_u + kb_b, b_off[g - A_LD], wave_b + (uint32_t)b_stage_at(sb) + (g - A_LD) * 1024);
+  };
+  auto issue_one = [&](int step, int g) {
+    if constexpr (kB3) {
+      issue_one_ab(step, step, step % 3, g);  // (start-up only: the loop passes its own stage counter)
+      return;
+    }
+    // measurement builds: bit 16 = both operands re-read the first two K steps (L2 hits), 512 / 1024 = only A / only B does
+    const int64_t kb = (CK_ABLATE & 16) ? (int64_t)(step & 1) * kRowBytes : (int64_t)step * kRowBytes;
+    const int64_t kb_hot = (int64_t)(step & 1) * kRowBytes;
+    const int64_t kb_b = BT ? (int64_t)((CK_ABLATE & (16 | 1024)) ? (step & 1) : step) * BK * prm.ldw * 2
+                            : ((CK_ABLATE & 1024) ? kb_hot : kb);  // BT: 64 contraction rows further down
+    const int64_t kb_a = AT ? (int64_t)step * BK * prm.lda * 2 : ((CK_ABLATE & 512) ? kb_hot : kb);
     const uint32_t st = (uint32_t)((step & (NSTAGE - 1)) * kStageBytes);
     if (g < A_LD) dma16(a_base_u + kb_a, a_off[g], wave_a + st + g * 1024);
-    else dma16(b_base_u + kb_b, b_off[g - A_LD], wave_b + st + (g - A_LD) * 1024);
+    else dma16(b_base_u + kb_b, b_off[g - A_LD], wave_b + (uint32_t)kAStage + st + (g - A_LD) * 1024);
   };
   auto issue = [&](int step) {
 #pragma unroll
     for (int g = 0; g < kLoadsPerStep; ++g) issue_one(step, g);
+  };
+  // CK_WARM: one more load per wave and K step, 4 bytes per lane, each lane in another line of the weight tile of a later
+  // K step (64 lines a wave, the tile's 256 lines over the four waves). It lands in a sink behind the stages; what it is
+  // for is the line's arrival in L2 ahead of the real loads. It is issued last in its step and the wait for the next
+  // stage leaves the one youngest load in flight, so nobody waits for it.
+  constexpr bool kWarm = CK_WARM > 0 && !kB3 && WGM == 2 && MODE != kDw;
+  uint32_t warm_off = 0;
+  if constexpr (kWarm) {
+    const int l = wave * 64 + lane;  // line of the tile's weight slice
+    if constexpr (BT) {  // 64 contraction rows x 4 lines (256 columns)
+      const int64_t col = min((int64_t)nt * BN + (l & 3) * 64, (int64_t)prm.N - 8);
+      warm_off = (uint32_t)(((int64_t)(l >> 2) * prm.ldw + col) * 2);
+    } else {  // 256 weight rows, one line each
+      int64_t n;
+      if constexpr (MODE == kSwiglu) {
+        const int half = (l % WN) / (WN / 2);
+        const int within = (l / WN) * (WN / 2) + (l % (WN / 2));
+        n = (int64_t)half * prm.I + min((int64_t)nt * (BN / 2) + within, (int64_t)prm.I - 1);
+      } else {
+        n = min((int64_t)nt * BN + l, (int64_t)prm.N - 1);
+      }
+      warm_off = (uint32_t)(n * prm.ldw * 2);
+    }
+  }
+  const uint32_t warm_sink = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)TL::kLdsBytes + wave * 256);
+  auto warm_b = [&](int step) {
+    if constexpr (kWarm) {
+      if (step > nk - 1) step = nk - 1;  // always issued (the waits count on it); past the end it touches the last step again
+      const int64_t kb_b = BT ? (int64_t)step * BK * prm.ldw * 2 : (int64_t)step * kRowBytes;
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(warm_sink), "v"(warm_off), "s"(b_base_u + kb_b) : "m0");
+    }
   };
 
   // ---- fragments: slice sl of a row is its 16-byte chunks 4 sl + lane / 16 (the lane's 8 contraction values)
@@ -300,7 +365,7 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
 #pragma unroll
   for (int sl = 0; sl < KS; ++sl) slice_off[sl] = ((4 * sl + fq) ^ fsw) * 16;
   const int fa_row = (wm * WM + (lane & 15)) * kRowBytes;
-  const int fb_row = BM * kRowBytes + (wn * WN + (lane & 15)) * kRowBytes;
+  const int fb_row = (wn * WN + (lane & 15)) * kRowBytes;  // within the B part of a stage
   constexpr bool kDouble = TL::kDouble;
   constexpr int kSets = kDouble ? 2 : 1;
   frag_t fa[kSets][MI], fb[kSets][NI];
@@ -320,7 +385,7 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   }
   auto read_a = [&](int set, int stage, int sl, int i) {
     if constexpr (AT) {
-      const char* p = lds_c + stage * kStageBytes + at_off[i] + 32 * sl * kAtRowBytes;
+      const char* p = lds_c + a_stage_at(stage) + at_off[i] + 32 * sl * kAtRowBytes;
       union {
         tr16x4 h[2];
         frag_t f;
@@ -329,7 +394,7 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
       u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr16x4 __attribute__((address_space(3)))*)(p + 4 * kAtRowBytes));
       fa[set][i] = u.f;
     } else {
-      fa[set][i] = *reinterpret_cast<const frag_t*>(lds_c + stage * kStageBytes + slice_off[sl] + fa_row + i * 16 * kRowBytes);
+      fa[set][i] = *reinterpret_cast<const frag_t*>(lds_c + a_stage_at(stage) + slice_off[sl] + fa_row + i * 16 * kRowBytes);
     }
   };
   int bt_off[NI];
@@ -338,12 +403,12 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
 #pragma unroll
     for (int j = 0; j < NI; ++j) {
       const int q = (wn * WN + j * 16) / 16;
-      bt_off[j] = BM * kRowBytes + (8 * g + n_low) * kBtRowBytes + (swap02(q) ^ (n_low | ((g & 1) << 2))) * 32 + 8 * (i & 3);
+      bt_off[j] = (8 * g + n_low) * kBtRowBytes + (swap02(q) ^ (n_low | ((g & 1) << 2))) * 32 + 8 * (i & 3);
     }
   }
   auto read_b = [&](int set, int stage, int sl, int j) {
     if constexpr (BT) {
-      const char* p = lds_c + stage * kStageBytes + bt_off[j] + 32 * sl * kBtRowBytes;
+      const char* p = lds_c + b_stage_at(stage) + bt_off[j] + 32 * sl * kBtRowBytes;
       union {
         tr16x4 h[2];
         frag_t f;
@@ -352,7 +417,7 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
       u.h[1] = __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr16x4 __attribute__((address_space(3)))*)(p + 4 * kBtRowBytes));
       fb[set][j] = u.f;
     } else {
-      fb[set][j] = *reinterpret_cast<const frag_t*>(lds_c + stage * kStageBytes + slice_off[sl] + fb_row + j * 16 * kRowBytes);
+      fb[set][j] = *reinterpret_cast<const frag_t*>(lds_c + b_stage_at(stage) + slice_off[sl] + fb_row + j * 16 * kRowBytes);
     }
   };
   auto mfma = [&](int set, int i, int j, auto first) {
@@ -391,9 +456,15 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   if constexpr (CK_STAMP != 0) st_loop = clock64();
   if (nk > 0) {
     issue(0);
-    if (nk > 1) {
+    if (kB3 && nk > 2) {  // A0 B0 A1 B1 B2: step 0 has landed when all but the last two steps' worth of loads are in
       issue(1);
-      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kLoadsPerStep) : "memory");  // step 0 landed, all waves
+#pragma unroll
+      for (int g = A_LD; g < kLoadsPerStep; ++g) issue_one_ab(0, 2, 2, g);
+      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kLoadsPerStep + B_LD) : "memory");
+    } else if (nk > 1) {
+      issue(1);
+      warm_b(1 + CK_WARM);
+      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kLoadsPerStep + (kWarm ? 1 : 0)) : "memory");  // step 0 landed, all waves
     } else {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       zero_pad_slots(0);
@@ -421,14 +492,19 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
     //   every kLoadGap MFMAs. Phase 1 is step nk - 2 (nothing left to fetch), phase 2 the last step (nothing to wait
     //   for, nothing to reload).
     constexpr int kLoadGap = CK_LOAD_GAP > 0 ? CK_LOAD_GAP : (MI * NI) / kLoadsPerStep;
-    auto slice = [&](int kt, auto sl, auto phase, auto idle, auto first) {
+    // bs: the B stage of step kt (kB3; unused otherwise). Phase 3 (kB3 only): step nk - 3, which still fetches A(nk - 1)
+    // but no B any more.
+    auto slice = [&](int kt, auto sl, auto phase, auto idle, auto first, int bs) {
       constexpr bool kIdle = decltype(idle)::value;  // this wave's rows are all pad rows: no fragments, no MFMAs
       constexpr bool kLast = decltype(sl)::value == KS - 1;
       constexpr int kPhase = decltype(phase)::value;
       const int ns = kLast ? (kt + 1) & (NSTAGE - 1) : kt & (NSTAGE - 1);
+      const int nsb = kB3 ? (kLast ? next3(bs) : bs) : ns;
       constexpr int nsl = kLast ? 0 : decltype(sl)::value + 1;
       constexpr bool kReload = !(kLast && kPhase == 2) && !(CK_ABLATE & 4) && !kIdle;
-      if constexpr (kLast && kPhase < 2) {
+      // kB3: while loads are still being issued, the youngest B_LD in flight belong to the step after the next
+      constexpr int kInFlight = kB3 && (kPhase == 0 || kPhase == 3) ? B_LD : (kWarm && kPhase == 0 ? 1 : 0);
+      if constexpr (kLast && kPhase != 2) {
         if constexpr ((CK_ABLATE & 1) != 0) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
         else if constexpr ((CK_ABLATE & 8) != 0) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         else if constexpr (AT && kPhase == 1) {  // the stage that has just landed is the last K step
@@ -438,7 +514,7 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
         } else if constexpr (CK_STAMP != 0) {
           asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
           const uint64_t t0 = clock64();
-          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kInFlight) : "memory");
           const uint64_t t1 = clock64();
           asm volatile("s_barrier" ::: "memory");
           const uint64_t t2 = clock64();
@@ -446,7 +522,7 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
           st_bar += t2 - t1;
           st_s0 += t0 - st_mark;  // slice 0 of this step (the slice in front of the wait)
           st_mark = t2;
-        } else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        } else asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kInFlight) : "memory");
       }
       constexpr int cur = kDouble ? (decltype(sl)::value & 1) : 0;
       constexpr int nxt = kDouble ? (cur ^ 1) : 0;
@@ -462,8 +538,12 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
           if (n % kFineGroup == 0) asm volatile("s_memtime %0" : "=s"(fine_t[n / kFineGroup]));
         }
         if constexpr (!kIdle) mfma(cur, i, j, first);
-        if constexpr (kLast && kPhase == 0 && !(CK_ABLATE & 2)) {
-          if (n % kLoadGap == 0 && n / kLoadGap < kLoadsPerStep) issue_one(kt + 2, n / kLoadGap);
+        if constexpr (kLast && (kPhase == 0 || kPhase == 3) && !(CK_ABLATE & 2)) {
+          if constexpr (kB3) {
+            if (n % kLoadGap == 0 && n / kLoadGap < (kPhase == 0 ? kLoadsPerStep : A_LD)) issue_one_ab(kt + 2, kt + 3, bs, n / kLoadGap);
+          } else {
+            if (n % kLoadGap == 0 && n / kLoadGap < kLoadsPerStep) issue_one(kt + 2, n / kLoadGap);
+          }
         }
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (kReload) {
@@ -473,21 +553,22 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
             if (n % kSpread == 0) {
               const int r = n / kSpread;
               if (r < MI) read_a(nxt, ns, nsl, r);
-              else if (r < MI + NI) read_b(nxt, ns, nsl, r - MI);
+              else if (r < MI + NI) read_b(nxt, nsb, nsl, r - MI);
             }
           } else {
             if (j == NI - 1) read_a(0, ns, nsl, i);
-            if (i == MI - 1) read_b(0, ns, nsl, j);
+            if (i == MI - 1) read_b(0, nsb, nsl, j);
           }
         }
       }
+      if constexpr (kWarm && kLast && kPhase == 0) warm_b(kt + 2 + CK_WARM);
       __builtin_amdgcn_sched_barrier(0);
       if constexpr (kFine) {
         asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(fine_t[MI * NI / kFineGroup])::"memory");
 #pragma unroll
         for (int g = 0; g < MI * NI / kFineGroup; ++g) st_fine[g] += fine_t[g + 1] - fine_t[g];
       }
-      if constexpr (CK_STAMP != 0 && kLast && kPhase < 2) {
+      if constexpr (CK_STAMP != 0 && kLast && kPhase != 2) {
         const uint64_t t3 = clock64();
         st_s1 += t3 - st_mark;  // slice 1: from the barrier to the end of the step
         st_mark = t3;
@@ -499,19 +580,37 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
       constexpr std::integral_constant<int, 0> s0{}, p0{};
       constexpr std::integral_constant<int, 1> s1{}, p1{};
       constexpr std::integral_constant<int, 2> p2{};
-      if constexpr (WGM == 2) slice(0, s0, p0, idle, std::true_type{});
-      else slice(0, s0, p0, idle, std::false_type{});
+      constexpr std::integral_constant<int, 3> p3{};
+      constexpr std::false_type later{};
+      int bs = 0;  // B stage of step kt (kB3)
+      if constexpr (WGM == 2) slice(0, s0, p0, idle, std::true_type{}, bs);
+      else slice(0, s0, p0, idle, later, bs);
       int kt = 0;
-      for (; kt + 2 < nk; ++kt) {
-        slice(kt, s1, p0, idle, std::false_type{});
-        slice(kt + 1, s0, p0, idle, std::false_type{});
+      if constexpr (kB3) {
+        for (; kt + 3 < nk; ++kt) {
+          slice(kt, s1, p0, idle, later, bs);
+          bs = next3(bs);
+          slice(kt + 1, s0, p0, idle, later, bs);
+        }
+        if (kt + 3 == nk) {
+          slice(kt, s1, p3, idle, later, bs);
+          bs = next3(bs);
+          slice(kt + 1, s0, p0, idle, later, bs);
+          ++kt;
+        }
+      } else {
+        for (; kt + 2 < nk; ++kt) {
+          slice(kt, s1, p0, idle, later, bs);
+          slice(kt + 1, s0, p0, idle, later, bs);
+        }
       }
       if (kt + 2 == nk) {
-        slice(kt, s1, p1, idle, std::false_type{});
-        slice(kt + 1, s0, p0, idle, std::false_type{});
+        slice(kt, s1, p1, idle, later, bs);
+        bs = next3(bs);
+        slice(kt + 1, s0, p0, idle, later, bs);
         ++kt;
       }
-      slice(kt, s1, p2, idle, std::false_type{});
+      slice(kt, s1, p2, idle, later, bs);
     };
     // A wave whose tile rows all lie past the expert's last row (the tile is the ragged end of a segment) still issues
     // its share of the loads and meets every barrier, but multiplies nothing: the wave it shares a SIMD with then has
@@ -826,7 +925,8 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
 template <typename T, int MODE, int BN, bool BT, int WGM, bool EXTRA>
 int launch_extra(const GemmParams& prm, unsigned blocks, hipStream_t s, const char* name) {
   auto kernel = grouped_gemm_line_kernel<T, MODE, BN, BT, WGM, EXTRA>;
-  constexpr size_t kLds = Tile<BN, WGM>::kLdsBytes;
+  constexpr size_t kLds = (CK_B3 != 0 && WGM == 2 && MODE != kDw) ? Tile<BN, WGM>::kLdsBytesB3
+                          : (CK_WARM > 0 && WGM == 2 && MODE != kDw) ? Tile<BN, WGM>::kLdsBytesWarm : Tile<BN, WGM>::kLdsBytes;
   static bool lds_reserved[kMaxDevices] = {};
   if (int rc = reserve_lds(reinterpret_cast<const void*>(kernel), kLds, lds_reserved, name)) return rc;
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(Tile<BN, WGM>::NT), kLds, s, prm);
