@@ -194,8 +194,11 @@ __device__ inline void store4(T* p, T v0, T v1, T v2, T v3) {
 
 // Tile order inside a run of tiles: groups of 8 along `a` (the side with a_count tiles), then `b`, with `a` fastest
 // inside a group -- 32 consecutive tiles form an 8 x 4 block that shares 8 + 4 operand panels.
+#ifndef CK_GROUP_M
+#define CK_GROUP_M 8  // tiles along M that walk the N direction together (measurement builds: 16, 32)
+#endif
 __device__ inline void grouped_order(int r, int a_count, int b_count, int& a, int& b) {
-  constexpr int GROUP = 8;
+  constexpr int GROUP = CK_GROUP_M;
   const int group_sz = GROUP * b_count;
   const int g = r / group_sz;
   const int first = g * GROUP;
