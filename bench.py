@@ -1,6 +1,6 @@
 """Benchmark of the MoE hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu-baseline] [--skip-secondary]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--skip-cpu-baseline] [--skip-secondary] [--lib FILE.so]
 
 A step is one forward+backward of the Mixtral-shape MoE layer of the baseline (T=16,384 tokens, H=4096, E=8, top-2,
 I=14,336, SwiGLU, bf16 with fp32 accumulation, Zipf(1.0) expert load, synthetic data, inputs resident in HBM).
@@ -26,16 +26,70 @@ PEAK_FP8_TFLOPS = 5000.0
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E
 
-# Bytes per launch between L2 and the fabric (fetched + written) from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of
-# this same command, FETCH_SIZE scaled x2.0 and WRITE_SIZE x1.0 against a 1 GiB device copy (known size);
-# summary and commands: profiles/grouped_gemm_c3_moe_fwd_bwd.md. Not measurable from inside this process.
-TRAFFIC_BYTES_PER_LAUNCH = {
-    "grouped_gemm_dw_rows": 2 * 5.951e6 * 1024 + 1.376e6 * 1024,  # both weight gradients, row-major operands
-    "grouped_gemm<swiglu>": 2 * 7.674e6 * 1024 + 2.782e6 * 1024,  # c_fc forward
-    "grouped_gemm_nn<scatter>": 2 * 8.342e6 * 1024 + 3.282e5 * 1024,  # c_fc dX, contraction-strided weights
-    "grouped_gemm_nn<grouped>": 2 * 4.002e6 * 1024 + 9.571e5 * 1024,  # c_proj dX, contraction-strided weights
-    "grouped_gemm<scatter>": 2 * 3.993e6 * 1024 + 3.259e5 * 1024,  # c_proj forward
-}
+# Bytes per launch between L2 and the fabric (fetched + written) are not measurable from inside this process: they come
+# from two rocprofv3 --pmc runs of this same command (FETCH_SIZE, then WRITE_SIZE, KiB per dispatch), summarised per
+# kernel name by `bench.py --summarize-pmc` into the tracked file below. A kernel whose name is not in that file (the
+# kernel changed since the counters were read) reports traffic null.
+TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "grouped_gemm_c3_hbm_traffic.txt")
+
+
+def load_traffic_summary(path: str = TRAFFIC_SUMMARY) -> dict:
+    """kernel name (as the kernel trace spells it) -> HBM bytes per launch, from the summary's tab-separated lines
+    `kernel<TAB>launches<TAB>fetch KiB per launch (scaled)<TAB>write KiB per launch (scaled)`."""
+    table = {}
+    if not os.path.exists(path):
+        return table
+    with open(path) as f:
+        for line in f:
+            if line.startswith("#") or not line.strip():
+                continue
+            name, _launches, fetch_kib, write_kib = line.rstrip("\n").split("\t")
+            table[name] = (float(fetch_kib) + float(write_kib)) * 1024.0
+    return table
+
+
+def summarize_pmc(fetch_dir: str, write_dir: str, out_path: str = TRAFFIC_SUMMARY) -> None:
+    """Reduce the counter_collection.csv files of two rocprofv3 --pmc runs of this benchmark with --copy-calibration
+    (FETCH_SIZE in one, WRITE_SIZE in the other) to one line per kernel: mean KiB per launch, each counter scaled by
+    what it reads for the 1 GiB device copy of the same run (known size: 2^20 KiB each way)."""
+    import csv
+    import glob
+
+    def per_kernel(directory: str, counter: str) -> dict:
+        sums: dict = {}
+        for path in glob.glob(os.path.join(directory, "**", "*counter_collection.csv"), recursive=True):
+            with open(path, newline="") as f:
+                for row in csv.DictReader(f):
+                    if row.get("Counter_Name") != counter:
+                        continue
+                    rec = sums.setdefault(row["Kernel_Name"], [0.0, 0])
+                    rec[0] += float(row["Counter_Value"])
+                    rec[1] += 1
+        return sums
+
+    def copy_factor(sums: dict, what: str) -> float:
+        # the calibration copy is the one elementwise copy kernel of 2^30 bytes: the largest per-launch reading among
+        # kernels whose name says "copy"
+        cands = [(v[0] / v[1], k) for k, v in sums.items() if "copy" in k.lower() and v[1] > 0]
+        if not cands:
+            raise SystemExit(f"no copy kernel in the {what} run: was bench.py run with --copy-calibration?")
+        reading = max(cands)[0]
+        return float(1 << 20) / reading
+
+    fetch, write = per_kernel(fetch_dir, "FETCH_SIZE"), per_kernel(write_dir, "WRITE_SIZE")
+    ff, wf = copy_factor(fetch, "FETCH_SIZE"), copy_factor(write, "WRITE_SIZE")
+    with open(out_path, "w") as f:
+        f.write("# HBM traffic per launch of the grouped GEMM kernels in `python bench.py --copy-calibration` (C3 workload)\n")
+        f.write(f"# from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (KiB per dispatch), scaled by {ff:.3f} and {wf:.3f}:\n")
+        f.write("# what makes the same counter read 2^20 KiB for the run's own 1 GiB device copy\n")
+        f.write("# kernel\tlaunches\tfetch_KiB_per_launch\twrite_KiB_per_launch\n")
+        for name in sorted(fetch):
+            if "grouped_gemm" not in name or name not in write:
+                continue
+            fv, wv = fetch[name], write[name]
+            f.write(f"{name}\t{fv[1]}\t{fv[0] / fv[1] * ff:.1f}\t{wv[0] / wv[1] * wf:.1f}\n")
+    print(f"wrote {out_path}")
+
 
 # the kernel instantiation each launch name runs at this workload, as rocprofv3's kernel trace spells it
 # (grouped_gemm_line_kernel<T, MODE, BN, BT, WGM, EXTRA>: MODE 0 grouped, 1 scatter, 2 swiglu, 4 dw; BT: contraction-strided
@@ -47,6 +101,19 @@ ROCPROF_KERNEL = {
     "grouped_gemm_nn<grouped>": "grouped_gemm_line_kernel<bf16, 0, 256, true, 2, false>",
     "grouped_gemm<scatter>": "grouped_gemm_line_kernel<bf16, 1, 256, false, 2, false>",
 }
+
+
+def traffic_for(launch_name: str, summary_path: str = TRAFFIC_SUMMARY):
+    """HBM bytes per launch of the kernel behind `launch_name`, or None when the tracked counter summary does not hold
+    that kernel (spelled as rocprofv3 spells it, template arguments included)."""
+    want = ROCPROF_KERNEL.get(launch_name)
+    if want is None:
+        return None
+    norm = lambda n: n.replace(" ", "").replace("__hip_bfloat16", "bf16").replace("__bf16", "bf16")
+    for name, nbytes in load_traffic_summary(summary_path).items():
+        if norm(want) in norm(name):
+            return nbytes
+    return None
 
 # workload: configs[2] of the baseline, the configuration its headline metric (MoE fwd+bwd TFLOP/s) is quoted on
 T, H, E, TOP_K, I = 16384, 4096, 8, 2, 14336
@@ -210,44 +277,59 @@ def secondary_hbm_kernels(dev):
     out["combine_rows_C3"] = {"us": dt * 1e6, "GB/s": b / dt / 1e9, "frac_hbm": b / dt / 1e9 / PEAK_HBM_GBS}
     del src, idx, expanded, gates
 
-    # stand-alone SwiGLU (packed, C3 rows x 2I) and RMSNorm (C5 rows: 65,536 x 4,096), forward and backward
+    # stand-alone SwiGLU (packed, C3 rows x 2I), RMSNorm and the fused residual add (C5 rows: 65,536 x 4,096), forward and
+    # backward: straight through the C ABI with caller-owned outputs and workspaces, like the count rows above (through
+    # autograd, a row would also time the allocator: 1.9 GB of fresh gradients per iteration)
     def rec(name, dt, b):
         out[name] = {"us": dt * 1e6, "GB/s": b / dt / 1e9, "frac_hbm": b / dt / 1e9 / PEAK_HBM_GBS}
 
-    xp = torch.randn(R, 2 * I, device=dev, dtype=torch.bfloat16, requires_grad=True)
-    rec("swiglu_packed_fwd_C3", timed(lambda: cute_kernels.swiglu_packed_cute(xp.detach())), 3 * R * I * 2)
-    yp = cute_kernels.swiglu_packed_cute(xp)
-    gy = torch.randn_like(yp)
-    rec("swiglu_packed_bwd_C3", timed(lambda: torch.autograd.grad(yp, xp, gy, retain_graph=True)), 5 * R * I * 2)
-    del xp, yp, gy
+    bf = _C.CK_BF16
+    xp = torch.randn(R, 2 * I, device=dev, dtype=torch.bfloat16)
+    yp = torch.empty(R, I, device=dev, dtype=torch.bfloat16)
+    up_p, gate_p = xp[:, :I], xp[:, I:]  # packed order: up first, gate second
+    rec("swiglu_packed_fwd_C3",
+        timed(lambda: _C.check(lib.ck_swiglu_fwd(gate_p.data_ptr(), 2 * I, up_p.data_ptr(), 2 * I, yp.data_ptr(), I, R, I, bf, stream))),
+        3 * R * I * 2)
+    gy = torch.randn(R, I, device=dev, dtype=torch.bfloat16)
+    dxp = torch.empty_like(xp)
+    d_up, d_gate = dxp[:, :I], dxp[:, I:]
+    rec("swiglu_packed_bwd_C3",
+        timed(lambda: _C.check(lib.ck_swiglu_bwd(gate_p.data_ptr(), 2 * I, up_p.data_ptr(), 2 * I, gy.data_ptr(), I, d_gate.data_ptr(),
+                                                 2 * I, d_up.data_ptr(), 2 * I, R, I, bf, stream))),
+        5 * R * I * 2)
+    del xp, yp, gy, dxp, up_p, gate_p, d_up, d_gate
     Bn, Hn = 65536, 4096
-    xn = torch.randn(Bn, Hn, device=dev, dtype=torch.bfloat16, requires_grad=True)
-    wn = torch.ones(Hn, device=dev, dtype=torch.bfloat16, requires_grad=True)
-    rec("rmsnorm_fwd_C5", timed(lambda: cute_kernels.rmsnorm_cute(xn.detach(), wn.detach(), 1e-6)), 2 * Bn * Hn * 2 + 4 * Bn)
-    yn = cute_kernels.rmsnorm_cute(xn, wn, 1e-6)
-    gn = torch.randn_like(yn)
-    rec("rmsnorm_bwd_C5", timed(lambda: torch.autograd.grad(yn, (xn, wn), gn, retain_graph=True)), 3 * Bn * Hn * 2 + 4 * Bn)
+    xn = torch.randn(Bn, Hn, device=dev, dtype=torch.bfloat16)
+    wn = torch.ones(Hn, device=dev, dtype=torch.bfloat16)
+    yn, gn, dxn = torch.empty_like(xn), torch.randn_like(xn), torch.empty_like(xn)
+    rstd = torch.empty(Bn, device=dev, dtype=torch.float32)
+    dwn = torch.empty(Hn, device=dev, dtype=torch.float32)
+    partial = torch.empty(max(lib.ck_rmsnorm_bwd_partial_rows(Bn), 1), Hn, device=dev, dtype=torch.float32)
+    rec("rmsnorm_fwd_C5",
+        timed(lambda: _C.check(lib.ck_rmsnorm_fwd(xn.data_ptr(), wn.data_ptr(), 1e-6, Bn, Hn, yn.data_ptr(), rstd.data_ptr(), bf, stream))),
+        2 * Bn * Hn * 2 + 4 * Bn)
+    rec("rmsnorm_bwd_C5",
+        timed(lambda: _C.check(lib.ck_rmsnorm_bwd(xn.data_ptr(), wn.data_ptr(), gn.data_ptr(), rstd.data_ptr(), 1e-6, Bn, Hn,
+                                                  dxn.data_ptr(), partial.data_ptr(), dwn.data_ptr(), bf, stream))),
+        3 * Bn * Hn * 2 + 4 * Bn)
     # the step that precedes an MoE block in a transformer: residual add fused into the norm (same rows); algorithmic
     # bytes: forward reads x, residual and writes y, added; backward reads added, d_y, d_added and writes d_x, d_residual
-    rn = torch.randn(Bn, Hn, device=dev, dtype=torch.bfloat16, requires_grad=True)
-    rec(
-        "fused_residual_add_rmsnorm_fwd_C5",
-        timed(lambda: cute_kernels.fused_residual_add_rmsnorm_cute(xn.detach(), rn.detach(), wn.detach(), 1e-6)),
-        4 * Bn * Hn * 2 + 4 * Bn,
-    )
-    yf, af = cute_kernels.fused_residual_add_rmsnorm_cute(xn, rn, wn, 1e-6)
-    ga = torch.randn_like(af)
-    rec(
-        "fused_residual_add_rmsnorm_bwd_C5",
-        timed(lambda: torch.autograd.grad((yf, af), (xn, rn, wn), (gn, ga), retain_graph=True)),
-        5 * Bn * Hn * 2 + 4 * Bn,
-    )
-    del yn, gn, rn, yf, af, ga
+    rn, an, ga, drn = torch.randn_like(xn), torch.empty_like(xn), torch.randn_like(xn), torch.empty_like(xn)
+    rec("fused_residual_add_rmsnorm_fwd_C5",
+        timed(lambda: _C.check(lib.ck_fused_residual_add_rmsnorm_fwd(xn.data_ptr(), rn.data_ptr(), wn.data_ptr(), 1e-6, 1.0, Bn, Hn,
+                                                                     yn.data_ptr(), an.data_ptr(), rstd.data_ptr(), bf, stream))),
+        4 * Bn * Hn * 2 + 4 * Bn)
+    rec("fused_residual_add_rmsnorm_bwd_C5",
+        timed(lambda: _C.check(lib.ck_fused_residual_add_rmsnorm_bwd(an.data_ptr(), wn.data_ptr(), gn.data_ptr(), ga.data_ptr(),
+                                                                     rstd.data_ptr(), 1e-6, 1.0, Bn, Hn, dxn.data_ptr(), drn.data_ptr(),
+                                                                     partial.data_ptr(), dwn.data_ptr(), bf, stream))),
+        5 * Bn * Hn * 2 + 4 * Bn)
+    del yn, gn, dxn, rn, an, ga, drn, partial
     # RMSNorm fused ahead of the router (one pass: normalised rows + router logits, optionally the e4m3 rows) against the
     # separate kernels (rmsnorm, the router's linear layer on the BLAS library, the row quantiser); algorithmic bytes:
     # rows in and out once, logits out (+ 1 byte per element and a scale per row with the e4m3 rows)
     for tag, (Bp, Hp, Ep) in {"C4": (8192, 2048, 64), "C5": (65536, 4096, 128)}.items():
-        xr_, wr_ = xn.detach()[:Bp, :Hp].contiguous(), wn.detach()[:Hp].contiguous()
+        xr_, wr_ = xn[:Bp, :Hp].contiguous(), wn[:Hp].contiguous()
         gr_ = (torch.randn(Ep, Hp, device=dev) * Hp**-0.5).to(torch.bfloat16)
         b_plain, b_quant = 2 * Bp * Hp * 2 + Bp * Ep * 2, 2 * Bp * Hp * 2 + Bp * Ep * 2 + Bp * Hp + 4 * Bp
         with torch.no_grad():
@@ -258,12 +340,14 @@ def secondary_hbm_kernels(dev):
         del xr_, wr_, gr_
     del xn, wn
     # router-logit statistics: softmax over all experts at the C5 router shape (65,536 x 128)
-    lg = torch.randn(Bn, 128, device=dev, dtype=torch.bfloat16, requires_grad=True)
-    rec("softmax_fwd_C5_router", timed(lambda: cute_kernels.softmax_cute(lg.detach())), 2 * Bn * 128 * 2)
-    sm = cute_kernels.softmax_cute(lg)
-    gs = torch.randn_like(sm)
-    rec("softmax_bwd_C5_router", timed(lambda: torch.autograd.grad(sm, lg, gs, retain_graph=True)), 3 * Bn * 128 * 2)
-    del lg, sm, gs
+    lg = torch.randn(Bn, 128, device=dev, dtype=torch.bfloat16)
+    sm, gs, dlg = torch.empty_like(lg), torch.randn_like(lg), torch.empty_like(lg)
+    rec("softmax_fwd_C5_router",
+        timed(lambda: _C.check(lib.ck_softmax_fwd(lg.data_ptr(), 1.0, Bn, 128, sm.data_ptr(), bf, stream)), iters=100), 2 * Bn * 128 * 2)
+    rec("softmax_bwd_C5_router",
+        timed(lambda: _C.check(lib.ck_softmax_bwd(sm.data_ptr(), gs.data_ptr(), 1.0, Bn, 128, dlg.data_ptr(), bf, stream)), iters=100),
+        3 * Bn * 128 * 2)
+    del lg, sm, gs, dlg
     torch.cuda.empty_cache()
 
     # C4: fine-grained MoE fwd+bwd behind an RMSNorm prologue (T=8192, H=2048, E=64, top-8, I=1408, uniform routing)
@@ -326,12 +410,11 @@ def secondary_hbm_kernels(dev):
     return out, configs
 
 
-def gemm_only(dev, launches: int, stamps: bool = False, fine: bool = False):
+def gemm_only(dev, launches: int, stamps: bool = False, zeros: bool = False):
     """Just the c_fc-forward-shape grouped GEMM (grouped epilogue) at the C3 shape: the target of counter runs.
-    stamps: with a CK_STAMP measurement build (build.py --define CK_STAMP=1 --output libck_stamp.so, loaded through
-    CK_MI355_LIB), also print where a wave's cycles go: main loop, waiting for loads, waiting at the barrier, epilogue.
-    fine: with a CK_STAMP=3 build, print the cycles per MFMA of each group of 8 MFMAs of a K step's second slice (the
-    last group also holds the bookkeeping additions of the stamps themselves)."""
+    stamps: with a CK_STAMP measurement build (build.py --define CK_STAMP=1 --output FILE.so, loaded with --lib FILE.so),
+    also print where a wave's cycles go: main loop, waiting for loads, waiting at the barrier, epilogue.
+    zeros: all-zero operands (the chip's clock under the same instruction stream)."""
     import numpy as np
     import torch
 
@@ -344,14 +427,14 @@ def gemm_only(dev, launches: int, stamps: bool = False, fine: bool = False):
     seg = cute_kernels.sort_by_expert(ids.to(dev), E, 256)
     x = torch.randn(T, H, device=dev, dtype=torch.bfloat16)
     w = torch.randn(E, 2 * I, H, device=dev, dtype=torch.bfloat16) * 0.02
-    if os.environ.get("CK_BENCH_ZEROS") == "1":  # all-zero operands: the chip's clock under the same instruction stream
+    if zeros:
         x.zero_()
         w.zero_()
     y = torch.empty(seg.max_rows, 2 * I, device=dev, dtype=torch.bfloat16)
     trace = None
-    if stamps or fine:
+    if stamps:
         trace = torch.zeros(8 * 8 * 20000, dtype=torch.int64, device=dev)
-        os.environ["CK_TRACE_PTR"] = hex(trace.data_ptr())  # read by the library at every call (stamp builds only)
+        _C.set_option("trace_buffer", trace.data_ptr())  # stamp builds write their per-wave cycle counts here
     for _ in range(2):
         scattermoe._gemm(x, TOP_K, w, seg, _C.CK_EPI_GROUPED, y)
     s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
@@ -364,17 +447,10 @@ def gemm_only(dev, launches: int, stamps: bool = False, fine: bool = False):
     flops = 4.0 * R * H * I
     rec = {"kernel": "grouped_gemm<grouped>", "shape": [R, 2 * I, H], "avg_launch_ms": ms,
            "TFLOP/s": flops / ms / 1e9, "frac_mfma": flops / ms / 1e9 / PEAK_BF16_TFLOPS}
-    if trace is not None and fine:
-        t = trace.view(-1, 8).cpu().numpy().astype(np.float64)
-        t = t[(t != 0).any(1)]
-        assert len(t) > 0, "no stamps: is CK_MI355_LIB a CK_STAMP=3 build?"
-        steps = H // 64 - 2  # the steady-state K steps carry the stamps (not the first, not the last two)
-        rec["second_slice_cycles_per_mfma_by_group_of_8"] = [round(float(v), 2) for v in t.mean(0) / steps / 8]
-        rec["waves"] = int(len(t))
-    elif trace is not None:
+    if trace is not None:
         t = trace.view(-1, 8).cpu().numpy().astype(np.float64)
         t = t[t[:, 5] > 0]  # waves that ran a main loop
-        assert len(t) > 0, "no stamps: is CK_MI355_LIB a CK_STAMP build?"
+        assert len(t) > 0, "no stamps: is --lib a CK_STAMP build?"
         tot = t[:, 0] + t[:, 1] + t[:, 4]
         rec["stamps"] = {
             "waves": int(len(t)), "k_steps": float(t[:, 5].mean()),
@@ -440,8 +516,12 @@ def main() -> int:
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run one 1 GiB device copy (outside the timed region): the known-size kernel that "
                     "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE readings are scaled by")
-    ap.add_argument("--fine-stamps", action="store_true",
-                    help="with --only-gemm and a CK_STAMP=3 measurement build: cycles per MFMA inside a K step's second slice")
+    ap.add_argument("--lib", default=None, metavar="FILE.so",
+                    help="load this build of the library (a measurement build from build.py --define ... --output) instead of the product one")
+    ap.add_argument("--zeros", action="store_true", help="with --only-gemm: all-zero operands")
+    ap.add_argument("--no-split", action="store_true", help="never split the last round of GEMM tiles (A/B measurement)")
+    ap.add_argument("--summarize-pmc", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
+                    help="no GPU work: reduce two rocprofv3 --pmc output directories to profiles/grouped_gemm_c3_hbm_traffic.txt")
     ap.add_argument("--stamps", action="store_true",
                     help="with --only-gemm and a CK_STAMP measurement build: print the per-wave cycle breakdown")
     ap.add_argument("--only-yardstick", action="store_true",
@@ -452,14 +532,22 @@ def main() -> int:
               file=sys.stderr)
         return 2
 
+    if args.summarize_pmc:
+        summarize_pmc(*args.summarize_pmc)
+        return 0
+
     import torch
 
-    from cute_kernels import scattermoe
+    from cute_kernels import _C, scattermoe
 
+    if args.lib:
+        _C.use_library(args.lib)
+    if args.no_split:
+        scattermoe.options.gemm_split = False
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     if args.only_gemm > 0:
-        gemm_only(dev, args.only_gemm, args.stamps, args.fine_stamps)
+        gemm_only(dev, args.only_gemm, args.stamps, args.zeros)
         return 0
     if args.only_yardstick:
         print(json.dumps({"library_gemm_yardstick": library_gemm_yardstick(dev)}))
@@ -509,8 +597,9 @@ def main() -> int:
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
         "frac": achieved / PEAK_BF16_TFLOPS,
-        "traffic": TRAFFIC_BYTES_PER_LAUNCH.get(dominant),
-        "traffic_source": "static: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, see profiles/ (not measured in this run)",
+        "traffic": traffic_for(dominant),
+        "traffic_source": "profiles/grouped_gemm_c3_hbm_traffic.txt: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this command, "
+        "matched by kernel name (null: that kernel is not in the summary); not measured in this run",
         "avg_launch_ms": d["ms"] / d["launches"],
         "flops_per_launch": d["flops"] / d["launches"],
     }

@@ -5,11 +5,11 @@
 Every translation unit under csrc/ is compiled with hipcc to an object file (in parallel) and linked into
 cute_kernels/libck_mi355.so. Nothing is compiled at import time: the package only ever dlopens the result.
 
-Measurement builds: `--define CK_ABLATE=2 --output libck_ablate2.so` compiles the same sources with the given
-preprocessor definitions into their own object directory and links a separately named library next to the product
-one (the product library is untouched). The package loads it instead when the environment variable CK_MI355_LIB names
-it (file name inside cute_kernels/, or a path); the switches are documented where they are used (CK_ABLATE, CK_STAMP
-in csrc/grouped_gemm_line.hip and csrc/grouped_gemm_fp8.hip).
+Measurement builds: `--define CK_ABLATE=2 --output /some/dir/libck_ablate2.so` compiles the same sources with the given
+preprocessor definitions into an object directory of their own and links the library where --output says (outside
+the package: only the product library lives in cute_kernels/, and it is untouched). `bench.py --lib FILE.so` loads
+such a build; the switches are documented where they are used (CK_ABLATE, CK_STAMP in csrc/grouped_gemm_line.hip and
+csrc/grouped_gemm_fp8.hip).
 """
 
 from __future__ import annotations
@@ -61,8 +61,11 @@ def _compile(src: str, force: bool, defines: tuple[str, ...] = (), obj_dir: str 
 def build(jobs: int = 8, force: bool = False, defines: tuple[str, ...] = (), output: str | None = None) -> str:
     if defines and not output:
         raise ValueError("a build with --define needs its own --output name: the product library takes no definitions")
-    lib_path = LIB_PATH if not output else os.path.join(os.path.dirname(LIB_PATH), os.path.basename(output))
+    lib_path = LIB_PATH if not output else os.path.abspath(output)
+    if output and os.path.dirname(lib_path) == os.path.dirname(LIB_PATH):
+        raise ValueError("--output must lie outside the package directory: only the product library lives there")
     obj_dir = OBJ_DIR if not output else os.path.join(OBJ_DIR, os.path.splitext(os.path.basename(output))[0])
+    os.makedirs(os.path.dirname(lib_path), exist_ok=True)
     os.makedirs(obj_dir, exist_ok=True)
     with ThreadPoolExecutor(max_workers=max(1, jobs)) as pool:
         objs = list(pool.map(lambda s: _compile(s, force, tuple(defines), obj_dir), _sources()))

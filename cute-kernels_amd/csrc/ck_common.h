@@ -3,6 +3,8 @@
 
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include "debug_options.h"
 #include <stdio.h>
 
 #include "ck_mi355.h"

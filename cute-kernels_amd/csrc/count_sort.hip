@@ -231,16 +231,14 @@ struct SortPlan {
   int64_t seg_len; // multiple of kWave
 };
 
-inline int64_t sort_ids_per_segment() {  // measurement knob (more, shorter segments lengthen the last block's scan: 1024 is best)
-  const char* env = getenv("CK_SORT_SEG");
-  return env ? atol(env) : 1024;
-}
+// ids per wave segment (measured at 256 .. 4096: more, shorter segments lengthen the last block's scan; 1024 is fastest)
+constexpr int64_t kSortIdsPerSegment = 1024;
 
 SortPlan make_sort_plan(int64_t R, int E) {
   int64_t cap = kSortTableWords / (E > 0 ? E : 1);
   cap = (cap / kWavesPerBlock) * kWavesPerBlock;
   if (cap < kWavesPerBlock) cap = kWavesPerBlock;
-  int64_t want = ceil_div(R > 0 ? R : 1, sort_ids_per_segment());
+  int64_t want = ceil_div(R > 0 ? R : 1, kSortIdsPerSegment);
   want = round_up(want, kWavesPerBlock);
   SortPlan p;
   p.segments = (int)(want < cap ? want : cap);
@@ -409,10 +407,6 @@ int launch_count(const char* name, const void* ids, int32_t ids_are_i64, int64_t
   if (blocks < 1) blocks = 1;
   const int64_t max_blocks = num_bins <= 8 ? 1024 : 512;
   if (blocks > max_blocks) blocks = max_blocks;
-  if (const char* env = getenv("CK_COUNT_BLOCKS")) {  // tuning knob for measurements
-    const long v = atol(env);
-    if (v >= 1 && v <= 65535) blocks = v;
-  }
   // up to 8 bins: ballot counters in registers (5.8 TB/s; LDS atomics on so few addresses serialise: 2.1-5.1 TB/s);
   // more bins: LDS atomics (6.3-6.5 TB/s; 16 register counters measured 3.3 TB/s)
   const int reg_bins = num_bins <= 8 ? 8 : 0;  // 16 register counters measured slower (3.3 TB/s) than LDS atomics (5.6)
@@ -498,6 +492,92 @@ extern "C" int ck_count_offsets_static(const void* ids, int32_t ids_are_i64, int
   hipLaunchKernelGGL(zero_words_kernel, dim3((unsigned)ceil_div(words, kBlock)), dim3(kBlock), 0, s, ws, (int)words);
   CK_CHECK_LAUNCH(name);
   return launch_count(name, ids, ids_are_i64, n, num_bins, counts, ends, starts, ws, s);
+}
+
+// The padded grouped layout from a sort somebody else did (torch.sort + bincount + cumsum in the reference's own layer):
+// every block derives the tile-aligned segment starts from the inclusive offsets (E is small), block 0 writes the tables,
+// and every sorted position p of expert e goes to padded row seg_starts[e] + (p - starts[e]).
+template <typename id_t, typename off_t>
+__global__ __launch_bounds__(kBlock) void segments_from_sorted_kernel(
+    const id_t* __restrict__ sorted_expert_idxs, const id_t* __restrict__ sorted_scattered_idxs,
+    const off_t* __restrict__ ends, int64_t R, int E, int align, int64_t max_tiles, uint32_t* __restrict__ counts,
+    int32_t* __restrict__ seg_starts, int32_t* __restrict__ row_slot, int32_t* __restrict__ row_pos,
+    int32_t* __restrict__ tile_expert) {
+  extern __shared__ uint32_t lds[];  // padded[E + 1], starts[E], count[E], scan scratch
+  uint32_t* padded = lds;
+  uint32_t* first = lds + E + 1;
+  uint32_t* count = first + E;
+  uint32_t* tmp = count + E;
+  const int t = threadIdx.x;
+  for (int e = t; e < E; e += kBlock) {
+    const uint32_t end = (uint32_t)ends[e], begin = e > 0 ? (uint32_t)ends[e - 1] : 0u;
+    const uint32_t c = end >= begin ? end - begin : 0u;
+    first[e] = begin;
+    count[e] = c;
+    padded[e] = (c + (uint32_t)align - 1) / (uint32_t)align * (uint32_t)align;
+  }
+  __syncthreads();
+  const uint32_t padded_total = block_exclusive_scan(padded, E, tmp);
+  if (t == 0) padded[E] = padded_total;
+  __syncthreads();
+  if (blockIdx.x == 0) {
+    for (int e = t; e < E; e += kBlock) counts[e] = count[e];
+    for (int e = t; e <= E; e += kBlock) seg_starts[e] = (int32_t)padded[e];
+    for (int64_t tile = t; tile < max_tiles; tile += kBlock) {
+      const uint32_t row = (uint32_t)(tile * align);
+      int32_t owner = -1;
+      if (row < padded_total) {  // last e with padded[e] <= row (empty experts share a start with their successor)
+        int lo = 0, hi = E - 1;
+        while (lo < hi) {
+          const int mid = (lo + hi + 1) >> 1;
+          if (padded[mid] <= row) lo = mid; else hi = mid - 1;
+        }
+        owner = lo;
+      }
+      tile_expert[tile] = owner;
+    }
+  }
+  for (int64_t p = (int64_t)blockIdx.x * kBlock + t; p < R; p += (int64_t)gridDim.x * kBlock) {
+    const int e = load_id(sorted_expert_idxs + p);
+    if ((unsigned)e >= (unsigned)E) continue;
+    const int64_t j = p - (int64_t)first[e];
+    if (j < 0 || j >= (int64_t)count[e]) continue;  // offsets that do not describe these ids: the row stays unowned
+    const int64_t dst = (int64_t)padded[e] + j;
+    row_slot[dst] = load_id(sorted_scattered_idxs + p);
+    row_pos[dst] = (int32_t)p;
+  }
+}
+
+extern "C" int ck_segments_from_sorted(const void* sorted_expert_idxs, const void* sorted_scattered_idxs,
+                                       int32_t idxs_are_i64, const void* expert_offsets, int32_t offsets_are_i64,
+                                       int64_t R, int32_t E, int32_t align, uint32_t* counts, int32_t* seg_starts,
+                                       int32_t* row_slot, int32_t* row_pos, int32_t* tile_expert, void* stream) {
+  const char* name = "ck_segments_from_sorted";
+  CK_REQUIRE(E >= 1 && E <= kMaxSortBins, "%s: E=%d outside [1, %d]", name, E, kMaxSortBins);
+  CK_REQUIRE(align >= 1, "%s: align=%d must be positive", name, align);
+  CK_REQUIRE(R >= 0 && R < (int64_t)0x7fffffff - (int64_t)E * align, "%s: R=%lld out of range", name, (long long)R);
+  CK_REQUIRE(expert_offsets && counts && seg_starts && row_slot && row_pos && tile_expert, "%s: NULL argument", name);
+  CK_REQUIRE(R == 0 || (sorted_expert_idxs && sorted_scattered_idxs), "%s: NULL index tensor", name);
+  const int64_t max_tiles = ck_sort_max_rows(R, E, align) / align;
+  int64_t blocks = ceil_div(R > 0 ? R : 1, (int64_t)kBlock * 4);
+  if (blocks > 1024) blocks = 1024;
+  const size_t lds_bytes = ((size_t)3 * E + 1 + kWavesPerBlock) * sizeof(uint32_t);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+#define CK_LAUNCH_SEGMENTS(ID_T, OFF_T)                                                                               \
+  hipLaunchKernelGGL((segments_from_sorted_kernel<ID_T, OFF_T>), dim3((unsigned)blocks), dim3(kBlock), lds_bytes, s, \
+                     static_cast<const ID_T*>(sorted_expert_idxs), static_cast<const ID_T*>(sorted_scattered_idxs),   \
+                     static_cast<const OFF_T*>(expert_offsets), R, (int)E, (int)align, max_tiles, counts, seg_starts, \
+                     row_slot, row_pos, tile_expert)
+  if (idxs_are_i64) {
+    if (offsets_are_i64) CK_LAUNCH_SEGMENTS(int64_t, int64_t);
+    else CK_LAUNCH_SEGMENTS(int64_t, int32_t);
+  } else {
+    if (offsets_are_i64) CK_LAUNCH_SEGMENTS(int32_t, int64_t);
+    else CK_LAUNCH_SEGMENTS(int32_t, int32_t);
+  }
+#undef CK_LAUNCH_SEGMENTS
+  CK_CHECK_LAUNCH(name);
+  return CK_OK;
 }
 
 extern "C" int64_t ck_sort_max_rows(int64_t R, int32_t E, int32_t align) {

@@ -29,7 +29,8 @@ struct GemmParams {
   const int32_t* seg_starts;
   const uint32_t* counts;
   const int32_t* tile_expert;
-  const int32_t* row_slot;
+  const int32_t* row_slot;      // padded row -> index of the A row it reads (gathered input)
+  const int32_t* row_slot_out;  // padded row -> output row of the scatter epilogue (ck_segments::row_slot_out, else row_slot)
   void* y;
   void* y_t;
   int64_t ld_t;
@@ -39,14 +40,19 @@ struct GemmParams {
   const float* w_scale;  // fp8 only: per-output-channel scale of w, [E, N]
   int act_kind;          // kSwiglu epilogue: CK_ACT_SWIGLU (up * gate * sigmoid(gate)) or CK_ACT_GLU (up * sigmoid(gate));
                          // kGrouped epilogue with aux: CK_ACT_GELU_TANH (aux = gelu(y), second output)
-  void* trace;           // measurement builds only: per-workgroup phase timestamps (8 x uint64 each), else NULL
+  void* trace;           // measurement builds only (CK_STAMP): per-wave cycle counts, 8 x uint64 each, else NULL
   // Split contraction for the last, partial round of tiles (128-byte-row kernel, grouped / scatter epilogues):
   // split_ws = [tiles][parts][4 waves][64 blocks][64 lanes] f32x4 partial accumulators (at most kSplitMaxTail tiles in
-  // kSplitParts parts or twice as many in half as many parts), followed by 2 * kSplitMaxTail int32 arrival counters (zero between launches); NULL = never split. split_base = the launch's grid
-  // without the extra workgroups (they are blockIdx split_base ..).
+  // kSplitParts parts or twice as many in half as many parts), followed by 2 * kSplitMaxTail arrival words; NULL = never
+  // split. split_base = the launch's grid without the extra workgroups (they are blockIdx split_base ..).
+  // An arrival word holds (launch epoch << 4) | parts arrived. A part that finds another epoch in the word starts the
+  // count afresh, so the words need no initial value and nothing resets them: whatever an earlier launch (or one that
+  // was cut short) left behind reads as "nobody has arrived yet". split_epoch: 1 .. 2^28 - 1, unique per launch.
   float* split_ws;
   int split_base;
+  uint32_t split_epoch;
 };
+uint32_t next_split_epoch();  // process-wide launch counter (grouped_gemm.hip)
 constexpr int kSplitParts = 4, kSplitMaxTail = 64, kSplitMaxRounds = 64, kSplitMinSteps = 16;
 constexpr int64_t kSplitPartFloats = 4 * 64 * 64 * 4;  // one workgroup's 256 x 256 fp32 tile
 constexpr int64_t kSplitWorkspaceBytes = kSplitMaxTail * kSplitParts * kSplitPartFloats * 4 + 2 * kSplitMaxTail * 4;
@@ -134,8 +140,13 @@ struct Mfma16<f16_t> {
     asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, 0" : "=a"(c) : "v"(a), "v"(b));
   }
 };
-// after the last run_acc, before anything else reads the accumulators: longer than any MFMA's result latency
+// After the last run_acc, before anything else reads the accumulators: longer than any MFMA's result latency. The wait
+// alone is not enough: nothing ties the compiler's own reads of the accumulators (v_accvgpr_read, spills) to it, and the
+// scheduler is free to hoist them above the wait, right behind the MFMA that writes them (it did: a few stale values
+// per tile). mfma_fence(c) makes c a result of an empty asm statement placed behind the wait; volatile asm statements
+// keep their order, so every later read of c stays behind the wait. Call it for every accumulator.
 __device__ inline void mfma_drain() { asm volatile("s_nop 15\n\ts_nop 15" ::: "memory"); }
+__device__ inline void mfma_fence(f32x4& c) { asm volatile("" : "+a"(c)); }
 
 // f(integral_constant<int, 0>) ... f(integral_constant<int, N - 1>): a loop whose index is a constant expression
 template <int N, typename F>
@@ -194,11 +205,9 @@ __device__ inline void store4(T* p, T v0, T v1, T v2, T v3) {
 
 // Tile order inside a run of tiles: groups of 8 along `a` (the side with a_count tiles), then `b`, with `a` fastest
 // inside a group -- 32 consecutive tiles form an 8 x 4 block that shares 8 + 4 operand panels.
-#ifndef CK_GROUP_M
-#define CK_GROUP_M 8  // tiles along M that walk the N direction together (measurement builds: 16, 32)
-#endif
+// (measured at 4 / 8 / 16 / 32 tiles per group on the Mixtral-shape and fine-grained layers: 8 is fastest on both)
 __device__ inline void grouped_order(int r, int a_count, int b_count, int& a, int& b) {
-  constexpr int GROUP = CK_GROUP_M;
+  constexpr int GROUP = 8;
   const int group_sz = GROUP * b_count;
   const int g = r / group_sz;
   const int first = g * GROUP;

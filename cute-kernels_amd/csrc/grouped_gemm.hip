@@ -10,7 +10,7 @@
 // 128-byte LDS rows in grouped_gemm_line.hip instead. Here: workgroup = 8 waves in a 4 x 2 grid (or 4 in 2 x 2), wave
 // tiles built from 32x32 MFMA blocks, and two pipelines -- K step 32 straight from global memory into four swizzled LDS
 // stages (K % 32 == 0), or K step 64 through registers into two padded LDS stages (any K % 8 == 0).
-#include <stdlib.h>
+#include <atomic>
 
 #include "gemm_common.h"
 
@@ -27,24 +27,11 @@ constexpr int kChunksPerRow = 8;  // 16-byte chunks per 64-element row
 #define CK_ABLATE 0  // measurement builds only: 1 no barrier, 2 no loads in the loop, 4 no fragment reads, 8 no load wait
 #endif
 
-// CK_GEMM_PIPE=0 in the environment forces the register-staged pipeline (A/B measurements)
-const bool g_force_pipe0 = [] {
-  const char* env = getenv("CK_GEMM_PIPE");
-  return env != nullptr && env[0] == '0';
-}();
-
-// CK_GEMM_WAVES=4 in the environment selects the 4-wave variant of the direct-to-LDS pipeline (default: 8 waves)
-const bool g_eight_waves = [] {
-  const char* env = getenv("CK_GEMM_WAVES");
-  return !(env != nullptr && env[0] == '4');
-}();
-
-// CK_GEMM_LINE=0 in the environment keeps every launch on the kernels of this file (A/B measurements); read per call, so
-// tests can switch it in-process.
-inline bool line_kernel_enabled() {
-  const char* env = getenv("CK_GEMM_LINE");
-  return !(env != nullptr && env[0] == '0');
-}
+// Which of two kernels that compute the same result a launch takes, as set through ck_debug_set_option (tests and
+// measurements); the defaults are what the product runs.
+inline bool force_register_pipeline() { return debug_options().gemm_register_pipeline.load(std::memory_order_relaxed) != 0; }
+inline bool eight_waves() { return debug_options().gemm_four_waves.load(std::memory_order_relaxed) == 0; }
+inline bool line_kernel_enabled() { return debug_options().gemm_line_kernel.load(std::memory_order_relaxed) != 0; }
 
 
 // PIPE 0: K step 64, global -> registers -> padded LDS, two stages (any K % 8 == 0).
@@ -121,7 +108,7 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
   int scatter_row = -1;
   if constexpr (MODE == kScatter) {
     for (int r = threadIdx.x; r < BM; r += 64 * WGM * 2)  // at most one trip per thread: BM <= threads
-      if (m0 + r < valid_end) scatter_row = prm.row_slot[m0 + r];
+      if (m0 + r < valid_end) scatter_row = prm.row_slot_out[m0 + r];
   }
 
 #if (CK_ABLATE & 256)
@@ -661,7 +648,7 @@ __global__ __launch_bounds__(64 * WGM * 2) void grouped_gemm_kernel(const GemmPa
         static_for<4>([&](auto s) {
           const int64_t p = p_base + s;
           out_row[s] = -1;
-          if (p < valid_end) out_row[s] = (MODE == kScatter) ? (int64_t)prm.row_slot[p] : p;
+          if (p < valid_end) out_row[s] = (MODE == kScatter) ? (int64_t)prm.row_slot_out[p] : p;
         });
         static_for<NI>([&](auto j) {
           const int64_t n = (int64_t)nt * BN + wn * WN + j * 32 + col_in_block;
@@ -768,8 +755,8 @@ int launch_pipe(const GemmParams& prm, unsigned blocks, hipStream_t s, const cha
 template <typename T, int BM, int BN, int MODE>
 int launch(const GemmParams& prm, unsigned blocks, hipStream_t s, const char* name) {
   const bool dma = (MODE == kDw) || (prm.K % 32 == 0);
-  if (dma && !g_force_pipe0) {
-    if (g_eight_waves) return launch_pipe<T, BM, BN, MODE, 1, 4>(prm, blocks, s, name);
+  if (dma && !force_register_pipeline()) {
+    if (eight_waves()) return launch_pipe<T, BM, BN, MODE, 1, 4>(prm, blocks, s, name);
     return launch_pipe<T, BM, BN, MODE, 1, 2>(prm, blocks, s, name);
   }
   return launch_pipe<T, BM, BN, MODE, 0, 2>(prm, blocks, s, name);
@@ -785,9 +772,28 @@ int launch_by_tile(const GemmParams& prm, int align, unsigned blocks_256, unsign
 }  // namespace
 }  // namespace ck
 
+namespace ck {
+uint32_t next_split_epoch() {
+  static std::atomic<uint32_t> counter{0};
+  uint32_t e;
+  do e = counter.fetch_add(1, std::memory_order_relaxed) + 1u; while ((e & 0x0fffffffu) == 0);
+  return e & 0x0fffffffu;
+}
+}  // namespace ck
+
 using namespace ck;
 
 namespace {
+inline void fill_segments(GemmParams& prm, const ck_segments* seg) {
+  prm.align = seg->align;
+  prm.num_experts = seg->num_experts;
+  prm.seg_starts = seg->seg_starts;
+  prm.counts = seg->counts;
+  prm.tile_expert = seg->tile_expert;
+  prm.row_slot = seg->row_slot;
+  prm.row_slot_out = seg->row_slot_out != nullptr ? seg->row_slot_out : seg->row_slot;
+  prm.trace = debug_options().trace_buffer.load(std::memory_order_relaxed);  // NULL unless a measurement build was given one
+}
 // workspace for the split last round (NULL: never split): kSplitWorkspaceBytes, 16-byte aligned, counters zero
 inline float* split_workspace(void* workspace, int64_t workspace_bytes) {
   if (workspace == nullptr || workspace_bytes < kSplitWorkspaceBytes || !aligned16(workspace)) return nullptr;
@@ -824,8 +830,8 @@ static int grouped_gemm_impl(const void* a, int32_t a_gather_div, const void* w,
 
   // rows are addressed with 32-bit byte offsets: from the operand base for a, from the expert's slice for w
   CK_REQUIRE((int64_t)N * K * 2 < ((int64_t)1 << 32), "%s: one expert's weight matrix must stay below 4 GiB", name);
-  const bool line_kernel = seg->align == kLineBM && K % kLineK == 0 && epilogue != CK_EPI_SWIGLU_BWD && !g_force_pipe0 &&
-                           line_kernel_enabled();
+  const bool line_kernel = seg->align == kLineBM && K % kLineK == 0 && epilogue != CK_EPI_SWIGLU_BWD &&
+                           !force_register_pipeline() && line_kernel_enabled();
   // the 128-byte-row kernel addresses a grouped input from each tile's first row; the general kernel from the operand base
   CK_REQUIRE(a_gather_div > 0 || line_kernel || seg->max_rows * (int64_t)K * 2 < ((int64_t)1 << 32),
              "%s: the grouped input must stay below 4 GiB", name);
@@ -839,21 +845,13 @@ static int grouped_gemm_impl(const void* a, int32_t a_gather_div, const void* w,
   prm.act_kind = act_kind;
   prm.N = N;
   prm.K = K;
-  prm.align = seg->align;
-  prm.num_experts = seg->num_experts;
-  prm.seg_starts = seg->seg_starts;
-  prm.counts = seg->counts;
-  prm.tile_expert = seg->tile_expert;
-  prm.row_slot = seg->row_slot;
+  fill_segments(prm, seg);
   prm.y = y;
   prm.y_t = y_t;
   prm.ld_t = ld_t;
   prm.aux = aux;
   prm.aux_in = aux_in;
   prm.split_ws = split_workspace(workspace, workspace_bytes);
-#if (CK_ABLATE & 256) || defined(CK_STAMP)
-  if (const char* t = getenv("CK_TRACE_PTR")) prm.trace = reinterpret_cast<void*>(strtoull(t, nullptr, 16));
-#endif
   int out_cols = N;  // columns that tile along the grid
   if (epilogue == CK_EPI_SWIGLU) {
     CK_REQUIRE(N % 16 == 0 && aux != nullptr, "%s: the SwiGLU epilogue needs N = 2*I with I %% 8 == 0 and aux", name);
@@ -932,12 +930,7 @@ static int grouped_gemm_nn_impl(const void* a, const void* w, int32_t N, int32_t
   prm.w_expert_stride = (int64_t)N * K;
   prm.N = N;
   prm.K = K;
-  prm.align = seg->align;
-  prm.num_experts = seg->num_experts;
-  prm.seg_starts = seg->seg_starts;
-  prm.counts = seg->counts;
-  prm.tile_expert = seg->tile_expert;
-  prm.row_slot = seg->row_slot;
+  fill_segments(prm, seg);
   prm.y = y;
   prm.split_ws = split_workspace(workspace, workspace_bytes);
   prm.n_tiles = (int)ceil_div(N, 256);
@@ -973,12 +966,7 @@ extern "C" int ck_grouped_gemm_dw_rows(const void* a, const void* b, int32_t M, 
   prm.ldw = N;
   prm.M = M;
   prm.N = N;
-  prm.align = seg->align;
-  prm.num_experts = seg->num_experts;
-  prm.seg_starts = seg->seg_starts;
-  prm.counts = seg->counts;
-  prm.tile_expert = seg->tile_expert;
-  prm.row_slot = seg->row_slot;
+  fill_segments(prm, seg);
   prm.y = dw;
   prm.m_tiles = (int)ceil_div(M, kLineBM);
   prm.n_tiles = (int)ceil_div(N, 256);
@@ -1004,20 +992,12 @@ extern "C" int ck_grouped_gemm_dw(const void* a_t, const void* b_t, int64_t ld_t
   prm.ldw = ld_t;
   prm.M = M;
   prm.N = N;
-  prm.align = seg->align;
-  prm.num_experts = seg->num_experts;
-  prm.seg_starts = seg->seg_starts;
-  prm.counts = seg->counts;
-  prm.tile_expert = seg->tile_expert;
-  prm.row_slot = seg->row_slot;
+  fill_segments(prm, seg);
   prm.y = dw;
-#if (CK_ABLATE & 256) || defined(CK_STAMP)
-  if (const char* t = getenv("CK_TRACE_PTR")) prm.trace = reinterpret_cast<void*>(strtoull(t, nullptr, 16));
-#endif
   hipStream_t s = static_cast<hipStream_t>(stream);
   // tile size follows the problem, not the segment alignment: small weight matrices get 128x128 tiles
   const bool big = (M >= 1024 && N >= 1024);
-  if (big && !g_force_pipe0 && line_kernel_enabled()) {
+  if (big && !force_register_pipeline() && line_kernel_enabled()) {
     const int bn = 256;
     prm.m_tiles = (int)ceil_div(M, kLineBM);
     prm.n_tiles = (int)ceil_div(N, bn);

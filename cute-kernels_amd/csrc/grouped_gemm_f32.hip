@@ -24,6 +24,7 @@ struct F32Params {
   const uint32_t* counts;
   const int32_t* tile_expert;
   const int32_t* row_slot;
+  const int32_t* row_slot_out;
 };
 
 __device__ inline f32x16 zero_acc() {
@@ -54,9 +55,8 @@ __global__ __launch_bounds__(NT) void grouped_gemm_f32_kernel(const F32Params pr
   if (tid < TM) {
     const int64_t p = p0 + tid;
     const bool ok = p < valid_end;
-    const int slot = ok && (prm.a_gather_div > 0 || prm.scatter) ? prm.row_slot[p] : 0;
-    a_rows[tid] = ok ? (prm.a_gather_div > 0 ? (int64_t)(slot / prm.a_gather_div) : p) : -1;
-    out_rows[tid] = ok ? (prm.scatter ? (int64_t)slot : p) : -1;
+    a_rows[tid] = ok ? (prm.a_gather_div > 0 ? (int64_t)(prm.row_slot[p] / prm.a_gather_div) : p) : -1;
+    out_rows[tid] = ok ? (prm.scatter ? (int64_t)prm.row_slot_out[p] : p) : -1;
   }
   __syncthreads();
   const float* w = prm.w + (int64_t)e * prm.w_expert_stride;
@@ -186,6 +186,7 @@ extern "C" int ck_grouped_gemm_f32(const float* a, int32_t a_gather_div, const f
   prm.counts = seg->counts;
   prm.tile_expert = seg->tile_expert;
   prm.row_slot = seg->row_slot;
+  prm.row_slot_out = seg->row_slot_out != nullptr ? seg->row_slot_out : seg->row_slot;
   const int64_t blocks = seg->max_rows / TM * prm.n_tiles;
   CK_REQUIRE(blocks < (int64_t)0x7fffffff, "%s: grid too large", name);
   hipLaunchKernelGGL(grouped_gemm_f32_kernel, dim3((unsigned)blocks), dim3(NT), 0, static_cast<hipStream_t>(stream), prm);

@@ -118,9 +118,8 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
   {
     const int64_t p = m0 + tid;
     if (p < valid_end) {
-      const int slot = (prm.a_gather_div > 0 || MODE == kScatter) ? prm.row_slot[p] : 0;
-      meta_scale = prm.a_scale[prm.a_gather_div > 0 ? (int64_t)(slot / prm.a_gather_div) : p];
-      meta_row = (MODE == kScatter) ? slot : tid;
+      meta_scale = prm.a_scale[prm.a_gather_div > 0 ? (int64_t)(prm.row_slot[p] / prm.a_gather_div) : p];
+      meta_row = (MODE == kScatter) ? prm.row_slot_out[p] : tid;
     }
   }
 
@@ -237,12 +236,18 @@ __global__ __launch_bounds__(NT) void grouped_gemm_fp8_kernel(const GemmParams p
       } else {
         k_step(0, p2, idle, first);
       }
+      // behind the last MFMA, inside this variant of the loop: wait out the MFMA result latency and tie every accumulator
+      // to that wait, so that none of the compiler's own accumulator reads can move in front of it (see mfma_fence)
+      mfma_drain();
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j) mfma_fence(acc[i][j]);
     };
     const bool wave_idle = m0 + wm * WM >= valid_end;
     if (__builtin_amdgcn_readfirstlane(wave_idle)) k_loop(std::true_type{});
     else k_loop(std::false_type{});
   }
-  mfma_drain();
 
   // ---- epilogue, straight from the accumulators (as in the 16-bit kernel): a lane holds, per 16x16 block (i, j), the 4
   // consecutive output columns j * 16 + 4 (lane / 16) + 0..3 of tile row i * 16 + lane % 16; both scales are applied in
@@ -529,6 +534,7 @@ extern "C" int ck_grouped_gemm_fp8(const void* a8, const float* a_scale, int32_t
   prm.counts = seg->counts;
   prm.tile_expert = seg->tile_expert;
   prm.row_slot = seg->row_slot;
+  prm.row_slot_out = seg->row_slot_out != nullptr ? seg->row_slot_out : seg->row_slot;
   prm.y = y;
   prm.aux = aux;
   prm.a_scale = a_scale;

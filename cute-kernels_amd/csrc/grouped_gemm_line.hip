@@ -21,24 +21,16 @@
 
 #include "gemm_common.h"
 
+// Measurement builds only (build.py --define NAME=n --output FILE.so; the product library is built without either):
+// CK_ABLATE, a bit set: 2 no loads in the loop, 4 no fragment reads in the loop, 16 every K step loads the first two K
+//   steps again (L2 hits), 512 / 1024 the same for the A operand / the weight operand alone, 128 no output stores.
+// CK_STAMP=1: every wave adds up the cycles it spends waiting for the loads and at the barrier of each K step and writes
+//   them, with its prologue, main-loop and epilogue cycles, to the buffer given to ck_debug_set_trace_buffer.
 #ifndef CK_ABLATE
-#define CK_ABLATE 0  // measurement builds only (build.py --define CK_ABLATE=n --output ...): 1 no barrier, 2 no loads in the loop, 4 no fragment reads, 8 no wait for the loads, 16 every step loads the first two K steps again (L2 hits), 32 no epilogue, 64 no MFMA, 128 no row-major output stores
-#endif
-
-#ifndef CK_LOAD_GAP
-#define CK_LOAD_GAP 0  // measurement builds only: MFMAs between two loads of the next-but-one K step (0: spread over the whole last slice)
-#endif
-#ifndef CK_B3
-#define CK_B3 0  // 1: three stages for the weight operand (its loads fly two K steps), see kB3 in the kernel
-#endif
-#ifndef CK_WARM
-#define CK_WARM 0  // n > 0: every K step also touches the weight lines of step kt + 2 + n (one 4-byte load per line), see warm_b
-#endif
-#ifndef CK_READ_SPREAD
-#define CK_READ_SPREAD 1
+#define CK_ABLATE 0
 #endif
 #ifndef CK_STAMP
-#define CK_STAMP 0  // measurement builds only: 1 = every wave adds up the cycles it spends waiting for the loads and at the barrier of each K step and writes them, with its main-loop and epilogue cycles, to GemmParams::trace; 3 = instead, the cycles of every group of 8 MFMAs of the second slice of a K step (the additions behind the last group count into it)
+#define CK_STAMP 0
 #endif
 
 namespace ck {
@@ -63,12 +55,10 @@ struct Tile {
   static constexpr int B_LD = BN * kRowBytes / (1024 * NW);
   static constexpr int kLoadsPerStep = A_LD + B_LD;
   static constexpr size_t kLdsBytes = (size_t)NSTAGE * kStageBytes;
-  static constexpr size_t kLdsBytesWarm = kLdsBytes + 256 * NW;  // + a sink for the line-touching loads (CK_WARM)
-  static constexpr size_t kLdsBytesB3 = (size_t)(2 * BM + 3 * BN) * kRowBytes;  // two stages of A, three of the weights
   // two fragment sets (the next slice is read a whole slice ahead) where the registers allow: 512 per lane with one
   // wave per SIMD, 256 with two
   static constexpr bool kDouble = WGM == 2;  // (contraction-strided operands: see the kernel)
-  static_assert(kLdsBytes <= 160 * 1024 && kLdsBytesB3 <= 160 * 1024, "the stages fit the LDS of a CU");
+  static_assert(kLdsBytes <= 160 * 1024, "the stages fit the LDS of a CU");
   static_assert(kLoadsPerStep <= MI * NI, "every load of a step has an MFMA of the last slice to hide behind");
   static_assert(NI % 4 == 0, "whole column-block pairs in each half of a wave's columns");
   static_assert(NT >= BM, "one thread per tile row");
@@ -90,7 +80,6 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);  // uniform: everything derived from it stays in scalar registers
   const int wm = wave >> 1, wn = wave & 1;
   [[maybe_unused]] uint64_t st_begin = 0, st_loop = 0, st_end = 0, st_vm = 0, st_bar = 0, st_s0 = 0, st_s1 = 0, st_mark = 0;
-  [[maybe_unused]] uint64_t st_fine[8] = {0, 0, 0, 0, 0, 0, 0, 0};
   if constexpr (CK_STAMP != 0) st_begin = clock64();
 
   // ---- which tile (same XCD-aware orders as the 256 x 256 kernel)
@@ -163,7 +152,7 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   // scatter epilogue: the output row of tile row `tid`, fetched now and parked in LDS once the main loop is over
   int scatter_row = -1;
   if constexpr (MODE == kScatter) {
-    if (tid < BM && m0 + tid < valid_end) scatter_row = prm.row_slot[m0 + tid];
+    if (tid < BM && m0 + tid < valid_end) scatter_row = prm.row_slot_out[m0 + tid];
   }
 
   // One wave per SIMD (WGM == 2): nothing zeroes the accumulators; the first slice of the tile multiplies with the
@@ -270,16 +259,10 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   }
   static_assert(!BT || kBtWindows % 8 == 0 || kBtWindows == 24, "window swizzle works on groups of 8 windows");
   const int nk = k_len / BK;
-  // Stage layout. Default: two stages, each A (BM rows) followed by B (BN rows). kB3 (forward and input-gradient
-  // launches of a CK_B3 build): A0 A1 B0 B1 B2 -- the loads of the weight operand are the ones that arrive late (with
-  // the activations re-read from L2 the wait for a stage stays, with the weights it goes), so they get a third stage and
-  // fly two K steps: step kt issues A(kt + 2) into A stage kt % 2 and then B(kt + 3) into B stage kt % 3, and the wait in
-  // front of step kt + 1's fragments leaves the B_LD youngest loads (B(kt + 2)) in flight.
-  constexpr bool kB3 = CK_B3 != 0 && WGM == 2 && MODE != kDw;
-  constexpr int kAStage = BM * kRowBytes, kBStage = BN * kRowBytes;
-  auto a_stage_at = [&](int sa) { return kB3 ? sa * kAStage : sa * kStageBytes; };
-  auto b_stage_at = [&](int sb) { return kB3 ? 2 * kAStage + sb * kBStage : sb * kStageBytes + kAStage; };
-  auto next3 = [](int sb) { return sb == 2 ? 0 : sb + 1; };
+  // Stage layout: two stages, each A (BM rows) followed by B (BN rows).
+  constexpr int kAStage = BM * kRowBytes;
+  auto a_stage_at = [&](int st) { return st * kStageBytes; };
+  auto b_stage_at = [&](int st) { return st * kStageBytes + kAStage; };
 
   // One 1 KiB wave-load: scalar base (the operand at this K step, uniform over the wave) + the lane's 32-bit byte offset,
   // so that a load costs no vector arithmetic (a 64-bit vector add per load delayed the MFMA behind it)
@@ -298,20 +281,8 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   const uint32_t lds_base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) char*)lds_c;
   const uint32_t wave_a = __builtin_amdgcn_readfirstlane(lds_base + wave * A_LD * 1024);
   const uint32_t wave_b = __builtin_amdgcn_readfirstlane(lds_base + wave * B_LD * 1024);
-  // load g of a step: g < A_LD: A of `step`; else B of `step_b` into B stage `sb` (kB3: step + 1 and its stage; otherwise
-  // `step` and step % 2)
-  auto issue_one_ab = [&](int step, int step_b, int sb, int g) {
-    const int64_t kb = (int64_t)step * kRowBytes;
-    const int64_t kb_b = BT ? (int64_t)step_b * BK * prm.ldw * 2 : (int64_t)step_b * kRowBytes;
-    const int64_t kb_a = AT ? (int64_t)step * BK * prm.lda * 2 : kb;
-    if (g < A_LD) dma16(a_base_u + kb_a, a_off[g], wave_a + (uint32_t)a_stage_at(step & 1) + g * 1024);
-    else dma16(b_base_u + kb_b, b_off[g - A_LD], wave_b + (uint32_t)b_stage_at(sb) + (g - A_LD) * 1024);
-  };
+  // load g of K step `step`: g < A_LD: a wave-load of A, else of the weight operand, into stage step % 2
   auto issue_one = [&](int step, int g) {
-    if constexpr (kB3) {
-      issue_one_ab(step, step, step % 3, g);  // (start-up only: the loop passes its own stage counter)
-      return;
-    }
     // measurement builds: bit 16 = both operands re-read the first two K steps (L2 hits), 512 / 1024 = only A / only B does
     const int64_t kb = (CK_ABLATE & 16) ? (int64_t)(step & 1) * kRowBytes : (int64_t)step * kRowBytes;
     const int64_t kb_hot = (int64_t)(step & 1) * kRowBytes;
@@ -326,38 +297,6 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
 #pragma unroll
     for (int g = 0; g < kLoadsPerStep; ++g) issue_one(step, g);
   };
-  // CK_WARM: one more load per wave and K step, 4 bytes per lane, each lane in another line of the weight tile of a later
-  // K step (64 lines a wave, the tile's 256 lines over the four waves). It lands in a sink behind the stages; what it is
-  // for is the line's arrival in L2 ahead of the real loads. It is issued last in its step and the wait for the next
-  // stage leaves the one youngest load in flight, so nobody waits for it.
-  constexpr bool kWarm = CK_WARM > 0 && !kB3 && WGM == 2 && MODE != kDw;
-  uint32_t warm_off = 0;
-  if constexpr (kWarm) {
-    const int l = wave * 64 + lane;  // line of the tile's weight slice
-    if constexpr (BT) {  // 64 contraction rows x 4 lines (256 columns)
-      const int64_t col = min((int64_t)nt * BN + (l & 3) * 64, (int64_t)prm.N - 8);
-      warm_off = (uint32_t)(((int64_t)(l >> 2) * prm.ldw + col) * 2);
-    } else {  // 256 weight rows, one line each
-      int64_t n;
-      if constexpr (MODE == kSwiglu) {
-        const int half = (l % WN) / (WN / 2);
-        const int within = (l / WN) * (WN / 2) + (l % (WN / 2));
-        n = (int64_t)half * prm.I + min((int64_t)nt * (BN / 2) + within, (int64_t)prm.I - 1);
-      } else {
-        n = min((int64_t)nt * BN + l, (int64_t)prm.N - 1);
-      }
-      warm_off = (uint32_t)(n * prm.ldw * 2);
-    }
-  }
-  const uint32_t warm_sink = __builtin_amdgcn_readfirstlane(lds_base + (uint32_t)TL::kLdsBytes + wave * 256);
-  auto warm_b = [&](int step) {
-    if constexpr (kWarm) {
-      if (step > nk - 1) step = nk - 1;  // always issued (the waits count on it); past the end it touches the last step again
-      const int64_t kb_b = BT ? (int64_t)step * BK * prm.ldw * 2 : (int64_t)step * kRowBytes;
-      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2" ::"s"(warm_sink), "v"(warm_off), "s"(b_base_u + kb_b) : "m0");
-    }
-  };
-
   // ---- fragments: slice sl of a row is its 16-byte chunks 4 sl + lane / 16 (the lane's 8 contraction values)
   typedef typename Mfma16<T>::frag frag_t;
   const int fsw = swz128(lane & 15), fq = lane >> 4;
@@ -421,11 +360,6 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
     }
   };
   auto mfma = [&](int set, int i, int j, auto first) {
-    if constexpr ((CK_ABLATE & 64) != 0) {
-      asm volatile("" ::"v"(fa[set][i]), "v"(fb[set][j]));
-      if constexpr (decltype(first)::value && WGM == 2) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
-      return;
-    }
     // weight fragment first: a lane gets 4 consecutive output columns of one row
     if constexpr (WGM == 2 && decltype(first)::value) Mfma16<T>::run_acc_first(fb[set][j], fa[set][i], acc[i][j]);
     else if constexpr (WGM == 2) Mfma16<T>::run_acc(fb[set][j], fa[set][i], acc[i][j]);
@@ -456,15 +390,9 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   if constexpr (CK_STAMP != 0) st_loop = clock64();
   if (nk > 0) {
     issue(0);
-    if (kB3 && nk > 2) {  // A0 B0 A1 B1 B2: step 0 has landed when all but the last two steps' worth of loads are in
+    if (nk > 1) {
       issue(1);
-#pragma unroll
-      for (int g = A_LD; g < kLoadsPerStep; ++g) issue_one_ab(0, 2, 2, g);
-      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kLoadsPerStep + B_LD) : "memory");
-    } else if (nk > 1) {
-      issue(1);
-      warm_b(1 + CK_WARM);
-      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kLoadsPerStep + (kWarm ? 1 : 0)) : "memory");  // step 0 landed, all waves
+      asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(kLoadsPerStep) : "memory");  // step 0 landed, all waves
     } else {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       zero_pad_slots(0);
@@ -491,30 +419,23 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
     //   been read by everyone, so in phase 0 the loads of step kt + 2 overwrite it under this slice's MFMAs, one load
     //   every kLoadGap MFMAs. Phase 1 is step nk - 2 (nothing left to fetch), phase 2 the last step (nothing to wait
     //   for, nothing to reload).
-    constexpr int kLoadGap = CK_LOAD_GAP > 0 ? CK_LOAD_GAP : (MI * NI) / kLoadsPerStep;
-    // bs: the B stage of step kt (kB3; unused otherwise). Phase 3 (kB3 only): step nk - 3, which still fetches A(nk - 1)
-    // but no B any more.
-    auto slice = [&](int kt, auto sl, auto phase, auto idle, auto first, int bs) {
+    constexpr int kLoadGap = (MI * NI) / kLoadsPerStep;
+    auto slice = [&](int kt, auto sl, auto phase, auto idle, auto first) {
       constexpr bool kIdle = decltype(idle)::value;  // this wave's rows are all pad rows: no fragments, no MFMAs
       constexpr bool kLast = decltype(sl)::value == KS - 1;
       constexpr int kPhase = decltype(phase)::value;
       const int ns = kLast ? (kt + 1) & (NSTAGE - 1) : kt & (NSTAGE - 1);
-      const int nsb = kB3 ? (kLast ? next3(bs) : bs) : ns;
       constexpr int nsl = kLast ? 0 : decltype(sl)::value + 1;
       constexpr bool kReload = !(kLast && kPhase == 2) && !(CK_ABLATE & 4) && !kIdle;
-      // kB3: while loads are still being issued, the youngest B_LD in flight belong to the step after the next
-      constexpr int kInFlight = kB3 && (kPhase == 0 || kPhase == 3) ? B_LD : (kWarm && kPhase == 0 ? 1 : 0);
       if constexpr (kLast && kPhase != 2) {
-        if constexpr ((CK_ABLATE & 1) != 0) asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-        else if constexpr ((CK_ABLATE & 8) != 0) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
-        else if constexpr (AT && kPhase == 1) {  // the stage that has just landed is the last K step
+        if constexpr (AT && kPhase == 1) {  // the stage that has just landed is the last K step
           asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
           zero_pad_slots(kt + 1);
           asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         } else if constexpr (CK_STAMP != 0) {
           asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
           const uint64_t t0 = clock64();
-          asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kInFlight) : "memory");
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
           const uint64_t t1 = clock64();
           asm volatile("s_barrier" ::: "memory");
           const uint64_t t2 = clock64();
@@ -522,52 +443,30 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
           st_bar += t2 - t1;
           st_s0 += t0 - st_mark;  // slice 0 of this step (the slice in front of the wait)
           st_mark = t2;
-        } else asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kInFlight) : "memory");
+        } else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       }
       constexpr int cur = kDouble ? (decltype(sl)::value & 1) : 0;
       constexpr int nxt = kDouble ? (cur ^ 1) : 0;
-      // CK_STAMP == 3: the clock is also read in front of every 8th MFMA of the second slice of a step (the
-      // reads are collected at the end of the slice, so that no wait for them sits between the MFMAs)
-      constexpr bool kFine = kPhase == 0 && !kIdle && !decltype(first)::value && CK_STAMP == 3 && kLast;
-      constexpr int kFineGroup = 8;
-      [[maybe_unused]] uint64_t fine_t[MI * NI / kFineGroup + 1];
 #pragma unroll
       for (int n = 0; n < MI * NI; ++n) {
         const int i = n / NI, j = n % NI;
-        if constexpr (kFine) {
-          if (n % kFineGroup == 0) asm volatile("s_memtime %0" : "=s"(fine_t[n / kFineGroup]));
-        }
         if constexpr (!kIdle) mfma(cur, i, j, first);
-        if constexpr (kLast && (kPhase == 0 || kPhase == 3) && !(CK_ABLATE & 2)) {
-          if constexpr (kB3) {
-            if (n % kLoadGap == 0 && n / kLoadGap < (kPhase == 0 ? kLoadsPerStep : A_LD)) issue_one_ab(kt + 2, kt + 3, bs, n / kLoadGap);
-          } else {
-            if (n % kLoadGap == 0 && n / kLoadGap < kLoadsPerStep) issue_one(kt + 2, n / kLoadGap);
-          }
+        if constexpr (kLast && kPhase == 0 && !(CK_ABLATE & 2)) {
+          if (n % kLoadGap == 0 && n / kLoadGap < kLoadsPerStep) issue_one(kt + 2, n / kLoadGap);
         }
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (kReload) {
           if constexpr (kDouble) {  // behind the first MI + NI MFMAs, in the order the next slice needs them (spreading
                                     // them over the whole slice measured the same)
-            constexpr int kSpread = CK_READ_SPREAD;  // MFMAs between two fragment reads (measurement switch; 1 in the product)
-            if (n % kSpread == 0) {
-              const int r = n / kSpread;
-              if (r < MI) read_a(nxt, ns, nsl, r);
-              else if (r < MI + NI) read_b(nxt, nsb, nsl, r - MI);
-            }
+            if (n < MI) read_a(nxt, ns, nsl, n);
+            else if (n < MI + NI) read_b(nxt, ns, nsl, n - MI);
           } else {
             if (j == NI - 1) read_a(0, ns, nsl, i);
-            if (i == MI - 1) read_b(0, nsb, nsl, j);
+            if (i == MI - 1) read_b(0, ns, nsl, j);
           }
         }
       }
-      if constexpr (kWarm && kLast && kPhase == 0) warm_b(kt + 2 + CK_WARM);
       __builtin_amdgcn_sched_barrier(0);
-      if constexpr (kFine) {
-        asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(fine_t[MI * NI / kFineGroup])::"memory");
-#pragma unroll
-        for (int g = 0; g < MI * NI / kFineGroup; ++g) st_fine[g] += fine_t[g + 1] - fine_t[g];
-      }
       if constexpr (CK_STAMP != 0 && kLast && kPhase != 2) {
         const uint64_t t3 = clock64();
         st_s1 += t3 - st_mark;  // slice 1: from the barrier to the end of the step
@@ -580,37 +479,30 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
       constexpr std::integral_constant<int, 0> s0{}, p0{};
       constexpr std::integral_constant<int, 1> s1{}, p1{};
       constexpr std::integral_constant<int, 2> p2{};
-      constexpr std::integral_constant<int, 3> p3{};
       constexpr std::false_type later{};
-      int bs = 0;  // B stage of step kt (kB3)
-      if constexpr (WGM == 2) slice(0, s0, p0, idle, std::true_type{}, bs);
-      else slice(0, s0, p0, idle, later, bs);
+      if constexpr (WGM == 2) slice(0, s0, p0, idle, std::true_type{});
+      else slice(0, s0, p0, idle, later);
       int kt = 0;
-      if constexpr (kB3) {
-        for (; kt + 3 < nk; ++kt) {
-          slice(kt, s1, p0, idle, later, bs);
-          bs = next3(bs);
-          slice(kt + 1, s0, p0, idle, later, bs);
-        }
-        if (kt + 3 == nk) {
-          slice(kt, s1, p3, idle, later, bs);
-          bs = next3(bs);
-          slice(kt + 1, s0, p0, idle, later, bs);
-          ++kt;
-        }
-      } else {
-        for (; kt + 2 < nk; ++kt) {
-          slice(kt, s1, p0, idle, later, bs);
-          slice(kt + 1, s0, p0, idle, later, bs);
-        }
+      for (; kt + 2 < nk; ++kt) {
+        slice(kt, s1, p0, idle, later);
+        slice(kt + 1, s0, p0, idle, later);
       }
       if (kt + 2 == nk) {
-        slice(kt, s1, p1, idle, later, bs);
-        bs = next3(bs);
-        slice(kt + 1, s0, p0, idle, later, bs);
+        slice(kt, s1, p1, idle, later);
+        slice(kt + 1, s0, p0, idle, later);
         ++kt;
       }
-      slice(kt, s1, p2, idle, later, bs);
+      slice(kt, s1, p2, idle, later);
+      // Behind the last MFMA, still inside this variant of the loop (in front of the point where the idle and the
+      // multiplying variant meet again, where the compiler may move accumulators around): wait out the MFMA result
+      // latency and tie every accumulator to that wait (see mfma_fence).
+      if constexpr (WGM == 2) {
+        mfma_drain();
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+          for (int j = 0; j < NI; ++j) mfma_fence(acc[i][j]);
+      }
     };
     // A wave whose tile rows all lie past the expert's last row (the tile is the ragged end of a segment) still issues
     // its share of the loads and meets every barrier, but multiplies nothing: the wave it shares a SIMD with then has
@@ -635,7 +527,7 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   // form 9 k, of which 5 k are the register reads, conversions and swaps and 4 k the stores).
   // Plain (cached) stores: L2 merges the two 64-byte halves of an output line before it leaves for memory (measured
   // against non-temporal stores: 3 % faster launches at K = 4096).
-  if constexpr (WGM == 2) mfma_drain();
+
   if constexpr (kSplit) {
     if (split_part >= 0) {
       // every part leaves its accumulators in the workspace, in its own register layout (16 bytes per lane)
@@ -645,17 +537,26 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
       for (int i = 0; i < MI; ++i)
 #pragma unroll
         for (int j = 0; j < NI; ++j) *reinterpret_cast<f32x4*>(mine + (i * NI + j) * kWave * 4) = acc[i][j];
-      int* counters = reinterpret_cast<int*>(prm.split_ws + (int64_t)kSplitMaxTail * kSplitParts * kSplitPartFloats);
-      int* flag = reinterpret_cast<int*>(lds_c);  // the stages are dead
+      uint32_t* arrivals = reinterpret_cast<uint32_t*>(prm.split_ws + (int64_t)kSplitMaxTail * kSplitParts * kSplitPartFloats);
+      uint32_t* flag = reinterpret_cast<uint32_t*>(lds_c);  // the stages are dead
       __threadfence();  // the partial tile is visible device-wide before the ticket is taken
       __syncthreads();
-      if (tid == 0) *flag = atomicAdd(&counters[split_slot], 1);
+      if (tid == 0) {
+        // ticket = arrivals of THIS launch so far: a word left by another launch (any epoch but ours) counts as zero
+        uint32_t cur = __hip_atomic_load(&arrivals[split_slot], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT), nxt;
+        for (;;) {  // bounded: another part of this tile (at most three) changed the word in between
+          nxt = (cur >> 4) == prm.split_epoch ? cur + 1u : ((prm.split_epoch << 4) | 1u);
+          const uint32_t seen = atomicCAS(&arrivals[split_slot], cur, nxt);
+          if (seen == cur) break;
+          cur = seen;
+        }
+        *flag = nxt & 15u;
+      }
       __syncthreads();
-      const bool last = *flag == split_parts - 1;
+      const bool last = *flag == (uint32_t)split_parts;
       __syncthreads();  // everyone has read the flag before the epilogue reuses LDS
       if (!last) return;
       __threadfence();  // the other parts' tiles are read from memory, not from a stale cache line
-      if (tid == 0) counters[split_slot] = 0;  // zero again for the next launch
       const float* theirs = slot_ws + ((int64_t)wave * MI * NI * kWave + lane) * 4;
 #pragma unroll
       for (int i = 0; i < MI; ++i)
@@ -670,16 +571,7 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
     }
   }
   if constexpr (CK_STAMP != 0) st_end = clock64();
-  if constexpr ((CK_ABLATE & 32) != 0) {
-    float keep = 0.f;
-    static_for<MI>([&](auto i) { static_for<NI>([&](auto j) { keep += acc[i][j][0] + acc[i][j][1] + acc[i][j][2] + acc[i][j][3]; }); });
-    if (keep == 123.456f) static_cast<float*>(prm.y)[0] = keep;
-    return;
-  }
-  auto store_out = [](void* p, const vec16& v) {
-    if constexpr ((CK_ABLATE & 256) != 0) store16_nt(p, v);  // measurement: non-temporal output stores
-    else store16(p, v);
-  };
+  auto store_out = [](void* p, const vec16& v) { store16(p, v); };
   const int lrow = lane & 15, lg = lane >> 4;
   const bool odd_group = (lg & 1) != 0;
   const T kZero = Elem<T>::down(0.f);
@@ -716,8 +608,7 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
     const u32x4_t d = {v.w[0], v.w[1], v.w[2], v.w[3]};
     // The two wait states behind the store are the hardware's rule for a store of more than 8 bytes whose data registers
     // the next vector instruction overwrites; the compiler inserts them for its own stores and cannot see into this one.
-    if constexpr ((CK_ABLATE & 256) != 0) asm volatile("global_store_dwordx4 %0, %1, %2 nt\n\ts_nop 1" ::"v"(off), "v"(d), "s"(base_u) : "memory");
-    else asm volatile("global_store_dwordx4 %0, %1, %2\n\ts_nop 1" ::"v"(off), "v"(d), "s"(base_u) : "memory");
+    asm volatile("global_store_dwordx4 %0, %1, %2\n\ts_nop 1" ::"v"(off), "v"(d), "s"(base_u) : "memory");
   };
   auto store_lines_at = [&](const vec16& v1, const vec16& v2, int j, char* base_u, uint32_t row_off, bool inside, bool row_in,
                             int cols_left) {
@@ -914,10 +805,6 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
       t[5] = (uint64_t)nk;
       t[6] = st_s0;
       t[7] = st_s1;
-      if constexpr (CK_STAMP == 3) {  // the eight groups of eight MFMAs of the second slice, summed over the K steps
-#pragma unroll
-        for (int g = 0; g < 8; ++g) t[g] = st_fine[g];
-      }
     }
   }
 }
@@ -925,8 +812,7 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
 template <typename T, int MODE, int BN, bool BT, int WGM, bool EXTRA>
 int launch_extra(const GemmParams& prm, unsigned blocks, hipStream_t s, const char* name) {
   auto kernel = grouped_gemm_line_kernel<T, MODE, BN, BT, WGM, EXTRA>;
-  constexpr size_t kLds = (CK_B3 != 0 && WGM == 2 && MODE != kDw) ? Tile<BN, WGM>::kLdsBytesB3
-                          : (CK_WARM > 0 && WGM == 2 && MODE != kDw) ? Tile<BN, WGM>::kLdsBytesWarm : Tile<BN, WGM>::kLdsBytes;
+  constexpr size_t kLds = Tile<BN, WGM>::kLdsBytes;
   static bool lds_reserved[kMaxDevices] = {};
   if (int rc = reserve_lds(reinterpret_cast<const void*>(kernel), kLds, lds_reserved, name)) return rc;
   hipLaunchKernelGGL(kernel, dim3(blocks), dim3(Tile<BN, WGM>::NT), kLds, s, prm);
@@ -972,6 +858,7 @@ int launch_line(const GemmParams& prm_in, int mode, int bn, bool bt, int dtype, 
   GemmParams prm = prm_in;
   if (prm.split_ws != nullptr && (mode == kGrouped || mode == kScatter)) {
     prm.split_base = (int)blocks;  // the extra workgroups of a split last round sit behind the regular grid
+    prm.split_epoch = next_split_epoch();
     blocks += kSplitMaxTail * (kSplitParts - 1);
   } else {
     prm.split_ws = nullptr;

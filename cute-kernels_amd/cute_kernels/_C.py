@@ -15,11 +15,6 @@ import torch
 
 _LIB_NAME = "libck_mi355.so"
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), _LIB_NAME)
-# Measurement builds (build.py --define ... --output libck_<name>.so) are loaded instead of the product library when
-# CK_MI355_LIB names one: a file name inside this directory, or a path. Still no fallback: a missing file raises.
-if os.environ.get("CK_MI355_LIB"):
-    _alt = os.environ["CK_MI355_LIB"]
-    _LIB_PATH = _alt if os.path.sep in _alt else os.path.join(os.path.dirname(os.path.abspath(__file__)), _alt)
 
 CK_F32, CK_F16, CK_BF16 = 0, 1, 2
 CK_EPI_GROUPED, CK_EPI_SCATTER, CK_EPI_SWIGLU, CK_EPI_SWIGLU_BWD = 0, 1, 2, 3
@@ -39,6 +34,7 @@ class ck_segments(Structure):
         ("max_rows", c_int64),
         ("num_experts", c_int32),
         ("align", c_int32),
+        ("row_slot_out", c_void_p),
     ]
 
 
@@ -46,6 +42,7 @@ class ck_segments(Structure):
 _SIGNATURES = {
     "ck_last_error_string": (c_char_p, []),
     "ck_abi_version": (c_int32, []),
+    "ck_debug_set_option": (c_int32, [c_char_p, c_int64]),
     "ck_count_workspace_words": (c_int64, [c_int32]),
     "ck_count_offsets": (c_int32, [c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p]),
     "ck_count_offsets_static": (c_int32, [c_void_p, c_int32, c_int64, c_int32, c_void_p, c_void_p, c_void_p, c_void_p]),
@@ -55,6 +52,10 @@ _SIGNATURES = {
     "ck_sort_max_rows": (c_int64, [c_int64, c_int32, c_int32]),
     "ck_sort_workspace_words": (c_int64, [c_int64, c_int32]),
     "ck_sort_by_expert": (c_int32, [c_void_p, c_int32, c_int64, c_int32, c_int32] + [c_void_p] * 10),
+    "ck_segments_from_sorted": (
+        c_int32,
+        [c_void_p, c_void_p, c_int32, c_void_p, c_int32, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p],
+    ),
     "ck_gather_rows": (c_int32, [c_void_p, c_void_p, c_void_p, c_int32, c_int64, c_int32, c_void_p, c_int32, c_void_p]),
     "ck_combine_rows": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_int32, c_void_p, c_void_p, c_void_p, c_int32, c_void_p]),
     "ck_gate_grad_f32": (c_int32, [c_void_p, c_void_p, c_int64, c_int32, c_int32, c_void_p, c_int32, c_void_p]),
@@ -121,6 +122,21 @@ _lib = None
 
 def library_path() -> str:
     return _LIB_PATH
+
+
+def use_library(path: str) -> None:
+    """Load another build of the library (a measurement build made with build.py --define ... --output FILE.so) instead
+    of the product one. Must be called before the first kernel call of the process; bench.py --lib does. Still no
+    fallback: a missing file raises on first use."""
+    global _LIB_PATH
+    if _lib is not None:
+        raise RuntimeError("use_library: the library is already loaded")
+    _LIB_PATH = os.path.abspath(path)
+
+
+def set_option(name: str, value: int) -> None:
+    """ck_debug_set_option: choose between kernels that compute the same result (tests and measurements)."""
+    check(lib().ck_debug_set_option(name.encode(), int(value)))
 
 
 def lib() -> ctypes.CDLL:

@@ -8,7 +8,7 @@ names are eager PyTorch statements of the same operators (torch_ops.py), kept fo
 
 from .fp8 import MoE_E4M3, quantize_expert_weights_e4m3, quantize_rows_e4m3, swiglu_experts_e4m3
 from .continuous_count import continuous_count_and_offsets_cute, continuous_count_cute
-from .modules import Experts, MoE, MoE_Triton
+from .modules import Experts, Experts_Triton, MoE, MoE_Triton
 from .fused_residual_add_rmsnorm import fused_residual_add_rmsnorm_cute
 from .rmsnorm import rmsnorm_cute
 from .rmsnorm_route import rmsnorm_route_cute
@@ -19,6 +19,8 @@ from .scattermoe import (
     gather_rows,
     route_topk_softmax,
     route_topk_softmax_raw,
+    scattered_experts,
+    segments_from_sorted,
     sort_by_expert,
     swiglu_experts,
 )

@@ -614,3 +614,74 @@ def _experts_down_bwd(ctx, grad_out, _expanded_grad):
 
 
 experts_down.register_autograd(_experts_down_bwd, setup_context=_experts_down_setup)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# the reference's expert-linear interface (three index tensors, unpadded grouped rows)
+# ---------------------------------------------------------------------------------------------------------------
+@custom_op(f"{NS}::scattered_experts", mutates_args=())
+def scattered_experts(
+    x: Tensor, w: Tensor, gates: Optional[Tensor], bias: Optional[Tensor], sorted_expert_idxs: Tensor,
+    sorted_scattered_idxs: Tensor, expert_offsets: Tensor, k: int, grouped_in: bool, grouped_out: bool,
+) -> tuple[Tensor, Tensor]:
+    """(out, the ungated rows [R, N] that the gates' gradient needs, or empty)"""
+    ctx = _Ctx()
+    out = _moe._ScatteredExperts.forward(
+        ctx, x, w, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, gates, grouped_in, grouped_out, bias
+    )
+    return out, _or_empty(ctx.saved_tensors[3], x)
+
+
+@scattered_experts.register_fake
+def _(x, w, gates, bias, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, k, grouped_in, grouped_out):
+    R, N = sorted_expert_idxs.shape[0], w.shape[1]
+    if gates is None:
+        return x.new_empty(R, N), x.new_empty(0)
+    return x.new_empty(gates.shape[0], N), x.new_empty(R, N)
+
+
+@custom_op(f"{NS}::scattered_experts_backward", mutates_args=())
+def scattered_experts_backward(
+    grad_out: Tensor, x: Tensor, w: Tensor, gates: Optional[Tensor], expanded: Tensor, sorted_expert_idxs: Tensor,
+    sorted_scattered_idxs: Tensor, expert_offsets: Tensor, k: int, grouped_in: bool, grouped_out: bool, need_x: bool,
+    need_w: bool, need_gates: bool, need_bias: bool,
+) -> tuple[Tensor, Tensor, Tensor, Tensor]:
+    ctx = _Ctx((need_x, need_w, False, False, False, False, need_gates, False, False, need_bias, False))
+    ctx.seg = _moe.segments_from_sorted(sorted_expert_idxs, sorted_scattered_idxs, expert_offsets)
+    ctx.k, ctx.grouped_in, ctx.grouped_out = k, grouped_in, grouped_out
+    ctx.saved_tensors = (x.contiguous(), w.contiguous(), None if gates is None else gates.contiguous(), expanded)
+    grads = _moe._ScatteredExperts.backward(ctx, grad_out)
+    return _or_empty(grads[0], x), _or_empty(grads[1], x), _or_empty(grads[6], x), _or_empty(grads[9], x)
+
+
+@scattered_experts_backward.register_fake
+def _(grad_out, x, w, gates, expanded, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, k, grouped_in, grouped_out,
+      need_x, need_w, need_gates, need_bias):
+    e = x.new_empty(0)
+    return (
+        torch.empty_like(x) if need_x else e,
+        torch.empty_like(w) if need_w else e,
+        torch.empty_like(gates) if need_gates and gates is not None else e,
+        x.new_empty(w.shape[0], w.shape[1]) if need_bias else e,
+    )
+
+
+def _scattered_experts_setup(ctx, inputs, output):
+    x, w, gates, _bias, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, *rest = inputs
+    ctx.has_gates = gates is not None
+    ctx.save_for_backward(x, w, gates, output[1], sorted_expert_idxs, sorted_scattered_idxs, expert_offsets)
+    ctx.rest = tuple(rest)
+
+
+def _scattered_experts_bwd(ctx, grad_out, _expanded_grad):
+    need_x, need_w, need_gates, need_bias = ctx.needs_input_grad[:4]
+    d_x, d_w, d_gates, d_bias = scattered_experts_backward(
+        grad_out.contiguous(), *ctx.saved_tensors, *ctx.rest, need_x, need_w, need_gates and ctx.has_gates, need_bias
+    )
+    return (
+        (d_x if need_x else None), (d_w if need_w else None), (d_gates if need_gates and ctx.has_gates else None),
+        (d_bias if need_bias else None), *(None,) * 6,
+    )
+
+
+scattered_experts.register_autograd(_scattered_experts_bwd, setup_context=_scattered_experts_setup)

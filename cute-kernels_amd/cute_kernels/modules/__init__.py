@@ -1,1 +1,1 @@
-from .moe import Experts, MoE, MoE_Triton
+from .moe import Experts, Experts_Triton, MoE, MoE_Triton

@@ -20,6 +20,20 @@ from .utils import is_tracing
 _ops = None  # cute_kernels.compile_ops, set by the package once it is imported (used only while torch.compile traces)
 
 
+@dataclass
+class Options:
+    """Switches between forms that compute the same result, for tests and measurements (bench.py sets them from its
+    command line). The defaults are what the library runs; nothing reads the environment."""
+
+    gemm_split: bool = True  # the last, partial round of GEMM tiles splits its contraction over the idle CUs
+    bias_fused: bool = True  # expert biases join the GEMM's fp32 accumulators (False: their own kernel after the GEMM)
+    gemm_nn: bool = True  # input-gradient GEMMs read the weight as stored (False: through a transposed copy)
+    dw_rows: bool = True  # weight-gradient GEMMs read row-major operands (False: transposed copies)
+
+
+options = Options()
+
+
 # ---------------------------------------------------------------------------------------------------------------
 # routing
 # ---------------------------------------------------------------------------------------------------------------
@@ -146,16 +160,23 @@ class ExpertSegments:
     max_rows: int
     num_experts: int
     align: int
+    # int32 [max_rows]: the sorted position a padded row stands for, i.e. its row in an UNPADDED grouped tensor [R, *]
+    # (the reference's grouped_in / grouped_out layout). Only segments_from_sorted fills it.
+    row_pos: torch.Tensor | None = None
 
-    def c_struct(self) -> _C.ck_segments:
+    def c_struct(self, rows_in: torch.Tensor | None = None, rows_out: torch.Tensor | None = None) -> _C.ck_segments:
+        """rows_in: table a gathered input is read through (default row_slot); rows_out: table the scatter epilogue writes
+        through (default: the same as rows_in)."""
+        rows_in = self.row_slot if rows_in is None else rows_in
         return _C.ck_segments(
             self.seg_starts.data_ptr(),
             self.counts.data_ptr(),
             self.tile_expert.data_ptr(),
-            self.row_slot.data_ptr(),
+            rows_in.data_ptr(),
             self.max_rows,
             self.num_experts,
             self.align,
+            None if rows_out is None else rows_out.data_ptr(),
         )
 
     @property
@@ -268,23 +289,21 @@ _split_workspaces: dict = {}
 
 
 def _split_workspace(device: torch.device) -> torch.Tensor:
-    """Workspace of ck_grouped_gemm_ws / ck_grouped_gemm_nn_ws (split last round of tiles): one zero-initialised buffer
-    per device and stream (the kernels leave its counters zero; two streams must not share one). CK_GEMM_SPLIT=0 in the
-    environment switches the split off (measurement knob)."""
-    import os
-
-    if os.environ.get("CK_GEMM_SPLIT", "1") == "0":
+    """Workspace of ck_grouped_gemm_ws / ck_grouped_gemm_nn_ws (split last round of tiles): one buffer per device and
+    stream (launches that may overlap must not share one; it needs no initial contents)."""
+    if not options.gemm_split:
         return None
     key = (device.index, torch.cuda.current_stream(device).cuda_stream)
     ws = _split_workspaces.get(key)
     if ws is None:
-        ws = _split_workspaces[key] = torch.zeros(_C.lib().ck_grouped_gemm_workspace_bytes(), dtype=torch.uint8, device=device)
+        ws = _split_workspaces[key] = torch.empty(_C.lib().ck_grouped_gemm_workspace_bytes(), dtype=torch.uint8, device=device)
     return ws
 
 
-def _gemm_f32(a, gather_div, w, w_is_kn: bool, N: int, K: int, seg: ExpertSegments, scatter: bool, y, bias=None):
+def _gemm_f32(a, gather_div, w, w_is_kn: bool, N: int, K: int, seg: ExpertSegments, scatter: bool, y, bias=None,
+              rows_in=None, rows_out=None):
     """The grouped GEMMs of fp32 tensors (fp32 MFMA; see ck_grouped_gemm_f32)."""
-    cs = seg.c_struct()
+    cs = seg.c_struct(rows_in, rows_out)
     with torch.cuda.device(w.device):
         _C.check(
             _C.lib().ck_grouped_gemm_f32(
@@ -294,12 +313,12 @@ def _gemm_f32(a, gather_div, w, w_is_kn: bool, N: int, K: int, seg: ExpertSegmen
         )
 
 
-def _gemm(a, gather_div, w, seg: ExpertSegments, epilogue, y, y_t=None, aux=None, aux_in=None):
+def _gemm(a, gather_div, w, seg: ExpertSegments, epilogue, y, y_t=None, aux=None, aux_in=None, rows_in=None, rows_out=None):
     E, N, K = w.shape
     if w.dtype == torch.float32:
         assert epilogue in (_C.CK_EPI_GROUPED, _C.CK_EPI_SCATTER) and y_t is None and aux is None
-        return _gemm_f32(a, gather_div, w, False, N, K, seg, epilogue == _C.CK_EPI_SCATTER, y, aux_in)
-    cs = seg.c_struct()
+        return _gemm_f32(a, gather_div, w, False, N, K, seg, epilogue == _C.CK_EPI_SCATTER, y, aux_in, rows_in, rows_out)
+    cs = seg.c_struct(rows_in, rows_out)
     if gather_div > 0:  # gathered rows are addressed with 32-bit byte offsets from the start of `a` (the library is not
         # told how many rows `a` has, so this limit is checked here)
         assert a.numel() * a.element_size() < 2**32, "the token-order input of a grouped GEMM must stay below 4 GiB"
@@ -322,11 +341,9 @@ def _gemm(a, gather_div, w, seg: ExpertSegments, epilogue, y, y_t=None, aux=None
 
 def _bias_in_epilogue(seg: ExpertSegments, K: int) -> bool:
     """Whether ck_grouped_gemm takes the per-expert bias as an operand of its grouped / scatter epilogue (the bias joins
-    the fp32 accumulators and the output is rounded once, like F.linear). CK_GEMM_BIAS_FUSED=0 in the environment adds it
-    with its own kernel after the GEMM instead (two roundings; kept for comparison)."""
-    import os
-
-    return os.environ.get("CK_GEMM_BIAS_FUSED", "1") != "0"
+    the fp32 accumulators and the output is rounded once, like F.linear). options.bias_fused = False adds it with its
+    own kernel after the GEMM instead (two roundings; kept for comparison)."""
+    return options.bias_fused
 
 
 def _fp32(t: torch.Tensor) -> bool:
@@ -335,15 +352,15 @@ def _fp32(t: torch.Tensor) -> bool:
     return t.dtype == torch.float32
 
 
-def _gemm_dx(d_y, w, seg: ExpertSegments, epilogue, out):
+def _gemm_dx(d_y, w, seg: ExpertSegments, epilogue, out, rows_out=None):
     """out = d_y @ w[e] per expert, w [E, out_features, in_features] as the forward stores it: the input-gradient GEMM.
     Reads w contraction-strided where the kernel for that exists (256-row tiles, out_features % 64 == 0); otherwise
-    through a transposed copy."""
+    through a transposed copy. rows_out: the table a scatter epilogue writes through (default seg.row_slot)."""
     E, n_out, n_in = w.shape
     if w.dtype == torch.float32:
-        return _gemm_f32(d_y, 0, w, True, n_in, n_out, seg, epilogue == _C.CK_EPI_SCATTER, out)
-    if seg.align == 256 and n_out % 64 == 0 and _nn_enabled():
-        cs = seg.c_struct()
+        return _gemm_f32(d_y, 0, w, True, n_in, n_out, seg, epilogue == _C.CK_EPI_SCATTER, out, None, None, rows_out)
+    if seg.align == 256 and n_out % 64 == 0 and options.gemm_nn:
+        cs = seg.c_struct(None, rows_out)
 
         def launch():
             with torch.cuda.device(w.device):
@@ -360,13 +377,7 @@ def _gemm_dx(d_y, w, seg: ExpertSegments, epilogue, out):
         else:
             launch_timer.time(_EPILOGUE_NAMES[epilogue].replace("grouped_gemm<", "grouped_gemm_nn<"), (n_in, n_out), launch)
         return
-    _gemm(d_y, 0, _transpose_weights(w), seg, epilogue, out)
-
-
-def _nn_enabled() -> bool:
-    import os
-
-    return os.environ.get("CK_GEMM_NN", "1") != "0"  # measurement knob: 0 = always go through the transposed copy
+    _gemm(d_y, 0, _transpose_weights(w), seg, epilogue, out, rows_out=rows_out)
 
 
 def _gemm_dw(a_t, b_t, seg: ExpertSegments, dw):
@@ -417,21 +428,19 @@ def _dw_from_rows(max_rows: int, num_experts: int, align: int, *shapes: tuple[in
     the 384-wide tiles the transposed form can use (measured: fine-grained layer 4 % faster, Mixtral-shape layer 0.4 %).
     A function of sizes only, so that forward, backward and the traced (fake) implementations agree on which tensors
     exist."""
-    import os
-
-    ok = os.environ.get("CK_GEMM_DW_ROWS", "1") != "0"  # measurement knob: 0 = always the transposed form
-    return ok and align % 64 == 0 and all(min(m, n) >= 256 and m % 8 == 0 and n % 8 == 0 for m, n in shapes)
+    return options.dw_rows and align % 64 == 0 and all(min(m, n) >= 256 and m % 8 == 0 and n % 8 == 0 for m, n in shapes)
 
 
-def _group_rows(src, coeff, fan_out, seg: ExpertSegments, want_grouped: bool, want_transposed: bool):
-    """Padded grouped copy of `src` rows (fan_out == 0: src is already padded-grouped) and / or its transpose."""
+def _group_rows(src, coeff, fan_out, seg: ExpertSegments, want_grouped: bool, want_transposed: bool, rows=None):
+    """Padded grouped copy of `src` rows (fan_out == 0: src is already padded-grouped) and / or its transpose. rows: the
+    table the rows are read through (default seg.row_slot)."""
     H = src.size(-1)
     grouped = torch.empty(seg.max_rows, H, dtype=src.dtype, device=src.device) if want_grouped else None
     grouped_t = torch.empty(H, seg.ld_t, dtype=src.dtype, device=src.device) if want_transposed else None
     with torch.cuda.device(src.device):
         _C.check(
             _C.lib().ck_group_rows_padded(
-                _C.ptr(src), _C.ptr(coeff), fan_out, H, _C.ptr(seg.row_slot), _C.ptr(seg.seg_starts), _C.ptr(seg.counts),
+                _C.ptr(src), _C.ptr(coeff), fan_out, H, _C.ptr(seg.row_slot if rows is None else rows), _C.ptr(seg.seg_starts), _C.ptr(seg.counts),
                 _C.ptr(seg.tile_expert), seg.align, seg.max_rows, _C.ptr(grouped), _C.ptr(grouped_t), seg.ld_t,
                 _C.dtype_code(src.dtype), _C.stream(),
             )
@@ -791,3 +800,164 @@ def swiglu_experts(
         )[0]
     _C.require_gpu(x, w_fc, w_proj, gates)
     return _SwigluExperts.apply(x, w_fc, w_proj, gates.to(x.dtype), seg, act_kind, _gate_slot(gates))
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# the reference's own expert-linear interface: three index tensors, unpadded grouped rows
+# ---------------------------------------------------------------------------------------------------------------
+def bincount(x: torch.Tensor, minlength: int) -> torch.Tensor:
+    """Histogram of expert ids as the reference's helper returns it (triton_implementation/ops.py:19-28): int64 counts,
+    computed by the count kernel (ids outside [0, minlength) are not counted, where torch.bincount would grow or raise)."""
+    from .continuous_count import continuous_count_cute
+
+    return continuous_count_cute(x.reshape(-1), minlength).to(torch.int64)
+
+
+_segments_cache: list = []  # [(sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, versions, align, ExpertSegments)]
+
+
+@torch.no_grad()
+def segments_from_sorted(
+    sorted_expert_idxs: torch.Tensor, sorted_scattered_idxs: torch.Tensor, expert_offsets: torch.Tensor,
+    align: int | None = None,
+) -> ExpertSegments:
+    """The padded grouped layout for a sort the caller did: (sorted_expert_idxs, sorted_scattered_idxs) =
+    selected_experts.flatten().sort() and expert_offsets = bincount(...).cumsum(-1), the arguments of the reference's
+    expert linears (triton_implementation/__init__.py:82-83). One small launch; the result for the last two distinct
+    argument triples is kept, so that c_fc and c_proj of one layer call share it."""
+    _C.require_gpu(sorted_expert_idxs, sorted_scattered_idxs, expert_offsets)
+    assert sorted_expert_idxs.dim() == 1 and sorted_expert_idxs.shape == sorted_scattered_idxs.shape
+    assert sorted_expert_idxs.dtype == sorted_scattered_idxs.dtype and sorted_expert_idxs.dtype in (torch.int32, torch.long)
+    assert expert_offsets.dim() == 1 and expert_offsets.dtype in (torch.int32, torch.uint32, torch.long)
+    R, E = sorted_expert_idxs.numel(), expert_offsets.numel()
+    if align is None:
+        align = choose_align(R, E)
+    tensors = (sorted_expert_idxs, sorted_scattered_idxs, expert_offsets)
+    versions = tuple(t._version for t in tensors)
+    for entry in _segments_cache:
+        if all(a is b for a, b in zip(entry[0], tensors)) and entry[1] == versions and entry[2] == align:
+            return entry[3]
+    se, ss, off = (t.contiguous() for t in tensors)
+    lib = _C.lib()
+    dev = se.device
+    max_rows = lib.ck_sort_max_rows(R, E, align)
+    i32 = dict(dtype=torch.int32, device=dev)
+    seg = ExpertSegments(
+        sorted_expert_idxs=se, sorted_scattered_idxs=ss, counts=torch.empty(E, dtype=torch.uint32, device=dev), ends=off,
+        starts=None, seg_starts=torch.empty(E + 1, **i32), row_slot=torch.empty(max(max_rows, 1), **i32),
+        tile_expert=torch.empty(max(max_rows // align, 1), **i32), max_rows=max_rows, num_experts=E, align=align,
+        row_pos=torch.empty(max(max_rows, 1), **i32),
+    )
+    with torch.cuda.device(dev):
+        _C.check(
+            lib.ck_segments_from_sorted(
+                _C.ptr(se), _C.ptr(ss), int(se.dtype == torch.long), _C.ptr(off), int(off.dtype == torch.long), R, E, align,
+                _C.ptr(seg.counts), _C.ptr(seg.seg_starts), _C.ptr(seg.row_slot), _C.ptr(seg.row_pos), _C.ptr(seg.tile_expert),
+                _C.stream(),
+            )
+        )
+    _segments_cache.insert(0, (tensors, versions, align, seg))
+    del _segments_cache[2:]
+    return seg
+
+
+class _ScatteredExperts(torch.autograd.Function):
+    """One expert linear on the reference's index tensors (triton_implementation/ops.py:143-292), w [E, N, K] as the
+    module stores it. Input rows: token order [T, K] read through sorted_scattered_idxs // k, or (grouped_in) unpadded
+    grouped rows [R, K] in sorted order. Output: [R, N] in (token, slot) order, or (grouped_out) in sorted order, or
+    (gates [T, fan]) the gated sum over a token's slots [T, N]. The GEMM runs on the padded layout and reads / writes the
+    caller's rows through the row tables, so no padded copy of the input or output is made in the forward pass."""
+
+    @staticmethod
+    def forward(ctx, x, w, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, gates, grouped_in, grouped_out,
+                bias=None, gate_slot=None):
+        assert not (gates is not None and grouped_out), "gated outputs are combined per token, not grouped"
+        seg = segments_from_sorted(sorted_expert_idxs, sorted_scattered_idxs, expert_offsets)
+        x = x.contiguous()
+        w = w.contiguous()
+        E, N, K = w.shape
+        R = sorted_expert_idxs.numel()
+        assert x.size(-1) == K and x.size(0) == (R if grouped_in else R // k), "input rows do not match the index tensors"
+        out = torch.empty(R, N, dtype=x.dtype, device=x.device)
+        fused_bias = bias is not None and (_fp32(x) or _bias_in_epilogue(seg, K))
+        _gemm(
+            x, 1 if grouped_in else k, w, seg, _C.CK_EPI_SCATTER, out, aux_in=bias.contiguous() if fused_bias else None,
+            rows_in=seg.row_pos if grouped_in else seg.row_slot, rows_out=seg.row_pos if grouped_out else seg.row_slot,
+        )
+        if bias is not None and not fused_bias:
+            row_expert = sorted_expert_idxs.to(torch.int32) if grouped_out else _slot_experts(seg)
+            _add_expert_bias(out, bias.contiguous(), seg, row_expert)
+        expanded = None
+        if gates is not None:
+            gates = gates.contiguous()
+            T, fan = gates.shape
+            assert T * fan == R, "gates do not match the index tensors"
+            expanded = out
+            out, _ = _combine(expanded, gates, T, fan, N)
+        ctx.save_for_backward(x, w, gates, expanded)
+        ctx.seg, ctx.k, ctx.grouped_in, ctx.grouped_out, ctx.gate_slot = seg, k, grouped_in, grouped_out, gate_slot
+        return out
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, w, gates, expanded = ctx.saved_tensors
+        seg, k, grouped_in, grouped_out = ctx.seg, ctx.k, ctx.grouped_in, ctx.grouped_out
+        E, N, K = w.shape
+        grad_out = grad_out.contiguous()
+        need = ctx.needs_input_grad
+        need_x, need_w, need_gates = need[0], need[1], need[6]
+        need_bias = len(need) > 9 and need[9]
+        d_x = d_w = d_gates = d_bias = None
+        # the output gradient as padded grouped rows: what both the weight- and the input-gradient GEMM read
+        if gates is not None:
+            T, fan = gates.shape
+            if need_gates:
+                d_gates = _gate_grad(expanded, grad_out, T, fan, N, gates.dtype, ctx.gate_slot)
+            d_y, _ = _group_rows(grad_out, gates, fan, seg, True, False)
+        elif grouped_out:
+            d_y, _ = _group_rows(grad_out, None, 1, seg, True, False, rows=seg.row_pos)
+        else:
+            d_y, _ = _group_rows(grad_out, None, 1, seg, True, False)
+        if need_bias:
+            d_bias = _expert_bias_grad(d_y, seg)
+        if need_w:
+            x_g, _ = _group_rows(x, None, 1 if grouped_in else k, seg, True, False, rows=seg.row_pos if grouped_in else None)
+            d_w = torch.empty_like(w)
+            if _fp32(x) or _dw_from_rows(seg.max_rows, E, seg.align, (N, K)):
+                _gemm_dw_rows(d_y, x_g, seg, d_w)
+            else:
+                _, d_y_t = _group_rows(d_y, None, 0, seg, False, True)
+                _, x_t = _group_rows(x_g, None, 0, seg, False, True)
+                _gemm_dw(d_y_t, x_t, seg, d_w)
+        if need_x:
+            R = seg.sorted_expert_idxs.numel()
+            d_rows = torch.empty(R, K, dtype=x.dtype, device=x.device)
+            _gemm_dx(d_y, w, seg, _C.CK_EPI_SCATTER, d_rows, rows_out=seg.row_pos if grouped_in else seg.row_slot)
+            d_x = d_rows if grouped_in or k == 1 else _combine(d_rows, None, x.size(0), k, K)[0]
+        return d_x, d_w, None, None, None, None, d_gates, None, None, d_bias, None
+
+
+def scattered_experts(
+    inputs: torch.Tensor, expert_weights: torch.Tensor, k: int, sorted_expert_idxs: torch.Tensor,
+    sorted_scattered_idxs: torch.Tensor, expert_offsets: torch.Tensor, gates: torch.Tensor | None = None,
+    grouped_in: bool = False, grouped_out: bool = False, bias: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """The reference's scattered_experts (triton_implementation/ops.py:295-316), same arguments in the same order:
+    expert_weights is the [E, in, out] VIEW `weight.permute(0, 2, 1)` of an [E, out, in] parameter (any other layout is
+    copied). `bias` [E, out] is this build's addition (the reference's launcher has none and its module drops the bias)."""
+    w = expert_weights.permute(0, 2, 1)  # back to the parameter's own layout: no copy when the argument was the view
+    _check_expert_dtypes(inputs, w)
+    assert bias is None or (bias.dtype == inputs.dtype and bias.shape == w.shape[:2]), "bias should be [E, out] in x.dtype"
+    if gates is not None:
+        gates_in = gates
+        gates = gates.to(inputs.dtype)
+    if is_tracing():
+        out = _ops.scattered_experts(
+            inputs, w, gates, bias, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, k, grouped_in, grouped_out
+        )
+        return out[0]
+    _C.require_gpu(inputs, w, gates, bias, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets)
+    return _ScatteredExperts.apply(
+        inputs, w, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, gates, grouped_in, grouped_out, bias,
+        _gate_slot(gates_in) if gates is not None else None,
+    )

@@ -60,6 +60,12 @@ class MoE_Torch(MoE):
             top, selected = router_logits.topk(self.top_k, dim=-1)
         return router_logits, torch.softmax(top.float(), dim=-1).type_as(hidden_states), selected
 
+    def _compute_expert_assignment(self, router_weights, selected_experts):
+        """torch_implementation.py:171-193 with a stable argsort (the reference's is stable only incidentally)."""
+        flat = selected_experts.flatten()
+        order = flat.argsort(stable=True)
+        return order // self.top_k, router_weights.flatten()[order], flat.bincount(minlength=self.num_experts)
+
     def _compute_experts(self, hidden_states, router_weights, selected_experts):
         out = torch.zeros_like(hidden_states)
         for e in range(self.num_experts):

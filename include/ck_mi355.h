@@ -33,8 +33,18 @@ extern "C" {
 
 /* Message for the last non-zero return on this thread ("" if none). Host pointer, valid until the next failing call. */
 const char* ck_last_error_string(void);
-/* ABI revision of the library; bumps when a signature changes. */
+/* ABI revision of the library; bumps when a signature or a struct changes. */
 int32_t ck_abi_version(void);
+/* Test and measurement hook, no counterpart in the reference: chooses, process-wide, between kernels of this library that
+ * compute the same result. The defaults are what the library runs in production; nothing here changes a result beyond
+ * the tolerance of the kernels' own tests. Not meant to be changed while other threads issue launches.
+ *   "gemm_line_kernel"       (default 1)  0: the 16-bit grouped GEMMs always run on the general kernel
+ *   "gemm_register_pipeline" (default 0)  1: the general kernel stages its operands through registers
+ *   "gemm_four_waves"        (default 0)  1: the general kernel's direct-to-LDS pipeline with 4 waves instead of 8
+ *   "trace_buffer"           (default 0)  device address (as an integer) that builds compiled with -DCK_STAMP write
+ *                                         per-wave cycle counts to; product builds never read it
+ * Unknown names return CK_ERR_ARG. */
+int ck_debug_set_option(const char* name, int64_t value);
 
 /* ---------------------------------------------------------------------------------------------------------------
  * (a) expert histogram + offsets
@@ -109,6 +119,20 @@ int ck_sort_by_expert(const void* expert_ids, int32_t ids_are_i64, int64_t R, in
                       int32_t* sorted_expert_idxs, int32_t* sorted_scattered_idxs, uint32_t* counts, uint32_t* ends,
                       uint32_t* starts, int32_t* seg_starts, int32_t* row_slot, int32_t* tile_expert,
                       uint32_t* workspace, void* stream);
+/* The tile-aligned segment tables from a sort the caller already has -- the three index tensors the reference's expert
+ * linears take: sorted_expert_idxs, sorted_scattered_idxs = selected_experts.flatten().sort() and expert_offsets =
+ * bincount(...).cumsum(-1) (inclusive ends) -- cute_kernels/kernels/scattermoe/triton_implementation/__init__.py:14-36,82-83,
+ * ops.py:295-316. Both index tensors int32 or both int64 (torch.sort returns int64); offsets int32 / uint32 or int64.
+ * Outputs as ck_sort_by_expert writes them (counts, seg_starts, row_slot, tile_expert), plus
+ *   row_pos[max_rows] -- padded row p of expert e holds sorted position starts[e] + p - seg_starts[e]: the row of an
+ *                        UNPADDED grouped tensor [R, *] (the reference's grouped_in / grouped_out layout) that padded row p
+ *                        stands for. Used as ck_segments::row_slot with a_gather_div = 1 to read such a tensor, and as
+ *                        ck_segments::row_slot_out to write one.
+ * One launch, no workspace. A position whose expert id is outside [0, E) or outside its expert's offset range owns no row. */
+int ck_segments_from_sorted(const void* sorted_expert_idxs, const void* sorted_scattered_idxs, int32_t idxs_are_i64,
+                            const void* expert_offsets, int32_t offsets_are_i64, int64_t R, int32_t E, int32_t align,
+                            uint32_t* counts, int32_t* seg_starts, int32_t* row_slot, int32_t* row_pos,
+                            int32_t* tile_expert, void* stream);
 
 /* ---------------------------------------------------------------------------------------------------------------
  * (b3) token-row gather / gated combine
@@ -166,10 +190,13 @@ typedef struct ck_segments {
   const int32_t* seg_starts;  /* [E + 1] */
   const uint32_t* counts;     /* [E] */
   const int32_t* tile_expert; /* [max_rows / align] */
-  const int32_t* row_slot;    /* [max_rows] */
+  const int32_t* row_slot;    /* [max_rows]: the A row a padded row reads (divided by a_gather_div) */
   int64_t max_rows;
   int32_t num_experts;
   int32_t align;
+  const int32_t* row_slot_out; /* [max_rows] or NULL (= row_slot): the output row a padded row writes in the scatter
+                                  epilogues. Differs from row_slot when input and output are indexed differently, e.g. token
+                                  rows in, unpadded grouped rows out (row_pos of ck_segments_from_sorted). */
 } ck_segments;
 
 /* Y = A_e * W[e]^T for every expert segment e. W [E, N, K].
@@ -178,7 +205,8 @@ typedef struct ck_segments {
  * Epilogue, selected by `epilogue`:
  *   CK_EPI_GROUPED        : y [max_rows, N] padded-grouped (valid rows only); y_t [N, ld_t] transposed copy with
  *                           zeros in pad rows, optional (NULL to skip)
- *   CK_EPI_SCATTER        : y [R, N]: valid row p is written to row row_slot[p] (back to (token, slot) order)
+ *   CK_EPI_SCATTER        : y [R, N]: valid row p is written to row row_slot_out[p] (row_slot[p] when that is NULL: back to
+ *                           (token, slot) order)
  *                           both: aux_in, if not NULL, is a bias [E, N] whose row e joins the fp32 accumulators of expert
  *                           e's rows before the one rounding (F.linear with a bias, torch_implementation.py:42)
  *   CK_EPI_GELU_TANH      : as CK_EPI_GROUPED (bias included), and aux [max_rows, N] = tanh-approximated GELU of y, computed
@@ -211,8 +239,9 @@ int ck_grouped_gemm(const void* a, int32_t a_gather_div, const void* w, int32_t 
  * fixed order (results do not depend on arrival order) and runs the epilogue. Grouped and scatter epilogues of the
  * 256-row-tile kernel; every other case behaves like ck_grouped_gemm. No counterpart in the reference (its launches
  * are not tile-quantised the same way).
- * workspace: ck_grouped_gemm_workspace_bytes() bytes, 16-byte aligned; its last 512 bytes (arrival counters) must be zero
- * before the first call and are zero again after every call, so one zero-initialised buffer per stream is reusable.
+ * workspace: ck_grouped_gemm_workspace_bytes() bytes, 16-byte aligned, no initial contents required (the arrival words at
+ * its end carry the launch's own epoch, so whatever an earlier or an interrupted launch left there reads as "nobody has
+ * arrived"). One buffer per stream: launches that may run concurrently must not share one.
  * workspace NULL or too small: never split. */
 int64_t ck_grouped_gemm_workspace_bytes(void);
 int ck_grouped_gemm_ws(const void* a, int32_t a_gather_div, const void* w, int32_t N, int32_t K,

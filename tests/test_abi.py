@@ -29,7 +29,7 @@ def test_library_exports_every_declared_symbol():
     for name in declared:
         assert hasattr(lib, name), f"{name} is declared in ck_mi355.h but not exported"
     assert declared == set(_C.EXPORTED_SYMBOLS), "ctypes signature table and header disagree"
-    assert lib.ck_abi_version() == 1
+    assert lib.ck_abi_version() == 2
 
 
 def test_argument_validation_returns_error_and_message():
