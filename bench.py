@@ -139,7 +139,7 @@ def zipf_bias(logits, k: int, s: float = 1.0):
     return best[2], best[3], best[1]
 
 
-def build_layer(dev):
+def build_layer(dev, reverse_load: bool = False):
     import torch
 
     import cute_kernels
@@ -150,6 +150,8 @@ def build_layer(dev):
     x = torch.randn(T, H, generator=torch.Generator().manual_seed(SEED)).to(torch.bfloat16).to(dev)
     with torch.no_grad():
         bias, freq, c = zipf_bias(moe.gate(x), TOP_K, 1.0)
+    if reverse_load:  # the same loads with the heaviest expert last (a measurement of tile-order robustness)
+        bias, freq = bias.flip(0), freq.flip(0)
     bias = bias.to(torch.bfloat16)
     # the router has no bias parameter (torch_implementation.py:83 of the reference): skew goes in through a hook
     moe.gate.register_forward_hook(lambda mod, inp, out: out + bias)
@@ -519,6 +521,8 @@ def main() -> int:
     ap.add_argument("--lib", default=None, metavar="FILE.so",
                     help="load this build of the library (a measurement build from build.py --define ... --output) instead of the product one")
     ap.add_argument("--zeros", action="store_true", help="with --only-gemm: all-zero operands")
+    ap.add_argument("--reverse-load", action="store_true",
+                    help="the C3 step with the expert loads reversed (heaviest expert last); not the headline workload")
     ap.add_argument("--no-split", action="store_true", help="never split the last round of GEMM tiles (A/B measurement)")
     ap.add_argument("--summarize-pmc", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
                     help="no GPU work: reduce two rocprofv3 --pmc output directories to profiles/grouped_gemm_c3_hbm_traffic.txt")
@@ -552,7 +556,7 @@ def main() -> int:
     if args.only_yardstick:
         print(json.dumps({"library_gemm_yardstick": library_gemm_yardstick(dev)}))
         return 0
-    moe, x, grad_out, freq, zipf_c = build_layer(dev)
+    moe, x, grad_out, freq, zipf_c = build_layer(dev, args.reverse_load)
     x.requires_grad_()
 
     if args.copy_calibration:
@@ -628,7 +632,8 @@ def main() -> int:
         "dtype": "bf16",
         "data": "synthetic",
         "config": {
-            "workload": "C3 Mixtral-shape MoE layer fwd+bwd: T=16384 H=4096 E=8 top-2 I=14336 SwiGLU, Zipf(1.0) load",
+            "workload": "C3 Mixtral-shape MoE layer fwd+bwd: T=16384 H=4096 E=8 top-2 I=14336 SwiGLU, Zipf(1.0) load"
+            + (" REVERSED (heaviest expert last)" if args.reverse_load else ""),
             "routed_rows": R,
             "flops_per_step": flops_step,
             "expert_load": [round(f, 4) for f in freq],

@@ -105,6 +105,28 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
     }
     mt = m_major ? a : b;
     nt = m_major ? b : a;
+    // `expert` so far is a position in the launch order. Experts differ in contraction length (their row counts), and
+    // the hardware hands tiles out in block order: the longest contractions go first, so that the tiles still running
+    // when the grid drains are the short ones (position r takes the expert with the r-th largest count, ties by index).
+    // Up to NT experts: one thread ranks one expert against the counts parked in LDS (the stages are not in use yet).
+    if (prm.num_experts <= NT) {
+      int* sh = reinterpret_cast<int*>(lds_c);
+      const int E = prm.num_experts;
+      if (tid < E) sh[tid] = (int)prm.counts[tid];
+      __syncthreads();
+      if (tid < E) {
+        const int c = sh[tid];
+        int rank = 0;
+        for (int i = 0; i < E; ++i) {
+          const int ci = sh[i];
+          rank += (ci > c || (ci == c && i < tid)) ? 1 : 0;
+        }
+        if (rank == expert) sh[NT] = tid;
+      }
+      __syncthreads();
+      expert = sh[NT];
+      __syncthreads();  // everyone holds its expert before the first loads land in the stages
+    }
     k_begin = prm.seg_starts[expert];
     k_len = (int)((prm.counts[expert] + BK - 1) / BK * BK);  // the transposed operands are zero up to the tile boundary
   } else {
@@ -283,13 +305,13 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   const uint32_t wave_b = __builtin_amdgcn_readfirstlane(lds_base + wave * B_LD * 1024);
   // load g of K step `step`: g < A_LD: a wave-load of A, else of the weight operand, into stage step % 2
   auto issue_one = [&](int step, int g) {
+    const uint32_t st = (uint32_t)((step & (NSTAGE - 1)) * kStageBytes);
     // measurement builds: bit 16 = both operands re-read the first two K steps (L2 hits), 512 / 1024 = only A / only B does
     const int64_t kb = (CK_ABLATE & 16) ? (int64_t)(step & 1) * kRowBytes : (int64_t)step * kRowBytes;
     const int64_t kb_hot = (int64_t)(step & 1) * kRowBytes;
     const int64_t kb_b = BT ? (int64_t)((CK_ABLATE & (16 | 1024)) ? (step & 1) : step) * BK * prm.ldw * 2
                             : ((CK_ABLATE & 1024) ? kb_hot : kb);  // BT: 64 contraction rows further down
     const int64_t kb_a = AT ? (int64_t)step * BK * prm.lda * 2 : ((CK_ABLATE & 512) ? kb_hot : kb);
-    const uint32_t st = (uint32_t)((step & (NSTAGE - 1)) * kStageBytes);
     if (g < A_LD) dma16(a_base_u + kb_a, a_off[g], wave_a + st + g * 1024);
     else dma16(b_base_u + kb_b, b_off[g - A_LD], wave_b + (uint32_t)kAStage + st + (g - A_LD) * 1024);
   };
