@@ -33,9 +33,31 @@ PEAK_HBM_GBS = 8000.0  # MI355X HBM3E
 TRAFFIC_SUMMARY = os.path.join(ROOT, "profiles", "grouped_gemm_c3_hbm_traffic.txt")
 
 
+def canonical_kernel_name(name: str) -> str:
+    """One spelling for the grouped GEMM kernel's instantiations, whichever way a rocprofv3 output file spells them: the
+    kernel trace and the counter files of one run mix mangled names (..grouped_gemm_line_kernelIDF16bLi4ELi256ELb1ELi2ELb0EE..),
+    demangled ones, and a mis-demangled form in which `DF16bLi1E` (bf16, 1) comes out as `bool _Accum, int, E`.
+    -> "grouped_gemm_line_kernel<bf16, 4, 256, true, 2, false>"; other kernels keep their name."""
+    import re
+
+    m = re.search(r"grouped_gemm_line_kernelI(DF16b|DF16_|Dh|f)Li(\d+)ELi(\d+)ELb([01])ELi(\d+)ELb([01])E", name)
+    if m:
+        dtype = {"DF16b": "bf16", "DF16_": "f16", "Dh": "f16", "f": "f32"}[m.group(1)]
+        flag = lambda b: "true" if b == "1" else "false"
+        return f"grouped_gemm_line_kernel<{dtype}, {m.group(2)}, {m.group(3)}, {flag(m.group(4))}, {m.group(5)}, {flag(m.group(6))}>"
+    m = re.search(r"grouped_gemm_line_kernel<(.*?)>\(", name + "(")
+    if m:
+        args = [a.strip() for a in m.group(1).split(",")]
+        if args[:3] == ["bool _Accum", "int", "E"]:  # the mis-demangled (bf16, 1)
+            args = ["bf16", "1"] + args[3:]
+        args[0] = {"__hip_bfloat16": "bf16", "__bf16": "bf16", "_Float16": "f16", "__half": "f16"}.get(args[0], args[0])
+        return "grouped_gemm_line_kernel<" + ", ".join(args) + ">"
+    return name
+
+
 def load_traffic_summary(path: str = TRAFFIC_SUMMARY) -> dict:
-    """kernel name (as the kernel trace spells it) -> HBM bytes per launch, from the summary's tab-separated lines
-    `kernel<TAB>launches<TAB>fetch KiB per launch (scaled)<TAB>write KiB per launch (scaled)`."""
+    """kernel name (canonical_kernel_name) -> HBM bytes per launch, from the summary's tab-separated lines
+    `kernel<TAB>launches<TAB>fetch KiB per launch (scaled)<TAB>write KiB per launch (scaled)<TAB>name in the counter file`."""
     table = {}
     if not os.path.exists(path):
         return table
@@ -43,8 +65,8 @@ def load_traffic_summary(path: str = TRAFFIC_SUMMARY) -> dict:
         for line in f:
             if line.startswith("#") or not line.strip():
                 continue
-            name, _launches, fetch_kib, write_kib = line.rstrip("\n").split("\t")
-            table[name] = (float(fetch_kib) + float(write_kib)) * 1024.0
+            name, _launches, fetch_kib, write_kib = line.rstrip("\n").split("\t")[:4]
+            table[canonical_kernel_name(name)] = (float(fetch_kib) + float(write_kib)) * 1024.0
     return table
 
 
@@ -56,25 +78,26 @@ def summarize_pmc(fetch_dir: str, write_dir: str, out_path: str = TRAFFIC_SUMMAR
     import glob
 
     def per_kernel(directory: str, counter: str) -> dict:
-        sums: dict = {}
+        sums: dict = {}  # name -> [sum, launches, largest single reading]
         for path in glob.glob(os.path.join(directory, "**", "*counter_collection.csv"), recursive=True):
             with open(path, newline="") as f:
                 for row in csv.DictReader(f):
                     if row.get("Counter_Name") != counter:
                         continue
-                    rec = sums.setdefault(row["Kernel_Name"], [0.0, 0])
-                    rec[0] += float(row["Counter_Value"])
+                    rec = sums.setdefault(row["Kernel_Name"], [0.0, 0, 0.0])
+                    value = float(row["Counter_Value"])
+                    rec[0] += value
                     rec[1] += 1
+                    rec[2] = max(rec[2], value)
         return sums
 
     def copy_factor(sums: dict, what: str) -> float:
-        # the calibration copy is the one elementwise copy kernel of 2^30 bytes: the largest per-launch reading among
-        # kernels whose name says "copy"
-        cands = [(v[0] / v[1], k) for k, v in sums.items() if "copy" in k.lower() and v[1] > 0]
-        if not cands:
-            raise SystemExit(f"no copy kernel in the {what} run: was bench.py run with --copy-calibration?")
-        reading = max(cands)[0]
-        return float(1 << 20) / reading
+        # the calibration copy (2^30 bytes, torch's device-to-device copy) is the largest single launch among the kernels
+        # whose name says "copy" (the runtime's copyBuffer kernel also serves every small copy of the run)
+        cands = [v[2] for k, v in sums.items() if "copy" in k.lower()]
+        if not cands or max(cands) < float(1 << 18):
+            raise SystemExit(f"no 1 GiB copy in the {what} run: was bench.py run with --copy-calibration?")
+        return float(1 << 20) / max(cands)
 
     fetch, write = per_kernel(fetch_dir, "FETCH_SIZE"), per_kernel(write_dir, "WRITE_SIZE")
     ff, wf = copy_factor(fetch, "FETCH_SIZE"), copy_factor(write, "WRITE_SIZE")
@@ -82,12 +105,12 @@ def summarize_pmc(fetch_dir: str, write_dir: str, out_path: str = TRAFFIC_SUMMAR
         f.write("# HBM traffic per launch of the grouped GEMM kernels in `python bench.py --copy-calibration` (C3 workload)\n")
         f.write(f"# from rocprofv3 --pmc FETCH_SIZE and --pmc WRITE_SIZE (KiB per dispatch), scaled by {ff:.3f} and {wf:.3f}:\n")
         f.write("# what makes the same counter read 2^20 KiB for the run's own 1 GiB device copy\n")
-        f.write("# kernel\tlaunches\tfetch_KiB_per_launch\twrite_KiB_per_launch\n")
-        for name in sorted(fetch):
+        f.write("# kernel\tlaunches\tfetch_KiB_per_launch\twrite_KiB_per_launch\tname_in_the_counter_file\n")
+        for name in sorted(fetch, key=canonical_kernel_name):
             if "grouped_gemm" not in name or name not in write:
                 continue
             fv, wv = fetch[name], write[name]
-            f.write(f"{name}\t{fv[1]}\t{fv[0] / fv[1] * ff:.1f}\t{wv[0] / wv[1] * wf:.1f}\n")
+            f.write(f"{canonical_kernel_name(name)}\t{fv[1]}\t{fv[0] / fv[1] * ff:.1f}\t{wv[0] / wv[1] * wf:.1f}\t{name}\n")
     print(f"wrote {out_path}")
 
 
@@ -109,11 +132,7 @@ def traffic_for(launch_name: str, summary_path: str = TRAFFIC_SUMMARY):
     want = ROCPROF_KERNEL.get(launch_name)
     if want is None:
         return None
-    norm = lambda n: n.replace(" ", "").replace("__hip_bfloat16", "bf16").replace("__bf16", "bf16")
-    for name, nbytes in load_traffic_summary(summary_path).items():
-        if norm(want) in norm(name):
-            return nbytes
-    return None
+    return load_traffic_summary(summary_path).get(want)
 
 # workload: configs[2] of the baseline, the configuration its headline metric (MoE fwd+bwd TFLOP/s) is quoted on
 T, H, E, TOP_K, I = 16384, 4096, 8, 2, 14336

@@ -45,3 +45,21 @@ def test_traced_max_rows_formula_matches_the_library():
         for E in (1, 8, 64, 128):
             for align in (128, 256):
                 assert compile_ops._max_rows(R, E, align) == lib.ck_sort_max_rows(R, E, align)
+
+
+class _LayerOnTheReferenceInterface(ck.MoE):
+    """_compute_experts written against the expert linears' reference call form (triton_implementation/__init__.py:79-103)."""
+
+    def _compute_experts(self, hidden_states, router_weights, selected_experts):
+        sorted_expert_idxs, sorted_scattered_idxs = selected_experts.flatten().sort()
+        expert_offsets = ck.scattermoe.bincount(sorted_expert_idxs, self.num_experts).cumsum(-1)
+        hidden_states = self.c_fc(hidden_states, self.top_k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, grouped_out=True)
+        hidden_states = self.act(hidden_states)
+        return self.c_proj(
+            hidden_states, 1, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, grouped_in=True, gates=router_weights
+        )
+
+
+def test_layer_on_the_reference_interface_traces():
+    moe = _LayerOnTheReferenceInterface(4, 2, 64, 32, torch.nn.GLU(), True, False, 0.02).to(torch.bfloat16)
+    _traces(lambda a: moe(a)[0], torch.randn(16, 64, dtype=torch.bfloat16, requires_grad=True))

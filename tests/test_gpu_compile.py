@@ -174,3 +174,30 @@ def test_cute_inductor_rewrites_match_the_torch_model(device, dtype, then_induct
         # weight gradients sum 333 rows: compare in units of the gradient's own scale
         scale = max(1.0, float(b.float().abs().max()))
         torch.testing.assert_close(a.float() / scale, b.float() / scale, **tol)
+
+
+def test_layer_on_the_reference_interface_compiled(device):
+    """A layer whose _compute_experts calls the expert linears the way the reference's accelerated layer does
+    (scattered_experts on sort / bincount / cumsum results) under torch.compile(fullgraph=True, backend="aot_eager"):
+    same kernels as eager, so everything that does not pass through d_gates is bit-identical (see the layer test above)."""
+    from test_compile_trace import _LayerOnTheReferenceInterface
+
+    torch.manual_seed(3)
+    moe = _LayerOnTheReferenceInterface(8, 2, 128, 256, ck.swiglu_packed_cute, True, False, 0.02).to(torch.bfloat16).to(device)
+    x = torch.randn(700, 128, dtype=torch.bfloat16, device=device)
+    xe, xc = x.clone().requires_grad_(), x.clone().requires_grad_()
+    y, _ = moe(xe)
+    y.float().square().sum().backward()
+    eager_grads = {n: p.grad.clone() for n, p in moe.named_parameters()}
+    for p in moe.parameters():
+        p.grad = None
+    compiled = torch.compile(moe, fullgraph=True, backend="aot_eager")
+    yc, _ = compiled(xc)
+    assert torch.equal(yc, y)
+    yc.float().square().sum().backward()
+    for n, p in moe.named_parameters():
+        if n == "gate.weight":
+            torch.testing.assert_close(eager_grads[n].float(), p.grad.float(), rtol=2e-2, atol=2e-2 * float(p.grad.float().abs().max()))
+        else:
+            assert torch.equal(eager_grads[n], p.grad), n
+    torch.testing.assert_close(xe.grad.float(), xc.grad.float(), rtol=2e-2, atol=2e-2 * float(xc.grad.float().abs().max()))

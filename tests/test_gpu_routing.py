@@ -181,7 +181,8 @@ def _check_sort(device, ids: torch.Tensor, E: int, align: int):
     return seg
 
 
-@pytest.mark.parametrize("R,E", [(32768, 64), (32768, 8), (65536, 64), (524288, 128), (1, 128), (2, 2), (1000, 1), (4097, 72), (8, 4096)])
+@pytest.mark.parametrize("R,E", [(32768, 64), (32768, 8), (65536, 64), (524288, 128), (1, 128), (2, 2), (1000, 1), (4097, 72), (8, 4096),
+                                  (65537, 64), (100000, 8), (40000, 800), (40000, 900)])
 @pytest.mark.parametrize("align", [128, 256])
 @pytest.mark.parametrize("dtype", [torch.int32, torch.long])
 def test_sort_by_expert_matches_oracle(device, R, E, align, dtype):
