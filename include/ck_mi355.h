@@ -342,9 +342,12 @@ int64_t ck_rmsnorm_bwd_partial_rows(int64_t B);
 int ck_rmsnorm_bwd(const void* x, const void* weight, const void* d_out, const float* rstd, float eps, int64_t B,
                    int32_t H, void* d_x, float* d_weight_partial, float* d_weight, int32_t dtype, void* stream);
 
-/* RMSNorm fused ahead of the router: one pass over x that writes y = rmsnorm(x) (as ck_rmsnorm_fwd), rstd, and the router
- * logits y @ gate_weight^T computed from the 16-bit y while the rows are in registers (fp32 accumulation, rounded to the
- * rows' dtype); with x8 / scale8, also the e4m3 rows and per-row scales that ck_quant_rows_e4m3 would derive from y.
+/* RMSNorm fused ahead of the router: one pass over x that writes y = rmsnorm(x), rstd, and the router logits
+ * y @ gate_weight^T computed from the 16-bit y while the rows are in registers (fp32 accumulation, rounded to the rows'
+ * dtype); with x8 / scale8, also the e4m3 rows and per-row scales that ck_quant_rows_e4m3 would derive from y.
+ * y agrees with ck_rmsnorm_fwd's to within one rounding step of the rows' dtype, not bit for bit: this kernel sums the
+ * squares of a row in another order, so rstd may differ in its last bits (about one element of y in a thousand then
+ * rounds the other way). Logits, x8 and scale8 are exact functions of the y this kernel writes.
  * Replaces, as one kernel: rmsnorm_forward_triton -- cute_kernels/kernels/rmsnorm/triton_implementation/forward.py:14-53 --
  *           and the router's linear layer, self.gate(hidden_states) -- cute_kernels/kernels/scattermoe/
  *           torch_implementation.py:122-124 (and the per-row quantiser ahead of ck_grouped_gemm_fp8).
