@@ -879,6 +879,10 @@ class _ScatteredExperts(torch.autograd.Function):
         R = sorted_expert_idxs.numel()
         assert x.size(-1) == K and x.size(0) == (R if grouped_in else R // k), "input rows do not match the index tensors"
         out = torch.empty(R, N, dtype=x.dtype, device=x.device)
+        ctx.seg, ctx.k, ctx.grouped_in, ctx.grouped_out, ctx.gate_slot = seg, k, grouped_in, grouped_out, gate_slot
+        if R == 0:  # no routed rows: nothing to launch
+            ctx.save_for_backward(x, w, gates, None)
+            return out if gates is None else torch.zeros(gates.size(0), N, dtype=x.dtype, device=x.device)
         fused_bias = bias is not None and (_fp32(x) or _bias_in_epilogue(seg, K))
         _gemm(
             x, 1 if grouped_in else k, w, seg, _C.CK_EPI_SCATTER, out, aux_in=bias.contiguous() if fused_bias else None,
@@ -895,7 +899,6 @@ class _ScatteredExperts(torch.autograd.Function):
             expanded = out
             out, _ = _combine(expanded, gates, T, fan, N)
         ctx.save_for_backward(x, w, gates, expanded)
-        ctx.seg, ctx.k, ctx.grouped_in, ctx.grouped_out, ctx.gate_slot = seg, k, grouped_in, grouped_out, gate_slot
         return out
 
     @staticmethod
@@ -908,6 +911,12 @@ class _ScatteredExperts(torch.autograd.Function):
         need_x, need_w, need_gates = need[0], need[1], need[6]
         need_bias = len(need) > 9 and need[9]
         d_x = d_w = d_gates = d_bias = None
+        if seg.sorted_expert_idxs.numel() == 0:  # no routed rows: every gradient is zero
+            return (
+                torch.zeros_like(x) if need_x else None, torch.zeros_like(w) if need_w else None, None, None, None, None,
+                torch.zeros_like(gates) if need_gates and gates is not None else None, None, None,
+                torch.zeros(E, N, dtype=w.dtype, device=w.device) if need_bias else None, None,
+            )
         # the output gradient as padded grouped rows: what both the weight- and the input-gradient GEMM read
         if gates is not None:
             T, fan = gates.shape

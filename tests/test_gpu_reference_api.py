@@ -227,3 +227,34 @@ def test_compute_expert_assignment(device):
     assert np.array_equal(fan_in.cpu().numpy(), want_s // k)
     assert np.array_equal(freq.cpu().numpy(), io.count(ids, E)) and freq.dtype == torch.int64
     assert torch.equal(batch_gates.cpu(), weights.flatten()[torch.from_numpy(want_s.astype(np.int64))])
+
+
+def test_no_tokens(device):
+    """Zero tokens (an empty micro-batch) pass through the reference interface and the layer: empty results of the right
+    shapes, zero gradients, no launch on NULL pointers."""
+    E, K, N, k = 4, 64, 128, 2
+    w1 = torch.randn(E, N, K, device=device, dtype=torch.bfloat16, requires_grad=True)
+    w2 = torch.randn(E, K, N, device=device, dtype=torch.bfloat16, requires_grad=True)
+    sel = torch.zeros(0, k, device=device, dtype=torch.long)
+    se, ss = sel.flatten().sort(stable=True)
+    off = scattermoe.bincount(se, E).cumsum(-1)
+    assert off.tolist() == [0] * E
+    x = torch.randn(0, K, device=device, dtype=torch.bfloat16, requires_grad=True)
+    gates = torch.zeros(0, k, device=device, dtype=torch.bfloat16, requires_grad=True)
+    h = cute_kernels.scattered_experts(x, w1.permute(0, 2, 1), k, se, ss, off, None, False, True)
+    assert h.shape == (0, N)
+    y = cute_kernels.scattered_experts(h, w2.permute(0, 2, 1), 1, se, ss, off, gates, True, False)
+    assert y.shape == (0, K)
+    y.sum().backward()
+    assert x.grad.shape == (0, K) and gates.grad.shape == (0, k)
+    assert float(w1.grad.abs().sum()) == 0.0 and float(w2.grad.abs().sum()) == 0.0
+
+    layer = cute_kernels.MoE(E, k, K, N, cute_kernels.swiglu_packed_cute, True, False, 0.02).to(torch.bfloat16).to(device)
+    x = torch.randn(2, 0, K, device=device, dtype=torch.bfloat16, requires_grad=True)
+    out, logits = layer(x)
+    assert out.shape == (2, 0, K) and logits.shape == (0, E)
+    out.sum().backward()
+    assert x.grad.shape == (2, 0, K)
+    norm_weight = torch.ones(K, device=device, dtype=torch.bfloat16)
+    out, logits = layer.forward_with_norm(x, norm_weight, 1e-5)
+    assert out.shape == (2, 0, K) and logits.shape == (0, E)
