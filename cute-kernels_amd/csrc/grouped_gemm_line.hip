@@ -280,7 +280,7 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
     }
   }
   static_assert(!BT || kBtWindows % 8 == 0 || kBtWindows == 24, "window swizzle works on groups of 8 windows");
-  const int nk = k_len / BK;
+  const int nk = __builtin_amdgcn_readfirstlane(k_len / BK);  // the same in every lane; says so to the compiler
   // Stage layout: two stages, each A (BM rows) followed by B (BN rows).
   constexpr int kAStage = BM * kRowBytes;
   auto a_stage_at = [&](int st) { return st * kStageBytes; };
@@ -304,7 +304,8 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
   const uint32_t wave_a = __builtin_amdgcn_readfirstlane(lds_base + wave * A_LD * 1024);
   const uint32_t wave_b = __builtin_amdgcn_readfirstlane(lds_base + wave * B_LD * 1024);
   // load g of K step `step`: g < A_LD: a wave-load of A, else of the weight operand, into stage step % 2
-  auto issue_one = [&](int step, int g) {
+  auto issue_one = [&](int step, int g) __attribute__((always_inline)) {
+    step = __builtin_amdgcn_readfirstlane(step);  // uniform; said to the compiler, which wants it in a scalar register
     const uint32_t st = (uint32_t)((step & (NSTAGE - 1)) * kStageBytes);
     // measurement builds: bit 16 = both operands re-read the first two K steps (L2 hits), 512 / 1024 = only A / only B does
     const int64_t kb = (CK_ABLATE & 16) ? (int64_t)(step & 1) * kRowBytes : (int64_t)step * kRowBytes;
@@ -435,14 +436,24 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
     // One 32-wide slice: MI x NI MFMAs, row block by row block, and the fragment reads for the slice after it (ns, nsl).
     // Two fragment sets: the reads go out one after each of the first MI + NI MFMAs, in the order the next slice needs
     // them. One set: fa[i] is reloaded once row block i is done, fb[j] after the MFMA (MI - 1, j).
-    // Slice 0 of a step: the next slice is in the same stage.
-    // Slice 1: the next slice is slice 0 of step kt + 1 in the other stage. Phase 0 / 1: wait for that stage (the only
-    //   loads in flight) and for this wave's own fragment reads, then meet the other waves -- the whole current stage has
-    //   been read by everyone, so in phase 0 the loads of step kt + 2 overwrite it under this slice's MFMAs, one load
-    //   every kLoadGap MFMAs. Phase 1 is step nk - 2 (nothing left to fetch), phase 2 the last step (nothing to wait
-    //   for, nothing to reload).
+    // Slice 0 of a step: the next slice is in the same stage. Phase 0 (and 3, the tile's first slice, whose early loads
+    //   test nk themselves): early loads of step kt + 2, see below; phase 2: nothing to fetch.
+    // Slice 1: the next slice is slice 0 of step kt + 1 in the other stage. Phase 0 / 1: wait for that stage (every
+    //   load older than this step's early ones) and for this wave's own fragment reads, then meet the other waves; in
+    //   phase 0 the late loads of step kt + 2 go out under this slice's MFMAs. Phase 1 is step nk - 2 (nothing left to
+    //   fetch), phase 2 the last step (nothing to wait for, nothing to reload).
     constexpr int kLoadGap = (MI * NI) / kLoadsPerStep;
-    auto slice = [&](int kt, auto sl, auto phase, auto idle, auto first) {
+    // Two barriers per K step. The stage a step reads is dead as soon as every wave holds its fragments of the step's
+    // second slice, i.e. early in the first slice (the reads go out behind its first MI + NI MFMAs): a barrier behind
+    // MFMA kWarAt of the first slice says so, and the first kEarly loads of step kt + 2 follow it under the rest of
+    // that slice; the others go out under the second slice, behind the barrier that publishes step kt + 1. The last
+    // load of a step is then in flight for 0.8 of a K step before it is waited for instead of 0.5 (8 early loads
+    // from MFMA 20 on, the late ones 6 MFMAs apart: 5 % faster launches than all 16 under the second slice; 6, 10, 12
+    // or 16 early loads, other starting points and denser early loads measured the same or slower).
+    constexpr int kEarly = kDouble ? 8 : 0, kWarAt = 20, kEarlyGap = 4, kLateGap = kEarly > 0 ? 6 : kLoadGap;
+    static_assert(kEarly == 0 || (kWarAt >= MI + NI && kWarAt + (kEarly - 1) * kEarlyGap < MI * NI && kEarly <= kLoadsPerStep), "early loads");
+    static_assert((kLoadsPerStep - kEarly - 1) * kLateGap < MI * NI, "late loads");
+    auto slice = [&](int kt, auto sl, auto phase, auto idle, auto first) __attribute__((always_inline)) {
       constexpr bool kIdle = decltype(idle)::value;  // this wave's rows are all pad rows: no fragments, no MFMAs
       constexpr bool kLast = decltype(sl)::value == KS - 1;
       constexpr int kPhase = decltype(phase)::value;
@@ -457,7 +468,8 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
         } else if constexpr (CK_STAMP != 0) {
           asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
           const uint64_t t0 = clock64();
-          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+          if constexpr (kPhase == 0) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kEarly) : "memory");
+          else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
           const uint64_t t1 = clock64();
           asm volatile("s_barrier" ::: "memory");
           const uint64_t t2 = clock64();
@@ -465,7 +477,8 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
           st_bar += t2 - t1;
           st_s0 += t0 - st_mark;  // slice 0 of this step (the slice in front of the wait)
           st_mark = t2;
-        } else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
+        } else if constexpr (kPhase == 0) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(kEarly) : "memory");
+        else asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory");
       }
       constexpr int cur = kDouble ? (decltype(sl)::value & 1) : 0;
       constexpr int nxt = kDouble ? (cur ^ 1) : 0;
@@ -474,7 +487,14 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
         const int i = n / NI, j = n % NI;
         if constexpr (!kIdle) mfma(cur, i, j, first);
         if constexpr (kLast && kPhase == 0 && !(CK_ABLATE & 2)) {
-          if (n % kLoadGap == 0 && n / kLoadGap < kLoadsPerStep) issue_one(kt + 2, n / kLoadGap);
+          if (n % kLateGap == 0 && n / kLateGap < kLoadsPerStep - kEarly) issue_one(kt + 2, kEarly + n / kLateGap);
+        }
+        if constexpr (!kLast && (kPhase == 0 || kPhase == 3) && kEarly > 0 && !(CK_ABLATE & 2)) {
+          // every wave holds its fragments of this stage's second slice: once all have said so the stage is dead and the
+          // first kEarly loads of step kt + 2 overwrite it under the rest of this slice
+          if (n == kWarAt) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+          if (n >= kWarAt && (n - kWarAt) % kEarlyGap == 0 && (n - kWarAt) / kEarlyGap < kEarly && (kPhase == 0 || nk > 2))
+            issue_one(kt + 2, (n - kWarAt) / kEarlyGap);
         }
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (kReload) {
@@ -495,23 +515,33 @@ __global__ __launch_bounds__(64 * 2 * WGM) void grouped_gemm_line_kernel(const G
         st_mark = t3;
       }
     };
-    // The first slice of the tile is peeled (its MFMAs start the accumulators); the loop body is the second slice of step
-    // kt followed by the first slice of step kt + 1 (the first slice of a step does not depend on the phase).
-    auto k_loop = [&](auto idle) {
+    // The first slice of the tile is peeled (its MFMAs start the accumulators). Every branch on the way has one arm
+    // and the loop body none: two variants of a slice meeting behind a two-armed branch make the compiler move the
+    // 256 accumulators around (spills between MFMAs whose results it cannot know to be in flight). The lambdas are
+    // force-inlined: left to the inliner's budget they become calls and the accumulators go to memory.
+    auto k_loop = [&](auto idle) __attribute__((always_inline)) {
       constexpr std::integral_constant<int, 0> s0{}, p0{};
       constexpr std::integral_constant<int, 1> s1{}, p1{};
       constexpr std::integral_constant<int, 2> p2{};
       constexpr std::false_type later{};
-      if constexpr (WGM == 2) slice(0, s0, p0, idle, std::true_type{});
-      else slice(0, s0, p0, idle, later);
+      // A step kt with kt + 2 < nk fetches step kt + 2 (phase 0 of both its slices); the first slice of the last two
+      // steps is phase 2 (nothing to fetch). The tile's very first slice is phase 3: its early loads sit under a test
+      // of nk each, so that one variant serves every tile and the accumulators start in one place.
+      constexpr std::integral_constant<int, 3> p3{};
+      if constexpr (WGM == 2) slice(0, s0, p3, idle, std::true_type{});
+      else slice(0, s0, p3, idle, later);
       int kt = 0;
-      for (; kt + 2 < nk; ++kt) {
-        slice(kt, s1, p0, idle, later);
-        slice(kt + 1, s0, p0, idle, later);
+      if (nk > 2) {
+        slice(0, s1, p0, idle, later);
+        for (kt = 1; kt + 2 < nk; ++kt) {
+          slice(kt, s0, p0, idle, later);
+          slice(kt, s1, p0, idle, later);
+        }
+        slice(kt, s0, p2, idle, later);
       }
       if (kt + 2 == nk) {
         slice(kt, s1, p1, idle, later);
-        slice(kt + 1, s0, p0, idle, later);
+        slice(kt + 1, s0, p2, idle, later);
         ++kt;
       }
       slice(kt, s1, p2, idle, later);
