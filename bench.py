@@ -543,6 +543,8 @@ def main() -> int:
     ap.add_argument("--reverse-load", action="store_true",
                     help="the C3 step with the expert loads reversed (heaviest expert last); not the headline workload")
     ap.add_argument("--no-split", action="store_true", help="never split the last round of GEMM tiles (A/B measurement)")
+    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                    help="ck_debug_set_option(NAME, VALUE) before the run (A/B measurement of kernel variants)")
     ap.add_argument("--summarize-pmc", nargs=2, metavar=("FETCH_DIR", "WRITE_DIR"),
                     help="no GPU work: reduce two rocprofv3 --pmc output directories to profiles/grouped_gemm_c3_hbm_traffic.txt")
     ap.add_argument("--stamps", action="store_true",
@@ -567,6 +569,9 @@ def main() -> int:
         _C.use_library(args.lib)
     if args.no_split:
         scattermoe.options.gemm_split = False
+    for item in args.option:
+        name, _, value = item.partition("=")
+        _C.set_option(name, int(value))
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     if args.only_gemm > 0:
