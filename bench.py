@@ -345,6 +345,12 @@ def secondary_hbm_kernels(dev):
                                                                      rstd.data_ptr(), 1e-6, 1.0, Bn, Hn, dxn.data_ptr(), drn.data_ptr(),
                                                                      partial.data_ptr(), dwn.data_ptr(), bf, stream))),
         5 * Bn * Hn * 2 + 4 * Bn)
+    # multiplier 1: both gradients are the same values and one buffer takes them (the Python wrapper's call)
+    rec("fused_residual_add_rmsnorm_bwd_one_buffer_C5",
+        timed(lambda: _C.check(lib.ck_fused_residual_add_rmsnorm_bwd(an.data_ptr(), wn.data_ptr(), gn.data_ptr(), ga.data_ptr(),
+                                                                     rstd.data_ptr(), 1e-6, 1.0, Bn, Hn, dxn.data_ptr(), dxn.data_ptr(),
+                                                                     partial.data_ptr(), dwn.data_ptr(), bf, stream))),
+        4 * Bn * Hn * 2 + 4 * Bn)
     del yn, gn, dxn, rn, an, ga, drn, partial
     # RMSNorm fused ahead of the router (one pass: normalised rows + router logits, optionally the e4m3 rows) against the
     # separate kernels (rmsnorm, the router's linear layer on the BLAS library, the row quantiser); algorithmic bytes:

@@ -515,11 +515,13 @@ inline int compute_units() {
 // per CU: H = 2,048: 45 / 71 / 77 / 73; H = 4,096: 60 / 74 / 67 / 65; H = 8,192: 75 / 73 / 66 / 72; counts that are not a
 // multiple of the CU count lose 5-10 points to the ragged last wave of blocks. With the residual fusion (3 streams in, 2
 // out) the curve is flat (68-70 % at 2-4 per CU) and 3 / 4 per CU are kept.
-inline int64_t workers_for(int64_t B, int tpr, int H, bool fused) {
+// `added_only`: the residual stream's gradient comes in but one buffer takes both outputs (3 streams in, 1 out):
+// 65,536 x 4,096 419 / 369 / 380 us at 2 / 3 / 4 per CU, 16,384 x 8,192 195 / 235 / 204.
+inline int64_t workers_for(int64_t B, int tpr, int H, bool fused, bool added_only = false) {
   const int rows_per_block = kBlock / tpr;
   int64_t w = B < kMaxWorkers ? B : kMaxWorkers;
   if (tpr == kBlock) {
-    const int per_cu = fused ? (H < 3072 ? 3 : 4) : (H < 3072 ? 3 : 2);
+    const int per_cu = fused ? (H < 3072 ? 3 : 4) : added_only ? (H < 6144 ? 3 : 2) : (H < 3072 ? 3 : 2);
     const int64_t cap = (int64_t)per_cu * compute_units();
     if (w > cap) w = cap;
     if (w > kMaxWorkers / 2) w = kMaxWorkers / 2;
@@ -628,7 +630,7 @@ static int rmsnorm_bwd_impl(const char* name, const void* x, const void* weight,
                          (d_added == nullptr || aligned16(d_added)) && (d_residual == nullptr || aligned16(d_residual));
     const Plan plan = make_plan<scalar_t>(H, aligned);
     const int rows_per_block = kBlock / plan.tpr;
-    const int64_t workers = workers_for(B, plan.tpr, (int)H, d_added != nullptr || d_residual != nullptr);
+    const int64_t workers = workers_for(B, plan.tpr, (int)H, d_residual != nullptr, d_added != nullptr);
     const int64_t blocks = workers / rows_per_block;
     const BwdFuse<scalar_t> fuse = {static_cast<const scalar_t*>(d_added), static_cast<scalar_t*>(d_residual), multiplier};
     CK_RMS_DISPATCH(CK_RMS_BWD, 0);
@@ -654,6 +656,8 @@ extern "C" int ck_fused_residual_add_rmsnorm_bwd(const void* added, const void* 
                                                  float* d_weight_partial, float* d_weight, int32_t dtype, void* stream) {
   const char* name = "ck_fused_residual_add_rmsnorm_bwd";
   CK_REQUIRE(B == 0 || d_residual != nullptr, "%s: d_residual is required", name);
-  return rmsnorm_bwd_impl(name, added, weight, d_out, d_added, rstd, eps, multiplier, B, H, d_x, d_residual,
-                          d_weight_partial, d_weight, dtype, stream);
+  CK_REQUIRE(d_residual != d_x || multiplier == 1.0f, "%s: d_x and d_residual may be one buffer only when multiplier is 1", name);
+  // multiplier == 1: both gradients are the same values; a caller that passes one buffer for both gets one store
+  return rmsnorm_bwd_impl(name, added, weight, d_out, d_added, rstd, eps, multiplier, B, H, d_x,
+                          d_residual == d_x ? nullptr : d_residual, d_weight_partial, d_weight, dtype, stream);
 }

@@ -215,6 +215,7 @@ def fused_residual_add_rmsnorm_backward(
     ctx = _Ctx()
     ctx.saved_tensors = (added, weight, None if memory_efficient else rstd)
     ctx.eps, ctx.multiplier = eps, multiplier
+    ctx.separate_outputs = True  # an operator's outputs may not alias each other
     x_grad, residual_grad, weight_grad, *_ = _frn._FusedResidualAddRMSNorm_Cute.backward(ctx, output_grad, added_grad)
     return x_grad, residual_grad, _or_empty(weight_grad, added)
 

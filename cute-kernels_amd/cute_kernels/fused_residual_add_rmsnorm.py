@@ -67,7 +67,10 @@ class _FusedResidualAddRMSNorm_Cute(torch.autograd.Function):
         B, H = get_num_elements_and_hidden_size(added_x_residual)
 
         x_grad = torch.empty_like(added_x_residual)
-        residual_grad = torch.empty_like(added_x_residual)
+        # multiplier 1: both gradients are the same values, so one tensor serves both (written once); the operator of a
+        # traced graph keeps two, its outputs may not alias
+        one_buffer = ctx.multiplier == 1.0 and not getattr(ctx, "separate_outputs", False)
+        residual_grad = x_grad if one_buffer else torch.empty_like(added_x_residual)
         lib = _C.lib()
         weight_grad = partial = None
         if weight is not None:

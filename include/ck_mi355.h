@@ -379,7 +379,9 @@ int ck_expert_bias_grad(const void* d_y, int32_t N, const ck_segments* seg, void
  * forward:  added = (x * multiplier) + residual, each step rounded to the tensor dtype (multiplier == 1: no scaling);
  *           out = rmsnorm(added). x, residual, out, added [B, H]; rstd as above.
  * backward: g = d rmsnorm(added)/d added applied to d_out, plus d_added (the gradient arriving through the residual
- *           stream; NULL = none); d_residual = g, d_x = g * multiplier. `added` is the forward's output.
+ *           stream; NULL = none); d_residual = g, d_x = g * multiplier. `added` is the forward's output. With
+ *           multiplier == 1 the two gradients are the same values: d_residual may then be the same buffer as d_x, and
+ *           the rows are written once (any other multiplier with one buffer is an error).
  * ------------------------------------------------------------------------------------------------------------- */
 int ck_fused_residual_add_rmsnorm_fwd(const void* x, const void* residual, const void* weight, float eps,
                                       float multiplier, int64_t B, int32_t H, void* out, void* added, float* rstd,

@@ -228,6 +228,47 @@ def test_fused_residual_add_rmsnorm_without_residual_gradient(device):
         torch.testing.assert_close(ours.grad.cpu(), ref.grad, rtol=1e-4, atol=1e-3)
 
 
+def test_fused_residual_add_rmsnorm_backward_into_one_buffer(device):
+    # multiplier 1: d_x and d_residual are the same values, and the C ABI takes one buffer for both (one store per row):
+    # bit-identical to the two-buffer call; any other multiplier with one buffer is refused. Through autograd the two
+    # leaves still end up with gradients of their own (a second backward accumulates into each separately).
+    from cute_kernels import _C
+
+    lib, stream = _C.lib(), torch.cuda.current_stream().cuda_stream
+    g = torch.Generator().manual_seed(5)
+    for B, H in ((300, 4096), (64, 512), (17, 8192)):
+        added, d_out, d_added = (torch.randn(B, H, generator=g).to(torch.bfloat16).to(device) for _ in range(3))
+        w = torch.randn(H, generator=g).to(torch.bfloat16).to(device)
+        rstd = added.float().square().mean(-1).add(1e-6).rsqrt()
+        partial = torch.empty(max(lib.ck_rmsnorm_bwd_partial_rows(B), 1), H, device=device, dtype=torch.float32)
+        outs = []
+        for one_buffer in (False, True):
+            d_x, d_w = torch.empty_like(added), torch.empty(H, device=device, dtype=torch.float32)
+            d_r = d_x if one_buffer else torch.empty_like(added)
+            _C.check(lib.ck_fused_residual_add_rmsnorm_bwd(
+                added.data_ptr(), w.data_ptr(), d_out.data_ptr(), d_added.data_ptr(), rstd.data_ptr(), 1e-6, 1.0, B, H,
+                d_x.data_ptr(), d_r.data_ptr(), partial.data_ptr(), d_w.data_ptr(), _C.CK_BF16, stream))
+            outs.append((d_x, d_r, d_w))
+        assert torch.equal(outs[0][0], outs[0][1]) and torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][2], outs[1][2])
+        d_x = torch.empty_like(added)
+        with pytest.raises(RuntimeError, match="one buffer"):
+            _C.check(lib.ck_fused_residual_add_rmsnorm_bwd(
+                added.data_ptr(), w.data_ptr(), d_out.data_ptr(), d_added.data_ptr(), rstd.data_ptr(), 1e-6, 0.5, B, H,
+                d_x.data_ptr(), d_x.data_ptr(), partial.data_ptr(), d_w.data_ptr(), _C.CK_BF16, stream))
+
+    x, r = (torch.randn(64, 512, generator=g).to(device).requires_grad_() for _ in range(2))
+    w = torch.randn(512, generator=g).to(device).requires_grad_()
+    for _ in range(2):  # the second pass accumulates
+        z, added = cute_kernels.fused_residual_add_rmsnorm_cute(x, r, w, 1e-6)
+        (z * 2 + added * 3).sum().backward()
+    assert x.grad.data_ptr() != r.grad.data_ptr() and torch.equal(x.grad, r.grad)
+    xc, rc, wc = (t.detach().cpu().clone().requires_grad_() for t in (x, r, w))
+    z_ref, added_ref = mo.fused_residual_add_rmsnorm_torch(xc, rc, wc, 1e-6, None)
+    (z_ref * 2 + added_ref * 3).sum().backward()
+    torch.testing.assert_close(x.grad.cpu(), 2 * xc.grad, rtol=1e-4, atol=4e-4)
+    torch.testing.assert_close(w.grad.cpu(), 2 * wc.grad, rtol=1e-4, atol=4e-3)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("logits_multiplier", [None, 0.7])
 def test_softmax_reference_grid(device, dtype, logits_multiplier):
